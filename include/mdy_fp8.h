@@ -1,0 +1,128 @@
+/* mdy_fp8.h - C ABI of libmdyfp8.so: DeepSeek-V3-style block-wise FP8 linear path
+ * for AMD MI355X (gfx950).
+ *
+ * Every entry point
+ *   - takes raw device pointers, sizes/strides in ELEMENTS and a HIP stream
+ *     (passed as void*; NULL = the null stream),
+ *   - enqueues its kernels on that stream and returns without synchronising,
+ *   - allocates nothing, keeps no mutable global state and is re-entrant,
+ *   - returns 0 on success, a negative MDY_E_* code for a rejected argument
+ *     (nothing was launched) or a positive hipError_t if the launch failed.
+ *     mdy_fp8_last_error() returns a thread-local message for the last non-zero
+ *     return on the calling thread.
+ *
+ * Reference interfaces are cited as file:line under the reference tree
+ * (triton_kernels/deepseekv3/offical_kernel.py = "offical_kernel.py",
+ *  triton_kernels/dpsk_fp8linear/fp8.py        = "fp8.py").
+ */
+#ifndef MDY_FP8_H_
+#define MDY_FP8_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MDY_FP8_ABI_VERSION 1
+
+/* error codes (negative = argument rejected before any launch) */
+#define MDY_OK 0
+#define MDY_E_NULL (-1)      /* a required pointer is NULL */
+#define MDY_E_SHAPE (-2)     /* a size/stride violates the documented precondition */
+#define MDY_E_ALIGN (-3)     /* a pointer or stride is not aligned as documented */
+#define MDY_E_DTYPE (-4)     /* unknown dtype / mode selector */
+#define MDY_E_DEVICE (-5)    /* the current device is not a gfx950 GPU */
+
+/* output dtype selectors */
+#define MDY_DT_BF16 0
+#define MDY_DT_F32 1
+
+/* quantizer dialects */
+#define MDY_QUANT_OFFICIAL 0 /* s = amax / 448                      offical_kernel.py:14 */
+#define MDY_QUANT_DEEPLINEAR 1 /* s = (min(amax,1e4) + 1e-8) / 448, saturating cast  fp8.py:109-111 */
+
+int mdy_fp8_abi_version(void);
+const char* mdy_fp8_last_error(void);
+
+/* Per-token 1x128 activation quantizer.
+ * Replaces act_quant (offical_kernel.py:21-28, kernel :9-18) with
+ * mode = MDY_QUANT_OFFICIAL, PM = M, PK = K, and quant_input(only_forward=True)
+ * (fp8.py:122-161, kernel :87-120) with mode = MDY_QUANT_DEEPLINEAR and the
+ * padded sizes that launcher computes.
+ *
+ *   x  bf16 [M, K], element (m, k) at x[m * x_row_stride + k]   (unit column stride)
+ *   y  e4m3fn [PM, PK] row-major; PM >= M, PK >= K, PK % 128 == 0; padding reads as 0
+ *   s  fp32, scale of row m, K-block kb at s[m * s_row_stride + kb * s_col_stride]
+ *      for m < PM, kb < PK / 128
+ * Vector path needs x 16-byte aligned with x_row_stride % 8 == 0 and K % 8 == 0;
+ * anything else takes an element-wise path inside the same kernel.
+ * y must be 8-byte aligned.  M == 0 is a no-op.
+ */
+int mdy_act_quant(const void* x, void* y, float* s, int64_t M, int64_t K, int64_t x_row_stride,
+                  int64_t PM, int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode,
+                  void* stream);
+
+/* 128x128 block weight quantizer.
+ * Replaces quant_weight(only_forward=True/False) (fp8.py:206-247, kernel :171-203)
+ * with mode = MDY_QUANT_DEEPLINEAR, and weight_quant_block
+ * (triton_kernels/deepseekv3/fp8_kernel.py:124-138, kernel :88-122) with
+ * mode = MDY_QUANT_OFFICIAL.
+ *
+ *   w   bf16 [N, K], element (n, k) at w[n * w_row_stride + k * w_col_stride]
+ *   y   e4m3fn [PN, PK] row-major, PN % 128 == 0, PK % 128 == 0, padding reads as 0
+ *   s   fp32 [PN/128, PK/128] row-major
+ *   y_t e4m3fn [PK, PN] row-major (transposed copy) or NULL
+ *   s_t fp32 [PK/128, PN/128] row-major or NULL (must be given iff y_t is)
+ */
+int mdy_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t, int64_t N, int64_t K,
+                     int64_t w_row_stride, int64_t w_col_stride, int64_t PN, int64_t PK, int mode,
+                     void* stream);
+
+/* 128x128 block weight dequantizer: y[n,k] = fp32(x[n,k]) * s[n/128, k/128].
+ * Replaces weight_dequant (offical_kernel.py:46-53, kernel :31-43).
+ *   x e4m3fn [N, K] row-major; s fp32 [ceil(N/128), ceil(K/128)] row-major;
+ *   y [N, K] row-major of out_dtype (MDY_DT_BF16 or MDY_DT_F32).
+ */
+int mdy_weight_dequant(const void* x, const float* s, void* y, int64_t N, int64_t K, int out_dtype,
+                       void* stream);
+
+/* Block-scaled FP8 GEMM, NT layout:
+ *   c[m,n] = sum_kb (sum_{k in kb} a[m,k] * b[n,k]) * a_s[m,kb] * b_s[n/128,kb]  (+ bias[n])
+ * Replaces fp8_gemm (offical_kernel.py:100-109, kernel :61-97) with
+ * as_row_stride = ceil(K/128), as_col_stride = 1, and fp8_matmul (fp8.py:307-311,
+ * i.e. deep_gemm.gemm_fp8_fp8_bf16_nt) with the column-major scale strides
+ * (1, PM) that quant_input returns; bias folds add_bias (fp8.py:297-305) into
+ * the epilogue.
+ *
+ *   a    e4m3fn [M, K] row-major         a_s fp32, (m,kb) at a_s[m*as_row_stride + kb*as_col_stride]
+ *   b    e4m3fn [N, K] row-major         b_s fp32 [ceil(N/128), ceil(K/128)] row-major
+ *   c    [M, N] row-major of out_dtype   bias bf16 [N] or NULL (added in fp32 before the cast)
+ * Any M, N, K >= 1 is accepted (M == 0 or N == 0 is a no-op); K % 128 == 0 with
+ * 16-byte aligned a and b takes the MFMA kernels, anything else a scalar kernel.
+ */
+int mdy_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
+                    const void* b, const float* b_s, void* c, const void* bias, int64_t M, int64_t N,
+                    int64_t K, int out_dtype, void* stream);
+
+/* In-place x[m, :] = bf16(fp32(x[m, :]) + fp32(b)) on bf16 x [M, N] row-major, bf16 b [N].
+ * Replaces add_bias (fp8.py:297-305, kernel :283-295). */
+int mdy_add_bias(void* x, const void* b, int64_t M, int64_t N, void* stream);
+
+/* Diagnostic: element-wise fp32 -> e4m3fn with the same device conversion the
+ * quantizers use (saturate != 0 clamps finite values to +-448 first).  No
+ * counterpart in the reference (the cast is implicit in tl.store, fp8.py:112);
+ * exists so that the cast can be checked against the format definition. */
+int mdy_cast_f32_to_e4m3(const float* x, void* y, int64_t n, int saturate, void* stream);
+
+/* Diagnostic: returns in out[0..3] the number of (amax, x) bf16 pairs, of fp32
+ * quotient mismatches and of e4m3fn byte mismatches between the quantizers'
+ * reciprocal+2-FMA quotient and IEEE division, over every finite bf16 amax in
+ * [amax_lo, amax_hi) (bit patterns) and every bf16 x with |x| <= amax, for the
+ * given dialect.  out is device memory, 4 x uint64, zeroed by the call. */
+int mdy_quotient_selfcheck(uint64_t* out, int amax_lo, int amax_hi, int mode, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MDY_FP8_H_ */

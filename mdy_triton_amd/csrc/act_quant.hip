@@ -1,0 +1,209 @@
+// Per-token 1x128 activation quantizer: bf16 -> e4m3fn bytes + one fp32 scale per group.
+//
+// Restates the arithmetic of act_quant_kernel
+// (/root/reference/triton_kernels/deepseekv3/offical_kernel.py:9-18) and of
+// _quant_input_kernel's forward half
+// (/root/reference/triton_kernels/dpsk_fp8linear/fp8.py:104-113) for wave64:
+//
+//   * 16 lanes own one 128-element group: one 16-byte load (8 bf16) per lane, so a
+//     wave covers 512 contiguous elements of a row per load instruction;
+//   * absmax by v_max3_f32 on the unpacked values, then a 4-step DPP butterfly
+//     inside the 16-lane row (no LDS, no barrier);
+//   * scale = amax / 448 and r = 1 / scale with IEEE division once per group; each
+//     element is x*r corrected by two FMAs (bit-identical to x / scale, proven
+//     exhaustively over bf16 x bf16); groups whose amax is tiny, above 1e4
+//     (DeepLinear dialect, needs the saturating cast) or non-finite divide plainly;
+//   * v_cvt_pk_fp8_f32 x4 -> one 8-byte store per lane; lane 0 of the row stores
+//     the scale at a caller-given (row, column) stride so that both the row-major
+//     [M, K/128] layout and the column-major padded [K/128][PM] layout come out
+//     of the same kernel.
+//
+// HBM traffic per element: 2 B in, 1 B out, 4/128 B scale = 3.03125 B.
+#include "common.h"
+
+namespace mdy {
+
+constexpr int kAqRowsPerWave = 4;
+constexpr int kAqWaves = 4;
+constexpr int kAqRowsPerBlock = kAqRowsPerWave * kAqWaves;  // 16 rows x 512 columns per block
+
+__device__ __forceinline__ float row16_max(float v) {
+    // butterfly over the 16 lanes of a DPP row: xor 1, xor 2 (quad_perm), then
+    // row_half_mirror (lane -> 7-lane inside each 8) and row_mirror (lane -> 15-lane)
+    int i = __float_as_int(v);
+    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0xB1, 0xF, 0xF, true))));   // quad_perm [1,0,3,2]
+    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0x4E, 0xF, 0xF, true))));   // quad_perm [2,3,0,1]
+    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0x141, 0xF, 0xF, true))));  // row_half_mirror
+    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0x140, 0xF, 0xF, true))));  // row_mirror
+    return __int_as_float(i);
+}
+
+template <int MODE>
+__device__ __forceinline__ uint2 quantize8(const float (&f)[8], float amax, float& scale_out) {
+    float s = group_scale<MODE>(amax);
+    scale_out = s;
+    float q[8];
+    bool fast = MODE == 0 ? fast_quotient_ok<0>(amax) : (amax <= 1e4f);
+    if (fast) {
+        float r = 1.0f / s;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i] = fast_quotient(f[i], s, r);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float v = f[i] / s;
+            if (MODE != 0) {
+                float c = __builtin_amdgcn_fmed3f(v, -kFp8Max, kFp8Max);
+                v = (v != v) ? v : c;
+            }
+            q[i] = v;
+        }
+    }
+    uint2 out;
+    out.x = pack4_e4m3(q[0], q[1], q[2], q[3]);
+    out.y = pack4_e4m3(q[4], q[5], q[6], q[7]);
+    return out;
+}
+
+// grid.x = ceil(PK / 512), grid.y = ceil(PM / 16), block = 256
+template <int MODE, bool VEC>
+__global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ y,
+                                                         float* __restrict__ s, int M, int K, int64_t x_row_stride,
+                                                         int PM, int PK, int64_t s_row_stride, int64_t s_col_stride) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int col = blockIdx.x * 512 + lane * 8;  // first of this lane's 8 columns
+    const int row0 = blockIdx.y * kAqRowsPerBlock + wave * kAqRowsPerWave;
+    const bool col_in_out = col < PK;  // PK % 128 == 0, so whole 16-lane rows agree
+
+    uint4 raw[kAqRowsPerWave];
+#pragma unroll
+    for (int r = 0; r < kAqRowsPerWave; ++r) {
+        const int row = row0 + r;
+        raw[r] = make_uint4(0u, 0u, 0u, 0u);
+        if (row < M && col < K) {
+            const uint16_t* p = x + (int64_t)row * x_row_stride + col;
+            if (VEC) {
+                raw[r] = *reinterpret_cast<const uint4*>(p);  // K % 8 == 0: all 8 columns in range
+            } else {
+                uint32_t w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    if (col + i < K) w[i >> 1] |= (uint32_t)p[i] << ((i & 1) * 16);
+                raw[r] = make_uint4(w[0], w[1], w[2], w[3]);
+            }
+        }
+    }
+
+#pragma unroll
+    for (int r = 0; r < kAqRowsPerWave; ++r) {
+        const int row = row0 + r;
+        float f[8];
+        f[0] = bf16_lo(raw[r].x); f[1] = bf16_hi(raw[r].x);
+        f[2] = bf16_lo(raw[r].y); f[3] = bf16_hi(raw[r].y);
+        f[4] = bf16_lo(raw[r].z); f[5] = bf16_hi(raw[r].z);
+        f[6] = bf16_lo(raw[r].w); f[7] = bf16_hi(raw[r].w);
+        float m = 0.0f;
+        m = fmaxf(fmaxf(fabsf(f[0]), fabsf(f[1])), m);
+        m = fmaxf(fmaxf(fabsf(f[2]), fabsf(f[3])), m);
+        m = fmaxf(fmaxf(fabsf(f[4]), fabsf(f[5])), m);
+        m = fmaxf(fmaxf(fabsf(f[6]), fabsf(f[7])), m);
+        const float amax = row16_max(m);
+        float scale;
+        const uint2 packed = quantize8<MODE>(f, amax, scale);
+        if (row < PM && col_in_out) {
+            *reinterpret_cast<uint2*>(y + (int64_t)row * PK + col) = packed;
+            if ((lane & 15) == 0) s[(int64_t)row * s_row_stride + (int64_t)(col >> 7) * s_col_stride] = scale;
+        }
+    }
+}
+
+int launch_act_quant(const void* x, void* y, float* s, int64_t M, int64_t K, int64_t x_row_stride, int64_t PM,
+                     int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode, hipStream_t stream) {
+    if (PM == 0 || PK == 0) return 0;
+    dim3 grid((unsigned)((PK + 511) / 512), (unsigned)((PM + kAqRowsPerBlock - 1) / kAqRowsPerBlock));
+    dim3 block(256);
+    const bool vec = (K % 8 == 0) && (x_row_stride % 8 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+    const uint16_t* xp = static_cast<const uint16_t*>(x);
+    uint8_t* yp = static_cast<uint8_t*>(y);
+#define MDY_AQ(MODE, VEC)                                                                                       \
+    hipLaunchKernelGGL((act_quant_kernel<MODE, VEC>), grid, block, 0, stream, xp, yp, s, (int)M, (int)K,        \
+                       x_row_stride, (int)PM, (int)PK, s_row_stride, s_col_stride)
+    if (mode == 0) {
+        if (vec) MDY_AQ(0, true); else MDY_AQ(0, false);
+    } else {
+        if (vec) MDY_AQ(1, true); else MDY_AQ(1, false);
+    }
+#undef MDY_AQ
+    return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// diagnostics
+// ---------------------------------------------------------------------------
+__global__ void cast_f32_to_e4m3_kernel(const float* __restrict__ x, uint8_t* __restrict__ y, int64_t n, int saturate) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float v = x[i];
+    if (saturate) {
+        float c = __builtin_amdgcn_fmed3f(v, -kFp8Max, kFp8Max);
+        v = (v != v) ? v : c;
+    }
+    y[i] = (uint8_t)(pack4_e4m3(v, 0.0f, 0.0f, 0.0f) & 0xFFu);
+}
+
+int launch_cast_f32_to_e4m3(const float* x, void* y, int64_t n, int saturate, hipStream_t stream) {
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(cast_f32_to_e4m3_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x,
+                       static_cast<uint8_t*>(y), n, saturate);
+    return (int)hipGetLastError();
+}
+
+// One block per amax bit pattern; threads stride over x patterns 0..amax (both signs).
+// Groups that the quantizers would divide plainly are counted in out[3] and skipped.
+template <int MODE>
+__global__ __launch_bounds__(256) void quotient_selfcheck_kernel(unsigned long long* out, int amax_lo) {
+    const uint32_t ai = (uint32_t)amax_lo + blockIdx.x;
+    const float amax = bf16_one((uint16_t)ai);
+    const float s = group_scale<MODE>(amax);
+    const bool fast = MODE == 0 ? fast_quotient_ok<0>(amax) : (amax <= 1e4f);
+    const float r = 1.0f / s;
+    unsigned long long pairs = 0, f32_bad = 0, fp8_bad = 0, plain = 0;
+    for (uint32_t t = threadIdx.x; t < 2 * (ai + 1); t += blockDim.x) {
+        const uint32_t xi = (t >> 1) | ((t & 1) << 15);
+        const float x = bf16_one((uint16_t)xi);
+        ++pairs;
+        if (!fast) {
+            ++plain;
+            continue;
+        }
+        const float ref = x / s;
+        const float q = fast_quotient(x, s, r);
+        const uint32_t bref = pack4_e4m3(ref, 0.f, 0.f, 0.f) & 0xFF;
+        const uint32_t bq = pack4_e4m3(q, 0.f, 0.f, 0.f) & 0xFF;
+        if (__float_as_uint(ref) != __float_as_uint(q) && !(ref != ref && q != q)) ++f32_bad;
+        if (bref != bq) ++fp8_bad;
+    }
+    atomicAdd(&out[0], pairs);
+    atomicAdd(&out[1], f32_bad);
+    atomicAdd(&out[2], fp8_bad);
+    atomicAdd(&out[3], plain);
+}
+
+__global__ void zero4_kernel(unsigned long long* out) {
+    if (threadIdx.x < 4) out[threadIdx.x] = 0ull;
+}
+
+int launch_quotient_selfcheck(uint64_t* out, int amax_lo, int amax_hi, int mode, hipStream_t stream) {
+    unsigned long long* o = reinterpret_cast<unsigned long long*>(out);
+    hipLaunchKernelGGL(zero4_kernel, dim3(1), dim3(64), 0, stream, o);
+    if (amax_hi <= amax_lo) return (int)hipGetLastError();
+    dim3 grid((unsigned)(amax_hi - amax_lo)), block(256);
+    if (mode == 0)
+        hipLaunchKernelGGL(quotient_selfcheck_kernel<0>, grid, block, 0, stream, o, amax_lo);
+    else
+        hipLaunchKernelGGL(quotient_selfcheck_kernel<1>, grid, block, 0, stream, o, amax_lo);
+    return (int)hipGetLastError();
+}
+
+}  // namespace mdy

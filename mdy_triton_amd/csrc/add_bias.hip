@@ -1,0 +1,57 @@
+// In-place row-broadcast bias add on a bf16 matrix:
+//   x[m, n] = bf16( fp32(x[m, n]) + fp32(b[n]) )
+// Restates _add_bias_kernel (/root/reference/triton_kernels/dpsk_fp8linear/fp8.py:283-295).
+// Streaming kernel: 8 bf16 (16 bytes) per lane, bias slice re-read from L2.
+// The GEMM entry point folds the same add into its epilogue; this kernel is for
+// callers that use add_bias on its own.
+#include "common.h"
+
+namespace mdy {
+
+template <bool VEC>
+__global__ __launch_bounds__(256) void add_bias_kernel(uint16_t* __restrict__ x, const uint16_t* __restrict__ b, int M,
+                                                        int N) {
+    const int col = (blockIdx.x * 256 + threadIdx.x) * 8;
+    if (col >= N) return;
+    float bias[8];
+    if (VEC) {
+        const uint4 v = *reinterpret_cast<const uint4*>(b + col);
+        bias[0] = bf16_lo(v.x); bias[1] = bf16_hi(v.x); bias[2] = bf16_lo(v.y); bias[3] = bf16_hi(v.y);
+        bias[4] = bf16_lo(v.z); bias[5] = bf16_hi(v.z); bias[6] = bf16_lo(v.w); bias[7] = bf16_hi(v.w);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) bias[i] = (col + i < N) ? bf16_one(b[col + i]) : 0.0f;
+    }
+    for (int row = blockIdx.y; row < M; row += gridDim.y) {
+        uint16_t* p = x + (int64_t)row * N + col;
+        if (VEC) {
+            uint4 v = *reinterpret_cast<const uint4*>(p);
+            v.x = pack2_bf16(bf16_lo(v.x) + bias[0], bf16_hi(v.x) + bias[1]);
+            v.y = pack2_bf16(bf16_lo(v.y) + bias[2], bf16_hi(v.y) + bias[3]);
+            v.z = pack2_bf16(bf16_lo(v.z) + bias[4], bf16_hi(v.z) + bias[5]);
+            v.w = pack2_bf16(bf16_lo(v.w) + bias[6], bf16_hi(v.w) + bias[7]);
+            *reinterpret_cast<uint4*>(p) = v;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (col + i < N) p[i] = (uint16_t)(pack2_bf16(bf16_one(p[i]) + bias[i], 0.0f) & 0xFFFFu);
+        }
+    }
+}
+
+int launch_add_bias(void* x, const void* b, int64_t M, int64_t N, hipStream_t stream) {
+    if (M == 0 || N == 0) return 0;
+    const unsigned gy = (unsigned)(M < 4096 ? M : 4096);
+    dim3 grid((unsigned)((N + 2047) / 2048), gy);
+    const bool vec = (N % 8 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0) &&
+                     ((reinterpret_cast<uintptr_t>(b) & 15) == 0);
+    if (vec)
+        hipLaunchKernelGGL(add_bias_kernel<true>, grid, dim3(256), 0, stream, static_cast<uint16_t*>(x),
+                           static_cast<const uint16_t*>(b), (int)M, (int)N);
+    else
+        hipLaunchKernelGGL(add_bias_kernel<false>, grid, dim3(256), 0, stream, static_cast<uint16_t*>(x),
+                           static_cast<const uint16_t*>(b), (int)M, (int)N);
+    return (int)hipGetLastError();
+}
+
+}  // namespace mdy

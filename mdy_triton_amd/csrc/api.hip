@@ -1,0 +1,145 @@
+// extern "C" entry points of libmdyfp8.so: argument validation + dispatch.
+// Declarations and the reference interface each one replaces: include/mdy_fp8.h.
+#include "../../include/mdy_fp8.h"
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "common.h"
+
+namespace {
+
+thread_local char g_err[256] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int launched(int hip_err, const char* what) {
+    if (hip_err == 0) return 0;
+    return fail(hip_err, "%s: launch failed: %s", what, hipGetErrorString(static_cast<hipError_t>(hip_err)));
+}
+
+bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+constexpr int64_t kMaxDim = (int64_t)1 << 30;  // kernels index rows/columns with 32-bit ints
+
+// The kernels are built for gfx950 only; refuse to launch elsewhere instead of
+// letting the runtime fail with a missing code object.
+int check_device() {
+    static thread_local int cached_dev = -1;
+    static thread_local int cached_ok = 0;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return fail(MDY_E_DEVICE, "no HIP device is current");
+    if (dev != cached_dev) {
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return fail(MDY_E_DEVICE, "cannot query device %d", dev);
+        cached_ok = (__builtin_strncmp(prop.gcnArchName, "gfx950", 6) == 0);
+        cached_dev = dev;
+        if (!cached_ok) return fail(MDY_E_DEVICE, "device %d is %s, this library is built for gfx950", dev, prop.gcnArchName);
+    }
+    if (!cached_ok) return fail(MDY_E_DEVICE, "device %d is not gfx950", dev);
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mdy_fp8_abi_version(void) { return MDY_FP8_ABI_VERSION; }
+
+const char* mdy_fp8_last_error(void) { return g_err; }
+
+int mdy_act_quant(const void* x, void* y, float* s, int64_t M, int64_t K, int64_t x_row_stride, int64_t PM,
+                  int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode, void* stream) {
+    if (mode != MDY_QUANT_OFFICIAL && mode != MDY_QUANT_DEEPLINEAR) return fail(MDY_E_DTYPE, "act_quant: unknown mode %d", mode);
+    if (M < 0 || K < 0 || PM < M || PK < K || PM > kMaxDim || PK > kMaxDim)
+        return fail(MDY_E_SHAPE, "act_quant: need 0 <= M <= PM, 0 <= K <= PK (M=%lld K=%lld PM=%lld PK=%lld)",
+                    (long long)M, (long long)K, (long long)PM, (long long)PK);
+    if (PK % 128 != 0) return fail(MDY_E_SHAPE, "act_quant: PK=%lld is not a multiple of 128", (long long)PK);
+    if (PM == 0 || PK == 0) return 0;
+    if (!y || !s || (!x && M > 0 && K > 0)) return fail(MDY_E_NULL, "act_quant: null pointer");
+    if (M > 0 && x_row_stride < K) return fail(MDY_E_SHAPE, "act_quant: x_row_stride=%lld < K=%lld", (long long)x_row_stride, (long long)K);
+    if (!aligned(y, 8)) return fail(MDY_E_ALIGN, "act_quant: y must be 8-byte aligned");
+    if (!aligned(x, 2) || !aligned(s, 4)) return fail(MDY_E_ALIGN, "act_quant: x/s misaligned for their element type");
+    if (int e = check_device()) return e;
+    return launched(mdy::launch_act_quant(x, y, s, M, K, x_row_stride, PM, PK, s_row_stride, s_col_stride, mode,
+                                          static_cast<hipStream_t>(stream)),
+                    "act_quant");
+}
+
+int mdy_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t, int64_t N, int64_t K,
+                     int64_t w_row_stride, int64_t w_col_stride, int64_t PN, int64_t PK, int mode, void* stream) {
+    if (mode != MDY_QUANT_OFFICIAL && mode != MDY_QUANT_DEEPLINEAR) return fail(MDY_E_DTYPE, "weight_quant: unknown mode %d", mode);
+    if (N < 0 || K < 0 || PN < N || PK < K || PN > kMaxDim || PK > kMaxDim)
+        return fail(MDY_E_SHAPE, "weight_quant: need 0 <= N <= PN, 0 <= K <= PK");
+    if (PN % 128 != 0 || PK % 128 != 0) return fail(MDY_E_SHAPE, "weight_quant: PN=%lld, PK=%lld must be multiples of 128", (long long)PN, (long long)PK);
+    if (PN / 128 > 65535) return fail(MDY_E_SHAPE, "weight_quant: PN too large");
+    if ((y_t == nullptr) != (s_t == nullptr)) return fail(MDY_E_NULL, "weight_quant: y_t and s_t must be given together");
+    if (PN == 0 || PK == 0) return 0;
+    if (!y || !s || (!w && N > 0 && K > 0)) return fail(MDY_E_NULL, "weight_quant: null pointer");
+    if (!aligned(y, 8) || (y_t && !aligned(y_t, 8))) return fail(MDY_E_ALIGN, "weight_quant: y / y_t must be 8-byte aligned");
+    if (int e = check_device()) return e;
+    return launched(mdy::launch_weight_quant(w, y, s, y_t, s_t, N, K, w_row_stride, w_col_stride, PN, PK, mode,
+                                             static_cast<hipStream_t>(stream)),
+                    "weight_quant");
+}
+
+int mdy_weight_dequant(const void* x, const float* s, void* y, int64_t N, int64_t K, int out_dtype, void* stream) {
+    if (out_dtype != MDY_DT_BF16 && out_dtype != MDY_DT_F32) return fail(MDY_E_DTYPE, "weight_dequant: unknown out_dtype %d", out_dtype);
+    if (N < 0 || K < 0 || N > kMaxDim || K > kMaxDim) return fail(MDY_E_SHAPE, "weight_dequant: bad shape");
+    if ((N + 15) / 16 > 65535) return fail(MDY_E_SHAPE, "weight_dequant: N too large");
+    if (N == 0 || K == 0) return 0;
+    if (!x || !s || !y) return fail(MDY_E_NULL, "weight_dequant: null pointer");
+    if (!aligned(y, out_dtype == MDY_DT_BF16 ? 2 : 4) || !aligned(s, 4)) return fail(MDY_E_ALIGN, "weight_dequant: misaligned pointer");
+    if (int e = check_device()) return e;
+    return launched(mdy::launch_weight_dequant(x, s, y, N, K, out_dtype, static_cast<hipStream_t>(stream)), "weight_dequant");
+}
+
+int mdy_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,
+                    const float* b_s, void* c, const void* bias, int64_t M, int64_t N, int64_t K, int out_dtype,
+                    void* stream) {
+    if (out_dtype != MDY_DT_BF16 && out_dtype != MDY_DT_F32) return fail(MDY_E_DTYPE, "fp8_gemm_nt: unknown out_dtype %d", out_dtype);
+    if (M < 0 || N < 0 || K < 1 || M > kMaxDim || N > kMaxDim || K > kMaxDim)
+        return fail(MDY_E_SHAPE, "fp8_gemm_nt: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+    if ((M + 15) / 16 > 65535) return fail(MDY_E_SHAPE, "fp8_gemm_nt: M too large");
+    if (M == 0 || N == 0) return 0;
+    if (!a || !a_s || !b || !b_s || !c) return fail(MDY_E_NULL, "fp8_gemm_nt: null pointer");
+    if (!aligned(c, out_dtype == MDY_DT_BF16 ? 2 : 4) || !aligned(a_s, 4) || !aligned(b_s, 4) || (bias && !aligned(bias, 2)))
+        return fail(MDY_E_ALIGN, "fp8_gemm_nt: misaligned pointer");
+    if (int e = check_device()) return e;
+    return launched(mdy::launch_fp8_gemm_nt(a, a_s, as_row_stride, as_col_stride, b, b_s, c, bias, M, N, K, out_dtype,
+                                            static_cast<hipStream_t>(stream)),
+                    "fp8_gemm_nt");
+}
+
+int mdy_add_bias(void* x, const void* b, int64_t M, int64_t N, void* stream) {
+    if (M < 0 || N < 0 || M > kMaxDim || N > kMaxDim) return fail(MDY_E_SHAPE, "add_bias: bad shape");
+    if (M == 0 || N == 0) return 0;
+    if (!x || !b) return fail(MDY_E_NULL, "add_bias: null pointer");
+    if (!aligned(x, 2) || !aligned(b, 2)) return fail(MDY_E_ALIGN, "add_bias: misaligned pointer");
+    if (int e = check_device()) return e;
+    return launched(mdy::launch_add_bias(x, b, M, N, static_cast<hipStream_t>(stream)), "add_bias");
+}
+
+int mdy_cast_f32_to_e4m3(const float* x, void* y, int64_t n, int saturate, void* stream) {
+    if (n < 0) return fail(MDY_E_SHAPE, "cast_f32_to_e4m3: n < 0");
+    if (n == 0) return 0;
+    if (!x || !y) return fail(MDY_E_NULL, "cast_f32_to_e4m3: null pointer");
+    if (int e = check_device()) return e;
+    return launched(mdy::launch_cast_f32_to_e4m3(x, y, n, saturate, static_cast<hipStream_t>(stream)), "cast_f32_to_e4m3");
+}
+
+int mdy_quotient_selfcheck(uint64_t* out, int amax_lo, int amax_hi, int mode, void* stream) {
+    if (!out) return fail(MDY_E_NULL, "quotient_selfcheck: null pointer");
+    if (amax_lo < 0 || amax_hi > 0x7F80 || amax_lo > amax_hi) return fail(MDY_E_SHAPE, "quotient_selfcheck: range must lie in [0, 0x7F80]");
+    if (mode != 0 && mode != 1) return fail(MDY_E_DTYPE, "quotient_selfcheck: unknown mode");
+    if (int e = check_device()) return e;
+    return launched(mdy::launch_quotient_selfcheck(out, amax_lo, amax_hi, mode, static_cast<hipStream_t>(stream)), "quotient_selfcheck");
+}
+
+}  // extern "C"

@@ -1,0 +1,93 @@
+// Shared device helpers and host-side launch declarations for libmdyfp8.so (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mdy {
+
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef int intx4 __attribute__((ext_vector_type(4)));
+typedef int intx8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+constexpr float kFp8Max = 448.0f;
+constexpr int kGroup = 128;  // quantization group / block edge
+
+// Smallest biased exponent of amax for which the reciprocal + 2-FMA quotient is
+// proven (exhaustively over all bf16 pairs) to give the same e4m3fn byte as IEEE
+// division in the official dialect; below it s = amax/448 is subnormal or the
+// residual underflows.  The DeepLinear dialect (eps keeps s normal) is clean for
+// every finite amax.
+constexpr uint32_t kFastQuotientMinExp = 23;
+
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); }
+__device__ __forceinline__ float bf16_one(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+
+// Scale of one quantization group from its absmax (fp32, IEEE division).
+template <int MODE>
+__device__ __forceinline__ float group_scale(float amax) {
+    if (MODE == 0) return amax / kFp8Max;
+    // clamp(amax, 0, 1e4) + 1e-8, NaN kept (fminf would drop it)
+    float c = amax > 1e4f ? 1e4f : amax;
+    return (c + 1e-8f) / kFp8Max;
+}
+
+// True when the fast quotient may be used for a group with this absmax.
+template <int MODE>
+__device__ __forceinline__ bool fast_quotient_ok(float amax) {
+    uint32_t b = __float_as_uint(amax);
+    if (MODE == 0) return b >= (kFastQuotientMinExp << 23) && b < 0x7F800000u;
+    return b < 0x7F800000u;
+}
+
+// x / s through r = RN(1/s): q0 = x*r, e = fma(q0, s, -x), q = fma(-e, r, q0).
+// The residual is kept negated so that x = -0 gives q = -0.
+__device__ __forceinline__ float fast_quotient(float x, float s, float r) {
+    float q0 = x * r;
+    float e = __builtin_fmaf(q0, s, -x);
+    return __builtin_fmaf(-e, r, q0);
+}
+
+template <int MODE>
+__device__ __forceinline__ float sat_for_mode(float q) {
+    // v_med3_f32 returns a non-NaN operand for a NaN input, so keep NaN by hand.
+    if (MODE == 0) return q;
+    float c = __builtin_amdgcn_fmed3f(q, -kFp8Max, kFp8Max);
+    return q != q ? q : c;
+}
+
+// four fp32 -> four e4m3fn bytes (RNE) packed little-endian into one dword
+__device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float d) {
+    int w = 0;
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, w, false);
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
+    return (uint32_t)w;
+}
+
+__device__ __forceinline__ uint32_t pack2_bf16(float a, float b) {
+    floatx2 f = {a, b};
+    bf16x2 h = __builtin_convertvector(f, bf16x2);
+    return __builtin_bit_cast(uint32_t, h);
+}
+
+// ---------------------------------------------------------------------------
+// host-side launchers (defined one per .hip file); all return hipError_t as int
+// ---------------------------------------------------------------------------
+int launch_act_quant(const void* x, void* y, float* s, int64_t M, int64_t K, int64_t x_row_stride,
+                     int64_t PM, int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode,
+                     hipStream_t stream);
+int launch_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t, int64_t N, int64_t K,
+                        int64_t w_row_stride, int64_t w_col_stride, int64_t PN, int64_t PK, int mode,
+                        hipStream_t stream);
+int launch_weight_dequant(const void* x, const float* s, void* y, int64_t N, int64_t K, int out_dtype,
+                          hipStream_t stream);
+int launch_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
+                       const void* b, const float* b_s, void* c, const void* bias, int64_t M, int64_t N,
+                       int64_t K, int out_dtype, hipStream_t stream);
+int launch_add_bias(void* x, const void* b, int64_t M, int64_t N, hipStream_t stream);
+int launch_cast_f32_to_e4m3(const float* x, void* y, int64_t n, int saturate, hipStream_t stream);
+int launch_quotient_selfcheck(uint64_t* out, int amax_lo, int amax_hi, int mode, hipStream_t stream);
+
+}  // namespace mdy

@@ -1,0 +1,393 @@
+// Block-scaled FP8 GEMM, NT layout, for gfx950 MFMA:
+//   c[m,n] = sum_kb (sum_{k in kb} a[m,k] b[n,k]) * a_s[m,kb] * b_s[n/128,kb] (+ bias[n])
+//
+// Restates fp8_gemm_kernel
+// (/root/reference/triton_kernels/deepseekv3/offical_kernel.py:61-97) and the contract
+// of the DeepGEMM call in /root/reference/triton_kernels/dpsk_fp8linear/fp8.py:307-311.
+//
+// Main kernel (K % 128 == 0):
+//   * one workgroup owns a BM x BN tile of C; per 128-wide K block the A and B
+//     panels (BM x 128 and BN x 128 bytes) are staged in LDS, double buffered;
+//   * LDS rows are 128 bytes; the eight 16-byte chunks of a row are XOR-swizzled
+//     with (row & 7) ^ (row>>3 & 1) so that both the 16-byte staging writes and the
+//     ds_read_b128 fragment reads are bank-conflict free;
+//   * v_mfma_f32_16x16x128_f8f6f4 consumes a whole 128-deep scale block per
+//     instruction.  The B rows go in as the MFMA "A" operand and the A rows as
+//     its "B" operand, so a lane ends up with 4 consecutive n of one m: the
+//     per-block scale a_s[m,kb]*b_s[n/128,kb] is ONE value per lane and
+//     sub-tile, and the epilogue stores 8 contiguous bytes per lane;
+//   * each MFMA starts from C = 0; its 4 results are folded into the fp32 master
+//     accumulator with v_fma_f32 (the promotion the reference does on its
+//     CUDA cores at offical_kernel.py:86);
+//   * workgroup ids are remapped so that the 32 workgroups that share an XCD's L2
+//     cover a compact 4 x 8 block of tiles.
+// Small-M kernel (M <= 64): weight streaming, one workgroup per 16 columns, waves
+// split K and reduce through LDS.  Scalar kernel: any other shape/alignment.
+#include "common.h"
+
+namespace mdy {
+
+// chunk swizzle of an LDS row; depends on row bits 0..3 only so that rows 16 apart share it
+__device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+template <typename OUT>
+__device__ __forceinline__ void store4(OUT* c, int64_t ldc, int m, int n, int M, int N, const float (&v)[4], bool vec_ok) {
+    if (m >= M || n >= N) return;
+    OUT* p = c + (int64_t)m * ldc + n;
+    if (vec_ok && n + 3 < N) {
+        if (sizeof(OUT) == 2) {
+            *reinterpret_cast<uint2*>(p) = make_uint2(pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]));
+        } else {
+            *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (n + i < N) {
+                if (sizeof(OUT) == 2)
+                    reinterpret_cast<uint16_t*>(p)[i] = (uint16_t)(pack2_bf16(v[i], 0.0f) & 0xFFFFu);
+                else
+                    reinterpret_cast<float*>(p)[i] = v[i];
+            }
+        }
+    }
+}
+
+// BM x BN block tile, WGM x WGN waves, each wave (BM/WGM) x (BN/WGN).
+template <int BM, int BN, int WGM, int WGN, typename OUT>
+__global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
+    const uint8_t* __restrict__ a, const float* __restrict__ a_s, int64_t as_rs, int64_t as_cs,
+    const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
+    const uint16_t* __restrict__ bias, int M, int N, int K, int tiles_m, int tiles_n) {
+    constexpr int T = WGM * WGN * 64;
+    constexpr int WM = BM / WGM, WN = BN / WGN;
+    constexpr int TI = WM / 16, TJ = WN / 16;
+    constexpr int A_CHUNKS = BM * 8 / T, B_CHUNKS = BN * 8 / T;
+    static_assert(BM * 8 % T == 0 && BN * 8 % T == 0, "tile/threads mismatch");
+    static_assert(WN % 16 == 0 && WM % 16 == 0, "wave tile must be a multiple of 16");
+
+    __shared__ __attribute__((aligned(16))) uint8_t lds_a[2][BM * 128];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_b[2][BN * 128];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WGN, wn = wave % WGN;
+
+    // ---- XCD-aware tile order: consecutive ids land on different XCDs (8 of them);
+    // give each XCD a contiguous run of tiles, walked in groups of 4 tile rows.
+    int pid = blockIdx.x;
+    const int ntiles = tiles_m * tiles_n;
+    {
+        const int per_xcd = (ntiles + 7) / 8;
+        const int xcd = pid & 7, local = pid >> 3;
+        int t = xcd * per_xcd + local;
+        if (ntiles % 8 != 0) t = pid;  // irregular counts: keep the plain order
+        pid = t;
+    }
+    constexpr int GM = 4;
+    const int group = pid / (GM * tiles_n);
+    const int first_m = group * GM;
+    const int gsz = min(tiles_m - first_m, GM);
+    const int tm = first_m + (pid % (GM * tiles_n)) % gsz;
+    const int tn = (pid % (GM * tiles_n)) / gsz;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    const int KB = K >> 7;
+
+    // ---- staging: thread -> (row, chunk) of the panels
+    const uint8_t* a_src[A_CHUNKS];
+    int a_dst[A_CHUNKS];
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) {
+        const int q = tid + T * i, row = q >> 3, ch = q & 7;
+        const int gr = min(m0 + row, M - 1);
+        a_src[i] = a + (int64_t)gr * K + ch * 16;
+        a_dst[i] = row * 128 + ((ch ^ swz(row)) << 4);
+    }
+    const uint8_t* b_src[B_CHUNKS];
+    int b_dst[B_CHUNKS];
+#pragma unroll
+    for (int i = 0; i < B_CHUNKS; ++i) {
+        const int q = tid + T * i, row = q >> 3, ch = q & 7;
+        const int gr = min(n0 + row, N - 1);
+        b_src[i] = b + (int64_t)gr * K + ch * 16;
+        b_dst[i] = row * 128 + ((ch ^ swz(row)) << 4);
+    }
+
+    // ---- fragment read offsets: lane -> row (lane%16) and the 32-byte K slice (lane/16)
+    const int frow = lane & 15, fk = lane >> 4;
+    int a_off[TI][2], b_off[TJ][2];
+#pragma unroll
+    for (int i = 0; i < TI; ++i) {
+        const int row = wm * WM + i * 16 + frow;
+        a_off[i][0] = row * 128 + (((2 * fk) ^ swz(row)) << 4);
+        a_off[i][1] = row * 128 + (((2 * fk + 1) ^ swz(row)) << 4);
+    }
+#pragma unroll
+    for (int j = 0; j < TJ; ++j) {
+        const int row = wn * WN + j * 16 + frow;
+        b_off[j][0] = row * 128 + (((2 * fk) ^ swz(row)) << 4);
+        b_off[j][1] = row * 128 + (((2 * fk + 1) ^ swz(row)) << 4);
+    }
+
+    // ---- scales: this lane's m for sub-tile i is m0 + wm*WM + 16*i + lane%16
+    const float* as_ptr[TI];
+#pragma unroll
+    for (int i = 0; i < TI; ++i) {
+        const int m = min(m0 + wm * WM + i * 16 + frow, M - 1);
+        as_ptr[i] = a_s + (int64_t)m * as_rs;
+    }
+    const int sKB = KB;  // row stride of b_s
+    // sub-tile j covers n0 + wn*WN + 16*j .. +15, inside one 128-block
+    int bs_row[TJ];
+#pragma unroll
+    for (int j = 0; j < TJ; ++j) bs_row[j] = min(n0 + wn * WN + 16 * j, N - 1) >> 7;
+
+    floatx4 acc[TI][TJ];
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    // ---- prologue: stage K block 0
+    intx4 ra[A_CHUNKS], rb[B_CHUNKS];
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) ra[i] = *reinterpret_cast<const intx4*>(a_src[i]);
+#pragma unroll
+    for (int i = 0; i < B_CHUNKS; ++i) rb[i] = *reinterpret_cast<const intx4*>(b_src[i]);
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) *reinterpret_cast<intx4*>(&lds_a[0][a_dst[i]]) = ra[i];
+#pragma unroll
+    for (int i = 0; i < B_CHUNKS; ++i) *reinterpret_cast<intx4*>(&lds_b[0][b_dst[i]]) = rb[i];
+    __syncthreads();
+
+    for (int kb = 0; kb < KB; ++kb) {
+        const int cur = kb & 1;
+        const bool has_next = kb + 1 < KB;
+        if (has_next) {
+#pragma unroll
+            for (int i = 0; i < A_CHUNKS; ++i) ra[i] = *reinterpret_cast<const intx4*>(a_src[i] + (int64_t)(kb + 1) * 128);
+#pragma unroll
+            for (int i = 0; i < B_CHUNKS; ++i) rb[i] = *reinterpret_cast<const intx4*>(b_src[i] + (int64_t)(kb + 1) * 128);
+        }
+        // combined scale per (i, distinct b_s row)
+        float sa[TI];
+#pragma unroll
+        for (int i = 0; i < TI; ++i) sa[i] = as_ptr[i][(int64_t)kb * as_cs];
+        float sb[TJ];
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) sb[j] = b_s[(int64_t)bs_row[j] * sKB + kb];
+
+        intx8 fa[TI];
+#pragma unroll
+        for (int i = 0; i < TI; ++i) {
+            const intx4 lo = *reinterpret_cast<const intx4*>(&lds_a[cur][a_off[i][0]]);
+            const intx4 hi = *reinterpret_cast<const intx4*>(&lds_a[cur][a_off[i][1]]);
+            fa[i] = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+            const intx4 lo = *reinterpret_cast<const intx4*>(&lds_b[cur][b_off[j][0]]);
+            const intx4 hi = *reinterpret_cast<const intx4*>(&lds_b[cur][b_off[j][1]]);
+            const intx8 fb = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+#pragma unroll
+            for (int i = 0; i < TI; ++i) {
+                const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+                // rows of the MFMA = n (B panel), columns = m (A panel)
+                const floatx4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa[i], zero, 0, 0, 0, 0, 0, 0);
+                const float sc = sa[i] * sb[j];
+                acc[i][j][0] = __builtin_fmaf(p[0], sc, acc[i][j][0]);
+                acc[i][j][1] = __builtin_fmaf(p[1], sc, acc[i][j][1]);
+                acc[i][j][2] = __builtin_fmaf(p[2], sc, acc[i][j][2]);
+                acc[i][j][3] = __builtin_fmaf(p[3], sc, acc[i][j][3]);
+            }
+        }
+        if (has_next) {
+            const int nxt = cur ^ 1;
+#pragma unroll
+            for (int i = 0; i < A_CHUNKS; ++i) *reinterpret_cast<intx4*>(&lds_a[nxt][a_dst[i]]) = ra[i];
+#pragma unroll
+            for (int i = 0; i < B_CHUNKS; ++i) *reinterpret_cast<intx4*>(&lds_b[nxt][b_dst[i]]) = rb[i];
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue: lane holds c[m][n..n+3], m = .. + lane%16, n = .. + 4*(lane/16)
+    const bool vec_ok = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
+#pragma unroll
+    for (int i = 0; i < TI; ++i) {
+        const int m = m0 + wm * WM + i * 16 + frow;
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+            const int n = n0 + wn * WN + j * 16 + 4 * fk;
+            float v[4] = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+            if (bias != nullptr) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (n + e < N) v[e] += bf16_one(bias[n + e]);
+            }
+            store4<OUT>(c, N, m, n, M, N, v, vec_ok);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Small-M kernel: M <= 16*MT rows.  One workgroup (4 waves) per 16 output
+// columns; wave w handles K blocks w, w+4, ...; B fragments come straight from
+// global memory (each row slice is one full 128-byte line), A fragments too (A is
+// tiny and L2 resident).  Partial sums are reduced through LDS.
+// ---------------------------------------------------------------------------
+template <int MT, typename OUT>
+__global__ __launch_bounds__(256) void fp8_gemm_smallm_kernel(const uint8_t* __restrict__ a,
+                                                               const float* __restrict__ a_s, int64_t as_rs,
+                                                               int64_t as_cs, const uint8_t* __restrict__ b,
+                                                               const float* __restrict__ b_s, OUT* __restrict__ c,
+                                                               const uint16_t* __restrict__ bias, int M, int N, int K) {
+    __shared__ float red[4][MT][64][4];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int frow = lane & 15, fk = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    const int KB = K >> 7;
+    const int nrow = min(n0 + frow, N - 1);
+    const uint8_t* bp = b + (int64_t)nrow * K + fk * 32;
+    const float* bsp = b_s + (int64_t)(n0 >> 7) * KB;
+
+    floatx4 acc[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    for (int kb = wave; kb < KB; kb += 4) {
+        const intx4 blo = *reinterpret_cast<const intx4*>(bp + (int64_t)kb * 128);
+        const intx4 bhi = *reinterpret_cast<const intx4*>(bp + (int64_t)kb * 128 + 16);
+        const intx8 fb = intx8{blo[0], blo[1], blo[2], blo[3], bhi[0], bhi[1], bhi[2], bhi[3]};
+        const float sb = bsp[kb];
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const int m = min(i * 16 + frow, M - 1);
+            const uint8_t* ap = a + (int64_t)m * K + (int64_t)kb * 128 + fk * 32;
+            const intx4 alo = *reinterpret_cast<const intx4*>(ap);
+            const intx4 ahi = *reinterpret_cast<const intx4*>(ap + 16);
+            const intx8 fa = intx8{alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
+            const float sc = a_s[(int64_t)m * as_rs + (int64_t)kb * as_cs] * sb;
+            const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+            const floatx4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, zero, 0, 0, 0, 0, 0, 0);
+            acc[i][0] = __builtin_fmaf(p[0], sc, acc[i][0]);
+            acc[i][1] = __builtin_fmaf(p[1], sc, acc[i][1]);
+            acc[i][2] = __builtin_fmaf(p[2], sc, acc[i][2]);
+            acc[i][3] = __builtin_fmaf(p[3], sc, acc[i][3]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) red[wave][i][lane][e] = acc[i][e];
+    __syncthreads();
+    if (wave == 0) {
+        const bool vec_ok = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                v[e] = (red[0][i][lane][e] + red[1][i][lane][e]) + (red[2][i][lane][e] + red[3][i][lane][e]);
+            const int m = i * 16 + frow, n = n0 + 4 * fk;
+            if (bias != nullptr) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (n + e < N) v[e] += bf16_one(bias[n + e]);
+            }
+            store4<OUT>(c, N, m, n, M, N, v, vec_ok);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Scalar kernel: any M, N, K, any alignment (K tail reads as zero, like the masked
+// loads at offical_kernel.py:82-83).  One thread per output element.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float e4m3_to_f32(uint8_t v) {
+    floatx2 f = __builtin_amdgcn_cvt_pk_f32_fp8((int)v, false);
+    return f.x;
+}
+
+template <typename OUT>
+__global__ __launch_bounds__(256) void fp8_gemm_scalar_kernel(const uint8_t* __restrict__ a,
+                                                               const float* __restrict__ a_s, int64_t as_rs,
+                                                               int64_t as_cs, const uint8_t* __restrict__ b,
+                                                               const float* __restrict__ b_s, OUT* __restrict__ c,
+                                                               const uint16_t* __restrict__ bias, int M, int N, int K) {
+    const int n = blockIdx.x * 16 + (threadIdx.x & 15);
+    const int m = blockIdx.y * 16 + (threadIdx.x >> 4);
+    if (m >= M || n >= N) return;
+    const int KB = (K + 127) >> 7;
+    float acc = 0.0f;
+    for (int kb = 0; kb < KB; ++kb) {
+        float p = 0.0f;
+        const int k1 = min(K, (kb + 1) * 128);
+        for (int k = kb * 128; k < k1; ++k)
+            p = __builtin_fmaf(e4m3_to_f32(a[(int64_t)m * K + k]), e4m3_to_f32(b[(int64_t)n * K + k]), p);
+        const float sc = a_s[(int64_t)m * as_rs + (int64_t)kb * as_cs] * b_s[(int64_t)(n >> 7) * KB + kb];
+        acc = __builtin_fmaf(p, sc, acc);
+    }
+    if (bias != nullptr) acc += bf16_one(bias[n]);
+    if (sizeof(OUT) == 2)
+        reinterpret_cast<uint16_t*>(c)[(int64_t)m * N + n] = (uint16_t)(pack2_bf16(acc, 0.0f) & 0xFFFFu);
+    else
+        reinterpret_cast<float*>(c)[(int64_t)m * N + n] = acc;
+}
+
+template <int BM, int BN, int WGM, int WGN, typename OUT>
+static int launch_mfma(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, const uint8_t* b,
+                       const float* b_s, OUT* c, const uint16_t* bias, int M, int N, int K, hipStream_t stream) {
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    dim3 grid((unsigned)(tiles_m * tiles_n)), block(WGM * WGN * 64);
+    hipLaunchKernelGGL((fp8_gemm_mfma_kernel<BM, BN, WGM, WGN, OUT>), grid, block, 0, stream, a, a_s, as_rs, as_cs, b,
+                       b_s, c, bias, M, N, K, tiles_m, tiles_n);
+    return (int)hipGetLastError();
+}
+
+template <typename OUT>
+static int dispatch(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, const uint8_t* b,
+                    const float* b_s, OUT* c, const uint16_t* bias, int M, int N, int K, hipStream_t stream) {
+    const bool mfma_ok = (K % 128 == 0) && ((reinterpret_cast<uintptr_t>(a) & 15) == 0) &&
+                         ((reinterpret_cast<uintptr_t>(b) & 15) == 0);
+    if (!mfma_ok) {
+        dim3 grid((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16));
+        hipLaunchKernelGGL((fp8_gemm_scalar_kernel<OUT>), grid, dim3(256), 0, stream, a, a_s, as_rs, as_cs, b, b_s, c,
+                           bias, M, N, K);
+        return (int)hipGetLastError();
+    }
+    if (M <= 64) {
+        dim3 grid((unsigned)((N + 15) / 16));
+#define MDY_SM(MT)                                                                                                 \
+    hipLaunchKernelGGL((fp8_gemm_smallm_kernel<MT, OUT>), grid, dim3(256), 0, stream, a, a_s, as_rs, as_cs, b, b_s, \
+                       c, bias, M, N, K)
+        if (M <= 16) MDY_SM(1);
+        else if (M <= 32) MDY_SM(2);
+        else if (M <= 48) MDY_SM(3);
+        else MDY_SM(4);
+#undef MDY_SM
+        return (int)hipGetLastError();
+    }
+    const long tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);
+    if (tiles256 >= 128) return launch_mfma<256, 128, 2, 2, OUT>(a, a_s, as_rs, as_cs, b, b_s, c, bias, M, N, K, stream);
+    return launch_mfma<128, 128, 2, 2, OUT>(a, a_s, as_rs, as_cs, b, b_s, c, bias, M, N, K, stream);
+}
+
+int launch_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,
+                       const float* b_s, void* c, const void* bias, int64_t M, int64_t N, int64_t K, int out_dtype,
+                       hipStream_t stream) {
+    if (M == 0 || N == 0) return 0;
+    const uint8_t* ap = static_cast<const uint8_t*>(a);
+    const uint8_t* bp = static_cast<const uint8_t*>(b);
+    const uint16_t* biasp = static_cast<const uint16_t*>(bias);
+    if (out_dtype == 0)
+        return dispatch<uint16_t>(ap, a_s, as_row_stride, as_col_stride, bp, b_s, static_cast<uint16_t*>(c), biasp,
+                                  (int)M, (int)N, (int)K, stream);
+    return dispatch<float>(ap, a_s, as_row_stride, as_col_stride, bp, b_s, static_cast<float*>(c), biasp, (int)M,
+                           (int)N, (int)K, stream);
+}
+
+}  // namespace mdy

@@ -1,0 +1,140 @@
+// 128x128 block weight quantizer: bf16 -> e4m3fn bytes + one fp32 scale per block,
+// optionally also the transposed copy (for the backward GEMMs).
+//
+// Restates _quant_weight_kernel
+// (/root/reference/triton_kernels/dpsk_fp8linear/fp8.py:171-203; clamp + eps dialect)
+// and _weight_quant_block_kernel
+// (/root/reference/triton_kernels/deepseekv3/fp8_kernel.py:88-122; plain amax/448).
+//
+// One 256-thread block per 128x128 tile.  Thread t owns columns (t%16)*8..+7 of
+// rows t/16 + 16*i, i = 0..7: eight 16-byte loads kept in registers (the tile is
+// read from HBM exactly once), absmax by DPP inside 16-lane rows, ds_swizzle-free
+// cross-row reduction with __shfl_xor, four wave results combined through LDS.
+// The quotient is the same reciprocal + 2-FMA form as the activation quantizer.
+// The transposed copy goes through a padded LDS byte tile.
+//
+// HBM traffic per element: 2 B in + 1 B out (+ 1 B for the transposed copy).
+#include "common.h"
+
+namespace mdy {
+
+template <int MODE, bool VEC>
+__global__ __launch_bounds__(256) void weight_quant_kernel(const uint16_t* __restrict__ w, uint8_t* __restrict__ y,
+                                                            float* __restrict__ s, uint8_t* __restrict__ y_t,
+                                                            float* __restrict__ s_t, int N, int K, int64_t w_row_stride,
+                                                            int64_t w_col_stride, int PN, int PK) {
+    __shared__ float wave_max[4];
+    __shared__ __attribute__((aligned(16))) uint8_t tile[128][128 + 16];
+
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    const int wave = t >> 6;
+    const int bn = blockIdx.y;  // block row (along N)
+    const int bk = blockIdx.x;  // block column (along K)
+    const int c0 = bk * 128 + (t & 15) * 8;
+    const int rbase = bn * 128 + (t >> 4);
+
+    float f[8][8];
+    float m = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int row = rbase + 16 * i;
+        uint32_t wd[4] = {0u, 0u, 0u, 0u};
+        if (row < N && c0 < K) {
+            if (VEC) {
+                const uint4 v = *reinterpret_cast<const uint4*>(w + (int64_t)row * w_row_stride + c0);
+                wd[0] = v.x; wd[1] = v.y; wd[2] = v.z; wd[3] = v.w;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (c0 + j < K)
+                        wd[j >> 1] |= (uint32_t)w[(int64_t)row * w_row_stride + (int64_t)(c0 + j) * w_col_stride]
+                                      << ((j & 1) * 16);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            f[i][2 * j] = bf16_lo(wd[j]);
+            f[i][2 * j + 1] = bf16_hi(wd[j]);
+            m = fmaxf(fmaxf(fabsf(f[i][2 * j]), fabsf(f[i][2 * j + 1])), m);
+        }
+    }
+    // wave-wide max, then across the 4 waves
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+    if (lane == 0) wave_max[wave] = m;
+    __syncthreads();
+    const float amax = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+
+    const float sc = group_scale<MODE>(amax);
+    const bool fast = MODE == 0 ? fast_quotient_ok<0>(amax) : (amax <= 1e4f);
+    const float r = 1.0f / sc;
+    if (t == 0) {
+        s[(int64_t)bn * (PK >> 7) + bk] = sc;
+        if (s_t) s_t[(int64_t)bk * (PN >> 7) + bn] = sc;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        float q[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (fast) {
+                q[j] = fast_quotient(f[i][j], sc, r);
+            } else {
+                float v = f[i][j] / sc;
+                if (MODE != 0) {
+                    float c = __builtin_amdgcn_fmed3f(v, -kFp8Max, kFp8Max);
+                    v = (v != v) ? v : c;
+                }
+                q[j] = v;
+            }
+        }
+        uint2 o;
+        o.x = pack4_e4m3(q[0], q[1], q[2], q[3]);
+        o.y = pack4_e4m3(q[4], q[5], q[6], q[7]);
+        const int row = rbase + 16 * i;  // < PN because PN % 128 == 0
+        *reinterpret_cast<uint2*>(y + (int64_t)row * PK + c0) = o;
+        if (y_t) *reinterpret_cast<uint2*>(&tile[(t >> 4) + 16 * i][(t & 15) * 8]) = o;
+    }
+    if (y_t) {
+        __syncthreads();
+        // y_t[k][n]: thread owns output columns (t%16)*8..+7 (n) of output rows t/16 + 16*i (k)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int kk = (t >> 4) + 16 * i;
+            const int nn = (t & 15) * 8;
+            uint32_t lo = 0u, hi = 0u;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                lo |= (uint32_t)tile[nn + j][kk] << (8 * j);
+                hi |= (uint32_t)tile[nn + 4 + j][kk] << (8 * j);
+            }
+            *reinterpret_cast<uint2*>(y_t + (int64_t)(bk * 128 + kk) * PN + bn * 128 + nn) = make_uint2(lo, hi);
+        }
+    }
+}
+
+int launch_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t, int64_t N, int64_t K,
+                        int64_t w_row_stride, int64_t w_col_stride, int64_t PN, int64_t PK, int mode,
+                        hipStream_t stream) {
+    if (PN == 0 || PK == 0) return 0;
+    dim3 grid((unsigned)(PK / 128), (unsigned)(PN / 128));
+    dim3 block(256);
+    const bool vec = (w_col_stride == 1) && (K % 8 == 0) && (w_row_stride % 8 == 0) &&
+                     ((reinterpret_cast<uintptr_t>(w) & 15) == 0);
+    const uint16_t* wp = static_cast<const uint16_t*>(w);
+    uint8_t* yp = static_cast<uint8_t*>(y);
+    uint8_t* ytp = static_cast<uint8_t*>(y_t);
+#define MDY_WQ(MODE, VEC)                                                                                      \
+    hipLaunchKernelGGL((weight_quant_kernel<MODE, VEC>), grid, block, 0, stream, wp, yp, s, ytp, s_t, (int)N, \
+                       (int)K, w_row_stride, w_col_stride, (int)PN, (int)PK)
+    if (mode == 0) {
+        if (vec) MDY_WQ(0, true); else MDY_WQ(0, false);
+    } else {
+        if (vec) MDY_WQ(1, true); else MDY_WQ(1, false);
+    }
+#undef MDY_WQ
+    return (int)hipGetLastError();
+}
+
+}  // namespace mdy

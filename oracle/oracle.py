@@ -1,0 +1,273 @@
+"""CPU oracle for the block-wise FP8 linear path.
+
+TEST INFRASTRUCTURE, NOT PRODUCT CODE.  Only `tests/`, `__graft_entry__.smoke()`
+and the `cpu_baseline` leg of `bench.py` may import this module; the product
+package (`mdy_triton_amd`) never imports anything from `oracle/` and has no CPU
+fallback.
+
+Every function restates, with torch CPU tensor ops in IEEE fp32, the algorithm
+of one reference function and cites it.  All paths are under /root/reference.
+
+Pinning status (what fixes each function besides its own formula):
+  act_quant / quant_input / quant_weight / weight_quant_block
+      the fp32->e4m3fn cast is pinned against the from-definition codec in
+      oracle/fp8_format.py on every code, every rounding midpoint +-1 ulp,
+      subnormals, 448/464/465, +-0, NaN, inf; the scale against numpy float32
+      division; invariants (the amax element encodes to +-448, half-ulp
+      reconstruction bound, idempotence) and hand-computed fixtures in
+      tests/golden/.
+  weight_dequant
+      s == 1 reduces to the 256-entry decode table; one fp32 multiply + RNE
+      to bf16 re-derived in numpy integer arithmetic.
+  fp8_gemm
+      float64 matmul on small shapes; exactly-representable integer cases that
+      must match bit for bit; one-hot rows; single-scale-block perturbation.
+  fp8_matmul (DeepLinear's GEMM)
+      PARITY UNPINNED at the third-party boundary: the reference calls
+      `deep_gemm.gemm_fp8_fp8_bf16_nt` (dpsk_fp8linear/fp8.py:310), an
+      un-vendored, un-pinned package whose source is not in the reference and
+      whose only recorded outputs are unseeded notebook prints.  The oracle
+      follows the in-tree formula with the same contract
+      (deepseekv3/offical_kernel.py:81-92) instead.
+"""
+from typing import Optional, Tuple
+
+import torch
+
+FP8 = torch.float8_e4m3fn
+FP8_MAX = 448.0
+BLOCK = 128
+
+
+def _cdiv(a: int, b: int) -> int:
+    return (a + b - 1) // b
+
+
+# ----------------------------------------------------------------------------
+# DeepSeek "official" dialect
+# ----------------------------------------------------------------------------
+def act_quant(x: torch.Tensor, block_size: int = BLOCK) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per 128 contiguous elements: s = max|x| / 448 ; y = (x / s) -> e4m3fn.
+
+    Follows triton_kernels/deepseekv3/offical_kernel.py:9-18 (kernel) and
+    :21-28 (launcher: contiguous, last dim % block_size == 0, y same shape,
+    s shape [..., K/block_size] fp32).  No eps, no clamp: an all-zero group gives
+    s = 0 and y = 0/0 = NaN.
+    """
+    assert x.is_contiguous()
+    assert x.size(-1) % block_size == 0
+    xf = x.detach().cpu().float().reshape(-1, block_size)
+    s = xf.abs().amax(dim=-1) / FP8_MAX                     # offical_kernel.py:14
+    y = (xf / s[:, None]).to(FP8)                           # offical_kernel.py:15-16
+    y = y.reshape(x.shape)
+    s = s.reshape(*x.shape[:-1], x.size(-1) // block_size)
+    return y, s
+
+
+def weight_dequant(x: torch.Tensor, s: torch.Tensor, block_size: int = BLOCK,
+                   dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """y[m, n] = fp32(x[m, n]) * s[m // 128, n // 128], rounded once to `dtype`.
+
+    Follows offical_kernel.py:31-43 (kernel; edge tiles masked at :39) and :46-53
+    (2-D contiguous inputs; output dtype is the caller's default dtype at :50).
+    """
+    assert x.is_contiguous() and s.is_contiguous()
+    assert x.dim() == 2 and s.dim() == 2
+    M, N = x.shape
+    assert s.shape == (_cdiv(M, block_size), _cdiv(N, block_size))
+    xf = x.detach().cpu().float()
+    sf = s.detach().cpu().float()
+    sfull = sf.repeat_interleave(block_size, 0)[:M].repeat_interleave(block_size, 1)[:, :N]
+    return (xf * sfull).to(dtype)                           # offical_kernel.py:42
+
+
+def dequant_rows(a: torch.Tensor, a_s: torch.Tensor, block_size: int = BLOCK) -> torch.Tensor:
+    """fp32 a[m, k] * a_s[m, k // 128] (activation side of the GEMM)."""
+    K = a.size(-1)
+    af = a.detach().cpu().float().reshape(-1, K)
+    sf = a_s.detach().cpu().float().reshape(af.size(0), -1)
+    return af * sf.repeat_interleave(block_size, 1)[:, :K]
+
+
+def fp8_gemm(a: torch.Tensor, a_s: torch.Tensor, b: torch.Tensor, b_s: torch.Tensor,
+             dtype: torch.dtype = torch.bfloat16, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """C = A . B^T with per-128-K scales: dequantize both operands, fp32 matmul.
+
+    C[m, n] = sum_kb (sum_{k in kb} a[m,k] b[n,k]) * a_s[m,kb] * b_s[n//128,kb]
+    (offical_kernel.py:81-92; launcher :100-109: a [.., K], b [N, K], a_s
+    [.., cdiv(K,128)], b_s [cdiv(N,128), cdiv(K,128)], out [.., N]).  Equal in
+    exact arithmetic to dequant(a) @ dequant(b).T, which is what is evaluated
+    here in fp32 and what the parity tolerance (rtol 1e-2, atol 1e-2) refers to.
+    """
+    K = a.size(-1)
+    N = b.size(0)
+    ad = dequant_rows(a, a_s)
+    bd = weight_dequant(b.reshape(N, K).contiguous(), b_s.contiguous(), dtype=torch.float32)
+    c = ad @ bd.t()
+    if bias is not None:
+        c = c + bias.detach().cpu().float()
+    return c.to(dtype).reshape(*a.shape[:-1], N)
+
+
+def fp8_gemm_f64(a, a_s, b, b_s) -> torch.Tensor:
+    """Same contraction in float64 (tight truth for small shapes); returns float64 [M, N]."""
+    K = a.size(-1)
+    N = b.size(0)
+    ad = a.detach().cpu().double().reshape(-1, K) * \
+        a_s.detach().cpu().double().reshape(-1, a_s.size(-1)).repeat_interleave(BLOCK, 1)[:, :K]
+    bd = b.detach().cpu().double().reshape(N, K) * \
+        b_s.detach().cpu().double().repeat_interleave(BLOCK, 0)[:N].repeat_interleave(BLOCK, 1)[:, :K]
+    return ad @ bd.t()
+
+
+def fp8_gemm_blockwise(a, a_s, b, b_s, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """The accumulation order of the kernel itself: one fp32 partial dot per
+    128-K block, scaled, then added (offical_kernel.py:80-91).  Small shapes only."""
+    K = a.size(-1)
+    N = b.size(0)
+    af = a.detach().cpu().float().reshape(-1, K)
+    bf = b.detach().cpu().float().reshape(N, K)
+    M = af.size(0)
+    asf = a_s.detach().cpu().float().reshape(M, -1)
+    bsf = b_s.detach().cpu().float()
+    acc = torch.zeros(M, N, dtype=torch.float32)
+    nrow = torch.arange(N) // BLOCK
+    for kb in range(_cdiv(K, BLOCK)):
+        k0, k1 = kb * BLOCK, min(K, (kb + 1) * BLOCK)
+        part = af[:, k0:k1] @ bf[:, k0:k1].t()
+        acc += part * asf[:, kb][:, None] * bsf[nrow, kb][None, :]
+    return acc.to(dtype).reshape(*a.shape[:-1], N)
+
+
+def weight_quant_block(w: torch.Tensor, block_size: int = BLOCK) -> Tuple[torch.Tensor, torch.Tensor]:
+    """128x128 block quantizer without eps: s = max|blk| / 448 ; y = blk / s.
+
+    Follows triton_kernels/deepseekv3/fp8_kernel.py:117-122 with
+    MAX = finfo(e4m3fn).max (:133); this is how block-quantized test weights
+    are produced.  Requires both dims % 128 == 0 (U = M // BLOCK_M at :128-129).
+    """
+    N, K = w.shape
+    assert N % block_size == 0 and K % block_size == 0
+    wf = w.detach().cpu().float().reshape(N // block_size, block_size, K // block_size, block_size)
+    s = wf.abs().amax(dim=(1, 3)) / FP8_MAX
+    y = (wf / s[:, None, :, None]).to(FP8).reshape(N, K)
+    return y, s
+
+
+# ----------------------------------------------------------------------------
+# DeepLinear dialect (clamp + eps, padded, column-major activation scales)
+# ----------------------------------------------------------------------------
+def _scale_from_amax(amax: torch.Tensor) -> torch.Tensor:
+    """clamp(amax, 0, 1e4) + 1e-8, then / 448, all in fp32 (fp8.py:109-110, 194-195)."""
+    return (amax.clamp(min=0.0, max=1e4) + torch.tensor(1e-8, dtype=torch.float32)) / 448
+
+
+def _cast_sat(v: torch.Tensor) -> torch.Tensor:
+    """fp32 -> e4m3fn with finite overflow saturating at +-448.
+
+    The reference's cast is the implicit one of `tl.store` to an fp8 pointer
+    (fp8.py:112, 198), which is `cvt.rn.satfinite` on the hardware it targets;
+    torch's CPU cast alone would turn |v| >= 465 into NaN.
+    """
+    return torch.where(v.isnan(), v, v.clamp(-FP8_MAX, FP8_MAX)).to(FP8)
+
+
+def quant_input(x: torch.Tensor, only_forward: bool = True):
+    """1x128 activation quantizer of DeepLinear.
+
+    Follows dpsk_fp8linear/fp8.py:87-120 (kernel) and :122-161 (launcher):
+    PN = cdiv(K,256)*256; PM = cdiv(M,4)*4 (forward only) or cdiv(M,256)*256;
+    padded elements read as 0 (:108); y [PM, PN] row-major; scales written
+    S[kb*PM + m] (:113) and returned transposed: logical [PM, B], strides (1, PM).
+    With only_forward=False also the transposed copy quantized per 128x128 block
+    with the block's max of the row amax' values (:115-120): y_t [PN, PM],
+    s_t [B, A] with A = PM/128.
+    """
+    M, K = x.shape
+    PN = _cdiv(K, 256) * 256
+    B = PN // BLOCK
+    PM = _cdiv(M, 4) * 4 if only_forward else _cdiv(M, 256) * 256
+    xp = torch.zeros(PM, PN, dtype=torch.float32)
+    xp[:M, :K] = x.detach().cpu().float()
+    g = xp.reshape(PM, B, BLOCK)
+    amaxp = g.abs().amax(-1).clamp(min=0.0, max=1e4) + torch.tensor(1e-8, dtype=torch.float32)
+    scale = amaxp / 448                                      # [PM, B]
+    y = _cast_sat(g / scale[:, :, None]).reshape(PM, PN)
+    s = scale.t().contiguous().t()                           # logical [PM, B], strides (1, PM)
+    if only_forward:
+        return y, s, None, None
+    A = PM // BLOCK
+    blk_amax = amaxp.reshape(A, BLOCK, B).amax(1)            # fp8.py:116 max over rows of the tile
+    blk_scale = blk_amax / 448                               # [A, B]
+    yb = g.reshape(A, BLOCK, B, BLOCK) / blk_scale[:, None, :, None]
+    y_t = _cast_sat(yb).reshape(PM, PN).t().contiguous()     # [PN, PM]
+    s_t = blk_scale.t().contiguous()                         # [B, A] (fp8.py:120)
+    return y, s, y_t, s_t
+
+
+def quant_weight(w: torch.Tensor, only_forward: bool = True):
+    """128x128 weight quantizer of DeepLinear.
+
+    Follows fp8.py:171-203 (kernel) and :206-247 (launcher): rows padded to 128
+    (256 when training), columns to 256; y [PM, PN]; s [A, B] row-major (:199);
+    with only_forward=False also y_t [PN, PM] and s_t [B, A] (:201-203).
+    """
+    N, K = w.shape
+    BA = 128 if only_forward else 256
+    PM, PN = _cdiv(N, BA) * BA, _cdiv(K, 256) * 256
+    A, B = PM // BLOCK, PN // BLOCK
+    wp = torch.zeros(PM, PN, dtype=torch.float32)
+    wp[:N, :K] = w.detach().cpu().float()
+    g = wp.reshape(A, BLOCK, B, BLOCK)
+    scale = _scale_from_amax(g.abs().amax(dim=(1, 3)))       # [A, B]
+    y = _cast_sat(g / scale[:, None, :, None]).reshape(PM, PN)
+    if only_forward:
+        return y, scale, None, None
+    return y, scale, y.t().contiguous(), scale.t().contiguous()
+
+
+def quant_grad_output(dy: torch.Tensor):
+    """Row-wise 1x128 and column-wise 128x1 quantization of the output gradient.
+
+    Follows fp8.py:13-44 (kernel) and :47-77 (launcher): PM, PN padded to 256;
+    y [PM, PN] with scales returned as logical [PM, B] (col-major); y_t [PN, PM]
+    quantized along M in groups of 128 with scales returned as logical [PN, A].
+    """
+    M, N = dy.shape
+    PM, PN = _cdiv(M, 256) * 256, _cdiv(N, 256) * 256
+    A, B = PM // BLOCK, PN // BLOCK
+    xp = torch.zeros(PM, PN, dtype=torch.float32)
+    xp[:M, :N] = dy.detach().cpu().float()
+    g = xp.reshape(PM, B, BLOCK)
+    scale = _scale_from_amax(g.abs().amax(-1))               # [PM, B]
+    y = _cast_sat(g / scale[:, :, None]).reshape(PM, PN)
+    s = scale.t().contiguous().t()
+    gt = xp.t().contiguous().reshape(PN, A, BLOCK)
+    scale_t = _scale_from_amax(gt.abs().amax(-1))            # [PN, A]
+    y_t = _cast_sat(gt / scale_t[:, :, None]).reshape(PN, PM)
+    s_t = scale_t.t().contiguous().t()
+    return y, s, y_t, s_t
+
+
+def add_bias(x: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """x[r, :] = (fp32(x[r, :]) + fp32(b)) -> x.dtype  (fp8.py:283-295, 297-305)."""
+    return (x.detach().cpu().float() + b.detach().cpu().float()).to(x.dtype)
+
+
+def fp8_matmul(qa, sa, qb, sb) -> torch.Tensor:
+    """bf16 out[PM, PNw] of DeepLinear's GEMM call (fp8.py:307-311); sa may be
+    column-major.  Third-party boundary: see the module header."""
+    return fp8_gemm(qa, sa.contiguous(), qb, sb.contiguous(), dtype=torch.bfloat16)
+
+
+def deep_linear_forward(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """Composition of fp8.py:313-328: flatten, quant_input, quant_weight,
+    fp8_matmul, add_bias, view back."""
+    shape = x.shape
+    x2 = x.reshape(-1, shape[-1])
+    qa, sa, _, _ = quant_input(x2, True)
+    qb, sb, _, _ = quant_weight(weight, True)
+    out = fp8_matmul(qa, sa, qb, sb)
+    if bias is not None:
+        out = add_bias(out, bias)
+    return out.view(*shape[:-1], -1)

@@ -1,0 +1,210 @@
+"""GPU parity of the block-scaled FP8 GEMM and of DeepLinear against the CPU oracle.
+
+Tolerance (from the benchmark definition): bf16 output within rtol 1e-2 / atol 1e-2 of
+dequantize-then-fp32-matmul.  Exactly-representable cases must match bit for bit."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import mdy_triton_amd as m
+from oracle import oracle as O
+from tests import problems as P
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+FP8 = torch.float8_e4m3fn
+DEV = "cuda:0"
+RTOL, ATOL = 1e-2, 1e-2
+
+
+def close(got, ref):
+    return torch.allclose(got.float().cpu(), ref.float(), rtol=RTOL, atol=ATOL)
+
+
+def quantized_problem(kind, M, N, K, seed):
+    x = P.activations(kind, M, K, seed)
+    a, a_s = O.act_quant(x)
+    _, wq, ws = P.weights(N, K, seed + 1000)
+    return a, a_s, wq, ws
+
+
+def test_gemm_golden_exact_bits():
+    d = np.load(os.path.join(GOLD, "gemm_exact.npz"))
+    a = torch.from_numpy(d["a"]).view(FP8).to(DEV)
+    b = torch.from_numpy(d["b"]).view(FP8).to(DEV)
+    a_s, b_s = torch.from_numpy(d["a_s"]).to(DEV), torch.from_numpy(d["b_s"]).to(DEV)
+    c32 = m.fp8_gemm(a, a_s, b, b_s, out_dtype=torch.float32)
+    assert np.array_equal(c32.cpu().numpy().view(np.uint32), d["c_f32"].view(np.uint32))
+    c16 = m.fp8_gemm(a, a_s, b, b_s, out_dtype=torch.bfloat16)
+    assert np.array_equal(c16.cpu().view(torch.int16).numpy().view(np.uint16), d["c_bf16_bits"])
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 512, 256), (300, 520, 384), (65, 130, 128), (100, 257, 256), (70, 1100, 512),
+                                   (512, 2304, 1024)])
+def test_gemm_exact_integer_cases_all_kernels(M, N, K):
+    """Integer-valued operands, power-of-two scales: every product and sum is exact, so the
+    result must equal the int64 computation bit for bit (catches any indexing mistake:
+    transposed scales, wrong n//128, K-block order, tile edges)."""
+    g = torch.Generator().manual_seed(M + N + K)
+    ai = torch.randint(-4, 5, (M, K), generator=g)
+    bi = torch.randint(-4, 5, (N, K), generator=g)
+    KB, NB = K // 128, (N + 127) // 128
+    ae = torch.randint(-2, 3, (M, KB), generator=g)
+    be = torch.randint(-2, 3, (NB, KB), generator=g)
+    c = torch.zeros(M, N, dtype=torch.float64)
+    for kb in range(KB):
+        part = (ai[:, kb * 128:(kb + 1) * 128].double() @ bi[:, kb * 128:(kb + 1) * 128].double().t())
+        c += part * torch.exp2((ae[:, kb][:, None] + be[torch.arange(N) // 128, kb][None, :]).double())
+    got = m.fp8_gemm(ai.float().to(FP8).to(DEV), torch.exp2(ae.float()).to(DEV), bi.float().to(FP8).to(DEV),
+                     torch.exp2(be.float()).to(DEV), out_dtype=torch.float32)
+    assert torch.equal(got.cpu().double(), c)
+
+
+@pytest.mark.parametrize("M", [1, 5, 16, 17, 33, 64])
+def test_gemm_small_m_exact(M):
+    test_gemm_exact_integer_cases_all_kernels(M, 272, 384)
+
+
+def test_gemm_one_hot_and_scale_block_perturbation():
+    N, K = 512, 512
+    g = torch.Generator().manual_seed(2)
+    b = torch.randint(0, 0x77, (N, K), generator=g, dtype=torch.uint8).view(FP8)
+    b_s = torch.rand(4, 4, generator=g) + 0.5
+    M = 128
+    a = torch.zeros(M, K).to(FP8)
+    hot = torch.randint(0, K, (M,), generator=g)
+    a.view(torch.uint8)[torch.arange(M), hot] = 0x38  # 1.0
+    a_s = torch.rand(M, 4, generator=g) + 0.5
+    c = m.fp8_gemm(a.to(DEV), a_s.to(DEV), b.to(DEV), b_s.to(DEV), out_dtype=torch.float32).cpu()
+    bd = O.weight_dequant(b, b_s, dtype=torch.float32)
+    expect = bd[:, hot].t() * a_s[torch.arange(M), hot // 128][:, None]
+    assert torch.allclose(c, expect, rtol=1e-6, atol=0)
+    b_s2 = b_s.clone(); b_s2[2, 1] *= 4
+    a2 = torch.randint(0, 0x60, (M, K), generator=g, dtype=torch.uint8).view(FP8)
+    a2_s = torch.ones(M, 4)
+    d = (m.fp8_gemm(a2.to(DEV), a2_s.to(DEV), b.to(DEV), b_s2.to(DEV), out_dtype=torch.float32)
+         - m.fp8_gemm(a2.to(DEV), a2_s.to(DEV), b.to(DEV), b_s.to(DEV), out_dtype=torch.float32)).cpu()
+    assert torch.count_nonzero(d[:, :256]) == 0 and torch.count_nonzero(d[:, 384:]) == 0
+    assert torch.count_nonzero(d[:, 256:384]) > 0
+
+
+def test_gemm_c1_cpu_reference_config_full():
+    kind, M, N, K = P.CONFIGS["C1_cpu_reference"]
+    a, a_s, wq, ws = quantized_problem(kind, M, N, K, 0)
+    ref = O.fp8_gemm(a, a_s, wq, ws, dtype=torch.bfloat16)
+    got = m.fp8_gemm(a.to(DEV), a_s.to(DEV), wq.to(DEV), ws.to(DEV), out_dtype=torch.bfloat16)
+    assert got.dtype == torch.bfloat16 and got.shape == (M, N)
+    assert close(got, ref)
+    truth = O.fp8_gemm_f64(a, a_s, wq, ws)
+    assert (got.cpu().double() - truth).abs().max() <= 2 ** -8 * truth.abs().max() + 1e-6
+
+
+@pytest.mark.parametrize("name", ["C2_q_a_proj", "C3_mlp_up_gate", "C4_mlp_down"])
+def test_gemm_full_size_configs_sampled_rows(name):
+    """Full-size GEMM on the device; the oracle is evaluated on a spread of rows (every
+    tile row is hit) with all N columns."""
+    kind, M, N, K = P.CONFIGS[name]
+    a, a_s, wq, ws = quantized_problem(kind, M, N, K, 10)
+    got = m.fp8_gemm(a.to(DEV), a_s.to(DEV), wq.to(DEV), ws.to(DEV), out_dtype=torch.bfloat16)
+    rows = torch.unique(torch.cat([torch.arange(0, M, 61), torch.tensor([0, 127, 128, 255, 256, M - 1])]))
+    ref = O.fp8_gemm(a[rows].contiguous(), a_s[rows].contiguous(), wq, ws, dtype=torch.bfloat16)
+    assert close(got[rows.to(DEV)], ref)
+    # linearity in the activation scales (size-independent property): doubling a_s doubles C exactly
+    got2 = m.fp8_gemm(a.to(DEV), (a_s * 2).to(DEV), wq.to(DEV), ws.to(DEV), out_dtype=torch.bfloat16)
+    assert torch.equal(got2, got * 2)
+
+
+@pytest.mark.parametrize("M,N,K", P.DECODE_SHAPES)
+def test_gemm_decode_shapes(M, N, K):
+    a, a_s, wq, ws = quantized_problem("normal", M, N, K, M)
+    ref = O.fp8_gemm(a, a_s, wq, ws, dtype=torch.bfloat16)
+    got = m.fp8_gemm(a.to(DEV), a_s.to(DEV), wq.to(DEV), ws.to(DEV), out_dtype=torch.bfloat16)
+    assert close(got, ref)
+
+
+@pytest.mark.parametrize("M,N,K", [(7, 5, 100), (33, 130, 200), (3, 3, 1), (64, 64, 130)])
+def test_gemm_ragged_k_scalar_path(M, N, K):
+    """K not a multiple of 128: the tail block is shorter (masked loads at offical_kernel.py:82-83)."""
+    g = torch.Generator().manual_seed(K)
+    a = torch.randint(0, 0x70, (M, K), generator=g, dtype=torch.uint8).view(FP8)
+    b = torch.randint(0, 0x70, (N, K), generator=g, dtype=torch.uint8).view(FP8)
+    KB = (K + 127) // 128
+    a_s = torch.rand(M, KB, generator=g) * 1e-2
+    b_s = torch.rand((N + 127) // 128, KB, generator=g) * 1e-2
+    ref = O.fp8_gemm(a, a_s, b, b_s, dtype=torch.float32)
+    got = m.fp8_gemm(a.to(DEV), a_s.to(DEV), b.to(DEV), b_s.to(DEV), out_dtype=torch.float32)
+    assert torch.allclose(got.cpu(), ref, rtol=1e-4, atol=1e-6)
+
+
+def test_gemm_leading_dims_default_dtype_and_bias():
+    a, a_s, wq, ws = quantized_problem("normal", 96, 384, 256, 5)
+    a3, a3_s = a.reshape(2, 48, 256), a_s.reshape(2, 48, 2)
+    got = m.fp8_gemm(a3.to(DEV), a3_s.to(DEV), wq.to(DEV), ws.to(DEV))
+    assert got.shape == (2, 48, 384) and got.dtype == torch.get_default_dtype()
+    ref = O.fp8_gemm(a3, a3_s, wq, ws, dtype=torch.float32)
+    assert torch.allclose(got.cpu(), ref, rtol=1e-4, atol=1e-5)
+    bias = torch.randn(384).bfloat16()
+    gb = m.fp8_gemm(a.to(DEV), a_s.to(DEV), wq.to(DEV), ws.to(DEV), out_dtype=torch.bfloat16, bias=bias.to(DEV))
+    rb = O.fp8_gemm(a, a_s, wq, ws, dtype=torch.bfloat16, bias=bias)
+    assert close(gb, rb)
+
+
+# ------------------------------------------------------------------ DeepLinear path
+@pytest.mark.parametrize("M,N,K", [(128, 1024, 1024), (64, 2048, 7168), (4, 128, 256), (4096, 1536, 7168)])
+def test_fp8_matmul_column_major_scales(M, N, K):
+    x = P.activations("normal", M, K, 3)
+    w, _, _ = P.weights(N, K, 4)
+    qa, sa, _, _ = m.quant_input(x.to(DEV), True)
+    qb, sb, _, _ = m.quant_weight(w.to(DEV), True)
+    assert sa.stride() == (1, qa.size(0))
+    out = m.fp8_matmul(qa, sa, qb, sb)
+    ra, rsa, _, _ = O.quant_input(x, True)
+    rb, rsb, _, _ = O.quant_weight(w, True)
+    rows = torch.unique(torch.cat([torch.arange(0, M, 37), torch.tensor([M - 1])]))
+    ref = O.fp8_matmul(ra[rows].contiguous(), rsa[rows].contiguous(), rb, rsb)
+    assert out.dtype == torch.bfloat16 and out.shape == (qa.size(0), qb.size(0))
+    assert close(out[rows.to(DEV)], ref)
+    buf = torch.empty_like(out)
+    assert m.fp8_matmul(qa, sa, qb, sb, out=buf).data_ptr() == buf.data_ptr() and torch.equal(buf, out)
+
+
+@pytest.mark.parametrize("bias", [True, False])
+@pytest.mark.parametrize("shape,N", [((2, 64, 512), 256), ((8, 1024), 384), ((1, 4, 7168), 2048)])
+def test_deep_linear_forward(shape, N, bias):
+    g = torch.Generator().manual_seed(sum(shape) + N)
+    K = shape[-1]
+    lin = m.DeepLinear(K, N, bias=bias, dtype=torch.bfloat16)
+    with torch.no_grad():
+        lin.weight.copy_((torch.randn(N, K, generator=g) * 0.02).bfloat16())
+        if bias:
+            lin.bias.copy_(torch.randn(N, generator=g).bfloat16())
+    x = torch.randn(*shape, generator=g).bfloat16()
+    ref = O.deep_linear_forward(x, lin.weight.detach(), lin.bias.detach() if bias else None)
+    lin = lin.to(DEV)
+    with torch.no_grad():
+        out = lin(x.to(DEV))
+        out_again = lin(x.to(DEV))          # second call uses the cached quantized weight
+        lin.cache_weight = False
+        out_nocache = lin(x.to(DEV))
+        lin.fuse_bias = True
+        out_fused = lin(x.to(DEV))
+    assert out.shape == (*shape[:-1], N) and out.dtype == torch.bfloat16
+    assert close(out, ref)
+    assert torch.equal(out, out_again) and torch.equal(out, out_nocache)
+    assert close(out_fused, ref)
+    # sanity band against the unquantized layer (the reference prints ~0.017 mean abs error at d=4096)
+    full = torch.nn.functional.linear(x.float(), lin.weight.detach().float().cpu(),
+                                      lin.bias.detach().float().cpu() if bias else None)
+    assert (out.float().cpu() - full).abs().mean() < 0.05
+
+
+def test_deep_linear_cache_follows_weight_updates():
+    lin = m.DeepLinear(256, 128, bias=False, dtype=torch.bfloat16, device=DEV)
+    x = torch.randn(8, 256, device=DEV).bfloat16()
+    with torch.no_grad():
+        y0 = lin(x)
+        lin.weight.mul_(2)
+        y1 = lin(x)
+    assert torch.allclose(y1.float(), 2 * y0.float(), rtol=2e-2, atol=1e-3) and not torch.equal(y0, y1)

@@ -1,0 +1,260 @@
+"""GPU parity of the quantizers and the dequantizer against the CPU oracle:
+e4m3fn bytes and fp32 scales bit-exact, dequantized bf16 bit-exact."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import mdy_triton_amd as m
+from mdy_triton_amd import _lib
+from oracle import fp8_format as F
+from oracle import oracle as O
+from tests import problems as P
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+FP8 = torch.float8_e4m3fn
+DEV = "cuda:0"
+
+
+def u8(t):
+    return t.contiguous().view(torch.uint8).cpu().numpy()
+
+
+def same_bytes_mod_nan(got, ref):
+    """Bit-exact, except that the two NaN codes (0x7F / 0xFF) compare equal."""
+    nan = (ref & 0x7F) == 0x7F
+    return np.array_equal((got & 0x7F) == 0x7F, nan) and np.array_equal(got[~nan], ref[~nan])
+
+
+def bf16_from_bits(bits):
+    return torch.from_numpy(bits.astype(np.uint16).view(np.int16).copy()).view(torch.bfloat16)
+
+
+# ------------------------------------------------------------------ the cast itself
+def _device_cast(x: np.ndarray, saturate: int) -> np.ndarray:
+    xt = torch.from_numpy(x.copy()).to(DEV)
+    y = torch.empty(x.size, dtype=torch.uint8, device=DEV)
+    _lib.check(_lib.load().mdy_cast_f32_to_e4m3(xt.data_ptr(), y.data_ptr(), x.size, saturate, None), "cast")
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+def test_device_cast_matches_format_definition():
+    tab = F.decode_table()
+    pos = np.sort(tab[:0x7F])
+    mids = ((pos[:-1].astype(np.float64) + pos[1:].astype(np.float64)) / 2).astype(np.float32)
+    pts = np.concatenate([pos, mids, -pos, -mids])
+    pts = np.concatenate([pts, np.nextafter(pts, np.float32(np.inf)), np.nextafter(pts, np.float32(-np.inf))])
+    rng = np.random.default_rng(0)
+    rnd = (rng.standard_normal(1 << 18) * rng.choice([1e-3, 1.0, 100.0, 300.0], size=1 << 18)).astype(np.float32)
+    rnd = rnd[np.abs(rnd) <= 448.0]
+    x = np.concatenate([pts, rnd, np.array([448.00003, -448.00003, 0.0, -0.0, 1e-30, -1e-30], np.float32)])
+    x = x[np.abs(x) < 464.0].astype(np.float32)
+    assert np.array_equal(_device_cast(x, 0), F.encode_rne(x))
+    # saturating flavour over the whole fp32 range, NaN kept
+    big = np.array([464.0, 465.0, 1e4, 3e38, np.inf, -464.0, -1e9, -np.inf, np.nan, 500.0], np.float32)
+    xs = np.concatenate([x, big])
+    assert same_bytes_mod_nan(_device_cast(xs, 1), F.encode_rne_sat(xs))
+
+
+def test_fast_quotient_equals_division_on_device():
+    """Every bf16 amax x every bf16 |x| <= amax, both dialects, on the device's own
+    divider and FMA: the byte (and where the fast path is taken, nothing else) agrees."""
+    out = torch.zeros(4, dtype=torch.int64, device=DEV)
+    for mode in (0, 1):
+        _lib.check(_lib.load().mdy_quotient_selfcheck(out.data_ptr(), 0, 0x7F80, mode, None), "selfcheck")
+        torch.cuda.synchronize()
+        pairs, f32_bad, fp8_bad, plain = out.cpu().tolist()
+        assert pairs == 1065402240
+        assert fp8_bad == 0
+        if mode == 0:
+            assert plain < pairs // 8   # only tiny-amax groups divide plainly
+
+
+# ------------------------------------------------------------------ act_quant (official dialect)
+def test_act_quant_golden_codes():
+    d = np.load(os.path.join(GOLD, "act_quant_codes.npz"))
+    y, s = m.act_quant(bf16_from_bits(d["x_bits"]).to(DEV))
+    assert np.array_equal(u8(y), d["y"])
+    assert np.array_equal(s.cpu().numpy().view(np.uint32), d["s"].view(np.uint32))
+
+
+@pytest.mark.parametrize("kind,M,K,seed", [
+    ("normal", 128, 1024, 0), ("outliers", 4096, 7168, 1), ("normal", 4096, 7168, 2), ("heavy", 4096, 18432, 3),
+    ("normal", 1, 2048, 4), ("normal", 16, 7168, 5), ("normal", 64, 2048, 6), ("normal", 3, 128, 7),
+    ("normal", 37, 640, 8),
+])
+def test_act_quant_bit_exact(kind, M, K, seed):
+    x = P.activations(kind, M, K, seed)
+    y_ref, s_ref = O.act_quant(x)
+    y, s = m.act_quant(x.to(DEV))
+    assert y.dtype == FP8 and y.shape == x.shape and s.shape == (M, K // 128) and s.dtype == torch.float32
+    assert torch.equal(s.cpu(), s_ref)
+    assert np.array_equal(u8(y), u8(y_ref))
+
+
+def test_act_quant_leading_dims_and_empty():
+    x = P.activations("normal", 24, 256, 9).reshape(2, 3, 4, 256)
+    y, s = m.act_quant(x.to(DEV))
+    y_ref, s_ref = O.act_quant(x)
+    assert y.shape == x.shape and s.shape == (2, 3, 4, 2)
+    assert np.array_equal(u8(y), u8(y_ref)) and torch.equal(s.cpu(), s_ref)
+    y0, s0 = m.act_quant(torch.empty(0, 256, dtype=torch.bfloat16, device=DEV))
+    assert y0.shape == (0, 256) and s0.shape == (0, 2)
+
+
+def test_act_quant_edge_values():
+    """Tiny, subnormal, huge, signed-zero, all-zero, inf and NaN groups."""
+    rng = np.random.default_rng(11)
+    rows = []
+    base = rng.standard_normal(128).astype(np.float32)
+    for scale in (1.0, 2.0 ** -100, 2.0 ** -110, 2.0 ** -120, 2.0 ** -126, 2.0 ** -130, 2.0 ** 100, 2.0 ** 120, 3e38 / 4):
+        rows.append(base * np.float32(scale))
+    z = np.zeros(128, np.float32)
+    rows.append(z.copy())                                   # all zero -> s = 0, y = NaN
+    nz = z.copy(); nz[0] = 1.0; nz[1] = -0.0; nz[2] = 2.0 ** -133  # signed zero / flush-to-zero quotient
+    rows.append(nz)
+    inf = base.copy(); inf[5] = np.inf; inf[6] = -np.inf
+    rows.append(inf)
+    x = torch.from_numpy(np.stack(rows)).bfloat16()
+    y_ref, s_ref = O.act_quant(x)
+    y, s = m.act_quant(x.to(DEV))
+    sr, sg = s_ref.numpy(), s.cpu().numpy()
+    assert np.array_equal(np.isnan(sr), np.isnan(sg))
+    assert np.array_equal(sr[~np.isnan(sr)].view(np.uint32), sg[~np.isnan(sg)].view(np.uint32))
+    assert same_bytes_mod_nan(u8(y), u8(y_ref))
+    assert np.all((u8(y)[9] & 0x7F) == 0x7F)
+    assert u8(y)[10][1] == 0x80
+
+
+def test_act_quant_nan_is_ignored_by_the_group_max():
+    """A NaN element stays NaN; the rest of its group is quantized with the max of the
+    finite values (the hardware max ignores NaN, as the reference's tl.max does)."""
+    x = P.activations("normal", 2, 256, 12)
+    x[0, 7] = float("nan")
+    y, s = m.act_quant(x.to(DEV))
+    xz = x.clone(); xz[0, 7] = 0.0
+    y_ref, s_ref = O.act_quant(xz)
+    assert torch.equal(s.cpu(), s_ref)
+    got, ref = u8(y), u8(y_ref)
+    assert (got[0, 7] & 0x7F) == 0x7F
+    got[0, 7] = ref[0, 7]
+    assert np.array_equal(got, ref)
+
+
+# ------------------------------------------------------------------ quant_input (DeepLinear dialect)
+@pytest.mark.parametrize("M,K,seed", [(128, 1024, 0), (4096, 7168, 1), (1, 2048, 2), (6, 300, 3), (37, 641, 4),
+                                      (64, 7168, 5), (255, 384, 6)])
+def test_quant_input_bit_exact(M, K, seed):
+    x = P.activations("outliers", M, K, seed)
+    y_ref, s_ref, _, _ = O.quant_input(x, True)
+    y, s, y_t, s_t = m.quant_input(x.to(DEV), True)
+    assert y_t is None and s_t is None
+    assert y.shape == y_ref.shape and s.shape == s_ref.shape and s.stride() == s_ref.stride()
+    assert torch.equal(s.cpu(), s_ref)
+    assert np.array_equal(u8(y), u8(y_ref))
+
+
+def test_quant_input_strided_rows_and_saturation():
+    big = P.activations("normal", 40, 1024, 7)
+    x = big[:, 128:128 + 512]                      # row stride 1024, column stride 1, offset 256 bytes
+    x[0, 0] = 3e4; x[0, 1] = -2e4; x[1, 3] = 1.5e4
+    y_ref, s_ref, _, _ = O.quant_input(x, True)
+    y, s, _, _ = m.quant_input(big.to(DEV)[:, 128:128 + 512], True)
+    assert torch.equal(s.cpu(), s_ref) and np.array_equal(u8(y), u8(y_ref))
+    xt = big.t()                                   # column stride != 1
+    y_ref, s_ref, _, _ = O.quant_input(xt, True)
+    y, s, _, _ = m.quant_input(big.to(DEV).t(), True)
+    assert torch.equal(s.cpu(), s_ref) and np.array_equal(u8(y), u8(y_ref))
+
+
+# ------------------------------------------------------------------ quant_weight
+@pytest.mark.parametrize("N,K,only_forward,seed", [(1024, 1024, True, 0), (1536, 7168, True, 1), (200, 300, True, 2),
+                                                   (200, 300, False, 3), (512, 256, False, 4), (129, 257, False, 5)])
+def test_quant_weight_bit_exact(N, K, only_forward, seed):
+    w, _, _ = P.weights(N, K, seed)
+    ref = O.quant_weight(w, only_forward)
+    got = m.quant_weight(w.to(DEV), only_forward)
+    for r, g in zip(ref, got):
+        if r is None:
+            assert g is None
+            continue
+        assert g.shape == r.shape
+        if r.dtype == FP8:
+            assert np.array_equal(u8(g), u8(r))
+        else:
+            assert torch.equal(g.cpu(), r)
+
+
+def test_quant_weight_transposed_view_input():
+    w, _, _ = P.weights(256, 384, 6)
+    ref = O.quant_weight(w.t(), True)
+    got = m.quant_weight(w.to(DEV).t(), True)
+    assert np.array_equal(u8(got[0]), u8(ref[0])) and torch.equal(got[1].cpu(), ref[1])
+
+
+# ------------------------------------------------------------------ weight_dequant
+def test_weight_dequant_golden_codes():
+    d = np.load(os.path.join(GOLD, "weight_dequant_codes.npz"))
+    x = torch.from_numpy(d["x"]).view(FP8).to(DEV)
+    y = m.weight_dequant(x, torch.from_numpy(d["s"]).to(DEV), out_dtype=torch.bfloat16)
+    got = y.cpu().view(torch.int16).numpy().view(np.uint16)
+    fin = d["finite"]
+    assert np.array_equal(got[:, fin], d["y_bits"][:, fin])
+    assert torch.isnan(y.cpu()[:, ~torch.from_numpy(fin)].float()).all()
+
+
+@pytest.mark.parametrize("N,K,seed", [(1024, 1024, 0), (1536, 7168, 1), (18432, 7168, 2), (7168, 18432, 3),
+                                      (7168, 2048, 4), (2048, 7168, 5), (200, 300, 6), (1, 128, 7), (130, 1000, 8)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_weight_dequant_bit_exact(N, K, seed, dtype):
+    if dtype == torch.float32 and N * K > 20_000_000:
+        pytest.skip("fp32 flavour is covered at the smaller shapes")
+    g = torch.Generator().manual_seed(seed)
+    codes = torch.randint(0, 256, (N, K), generator=g, dtype=torch.uint8)
+    codes[(codes & 0x7F) == 0x7F] = 0x3A
+    s = torch.rand((N + 127) // 128, (K + 127) // 128, generator=g) * 3e-3 + 1e-5
+    ref = O.weight_dequant(codes.view(FP8), s, dtype=dtype)
+    got = m.weight_dequant(codes.view(FP8).to(DEV), s.to(DEV), out_dtype=dtype)
+    assert got.dtype == dtype and got.shape == (N, K)
+    assert torch.equal(got.cpu().view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
+                       ref.view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
+
+
+def test_weight_dequant_honours_default_dtype():
+    codes = torch.randint(0, 120, (128, 256), dtype=torch.uint8).view(FP8).to(DEV)
+    s = torch.ones(1, 2, device=DEV)
+    old = torch.get_default_dtype()
+    try:
+        torch.set_default_dtype(torch.bfloat16)
+        assert m.weight_dequant(codes, s).dtype == torch.bfloat16
+    finally:
+        torch.set_default_dtype(old)
+    assert m.weight_dequant(codes, s).dtype == torch.float32
+
+
+def test_quantize_then_dequantize_round_trip_bound():
+    """Size-independent property at the full C3 weight shape: |dequant(quant(w)) - w| <= half an
+    e4m3 ulp of the block maximum's grid, i.e. <= s * 16 (= 2**4, half of the top binade's step 32)."""
+    w, _, _ = P.weights(2048, 7168, 10)
+    wd = w.to(DEV)
+    q, s, _, _ = m.quant_weight(wd, True)
+    back = m.weight_dequant(q, s, out_dtype=torch.float32)
+    sfull = s.repeat_interleave(128, 0).repeat_interleave(128, 1)
+    assert torch.all((back - wd.float()).abs() <= sfull * 16.0 * (1 + 1e-6))
+
+
+# ------------------------------------------------------------------ add_bias
+@pytest.mark.parametrize("M,N", [(128, 1024), (5, 18432), (7, 100), (1, 7)])
+def test_add_bias_bit_exact(M, N):
+    g = torch.Generator().manual_seed(M * 31 + N)
+    x = torch.randn(M, N, generator=g).bfloat16()
+    b = torch.randn(N, generator=g).bfloat16()
+    ref = O.add_bias(x, b)
+    xd = x.to(DEV)
+    out = m.add_bias(xd, b.to(DEV))
+    assert out.data_ptr() == xd.data_ptr()
+    assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))

@@ -1,0 +1,250 @@
+"""Pins the CPU oracle (oracle/oracle.py) from outside its own formulas: golden
+fixtures derived from the format definition, numpy re-derivations, invariants,
+float64 truth and exactly-representable GEMM cases."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import fp8_format as F
+from oracle import oracle as O
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+FP8 = torch.float8_e4m3fn
+
+
+def bf16_from_bits(bits: np.ndarray) -> torch.Tensor:
+    return torch.from_numpy(bits.astype(np.uint16).view(np.int16).copy()).view(torch.bfloat16)
+
+
+def u8(t: torch.Tensor) -> np.ndarray:
+    return t.contiguous().view(torch.uint8).numpy()
+
+
+# ------------------------------------------------------------------ act_quant
+def test_act_quant_golden_codes():
+    d = np.load(os.path.join(GOLD, "act_quant_codes.npz"))
+    x = bf16_from_bits(d["x_bits"])
+    y, s = O.act_quant(x)
+    assert np.array_equal(u8(y), d["y"])
+    assert np.array_equal(s.numpy().view(np.uint32), d["s"].view(np.uint32))
+
+
+def test_act_quant_numpy_rederivation_and_invariants():
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(64, 1024, generator=g).bfloat16()
+    x[3, 5] *= 50  # an outlier group
+    y, s = O.act_quant(x)
+    xf = F.bf16_bits_to_f32(x.view(torch.int16).numpy().view(np.uint16)).reshape(-1, 128)
+    amax = np.abs(xf).max(axis=1)
+    s_np = (amax / np.float32(448.0)).astype(np.float32)
+    assert np.array_equal(s.numpy().reshape(-1).view(np.uint32), s_np.view(np.uint32))
+    y_np = F.encode_rne((xf / s_np[:, None]).astype(np.float32))
+    assert np.array_equal(u8(y).reshape(-1, 128), y_np)
+    # the absmax element encodes to +-448
+    assert np.all((y_np & 0x7F).max(axis=1) == 0x7E)
+    # reconstruction error at most half an e4m3 ulp of the quotient (8 ulps of 2**-3 relative, or the subnormal step)
+    q = xf / s_np[:, None]
+    deq = F.decode(y_np)
+    ulp = np.maximum(2.0 ** (np.floor(np.log2(np.maximum(np.abs(q), 2.0 ** -6))) - 3), 2.0 ** -9)
+    assert np.all(np.abs(deq - q) <= ulp / 2 * (1 + 1e-6))
+
+
+def test_act_quant_idempotent_on_its_own_output():
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(16, 256, generator=g).bfloat16()
+    y, s = O.act_quant(x)
+    # use power-of-two scales so that the dequantized tensor is exact in bf16
+    s2 = torch.exp2(torch.floor(torch.log2(s)))
+    xd = (y.float().reshape(16, 2, 128) * s2[:, :, None]).reshape(16, 256)
+    y[:, 0] = torch.tensor(448.0).to(FP8)  # make sure the absmax is 448 in group 0 of every row
+    y[:, 128] = torch.tensor(-448.0).to(FP8)
+    xd = (y.float().reshape(16, 2, 128) * s2[:, :, None]).reshape(16, 256).bfloat16()
+    y2, s3 = O.act_quant(xd)
+    assert torch.equal(s3, s2)
+    assert np.array_equal(u8(y2), u8(y))
+
+
+def test_act_quant_zero_group_is_nan_and_negative_zero_keeps_sign():
+    x = torch.zeros(1, 256, dtype=torch.bfloat16)
+    x[0, 128] = 1.0
+    x[0, 129] = -0.0
+    y, s = O.act_quant(x)
+    b = u8(y)[0]
+    assert s[0, 0] == 0 and np.all((b[:128] & 0x7F) == 0x7F)
+    assert b[128] == 0x7E and b[129] == 0x80 and b[130] == 0x00
+
+
+# ------------------------------------------------------------------ weight_dequant
+def test_weight_dequant_golden_codes():
+    d = np.load(os.path.join(GOLD, "weight_dequant_codes.npz"))
+    x = torch.from_numpy(d["x"]).view(FP8)
+    y = O.weight_dequant(x, torch.from_numpy(d["s"]), dtype=torch.bfloat16)
+    got = y.view(torch.int16).numpy().view(np.uint16)
+    fin = d["finite"]
+    assert np.array_equal(got[:, fin], d["y_bits"][:, fin])
+    assert torch.isnan(y[:, ~torch.from_numpy(fin)].float()).all()
+
+
+def test_weight_dequant_numpy_rederivation_ragged():
+    rng = np.random.default_rng(5)
+    N, K = 200, 300
+    codes = rng.integers(0, 256, size=(N, K), dtype=np.uint8)
+    codes[(codes & 0x7F) == 0x7F] = 0x3C
+    s = rng.uniform(1e-4, 3e-3, size=(2, 3)).astype(np.float32)
+    y = O.weight_dequant(torch.from_numpy(codes).view(FP8), torch.from_numpy(s), dtype=torch.bfloat16)
+    sfull = np.repeat(np.repeat(s, 128, 0)[:N], 128, 1)[:, :K]
+    prod = (F.decode(codes) * sfull).astype(np.float32)
+    assert np.array_equal(y.view(torch.int16).numpy().view(np.uint16), F.f32_to_bf16_bits_rne(prod))
+    y32 = O.weight_dequant(torch.from_numpy(codes).view(FP8), torch.from_numpy(s), dtype=torch.float32)
+    assert np.array_equal(y32.numpy().view(np.uint32), prod.view(np.uint32))
+
+
+# ------------------------------------------------------------------ fp8_gemm
+def _rand_problem(M, N, K, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) * 0.02).bfloat16()
+    a, a_s = O.act_quant(x)
+    Np = (N + 127) // 128 * 128
+    wp = torch.zeros(Np, K, dtype=torch.bfloat16)
+    wp[:N] = w
+    wp[N:] = 0.01
+    b, b_s = O.weight_quant_block(wp)
+    return x, w, a, a_s, b[:N].contiguous(), b_s
+
+
+def test_fp8_gemm_golden_exact():
+    d = np.load(os.path.join(GOLD, "gemm_exact.npz"))
+    a = torch.from_numpy(d["a"]).view(FP8)
+    b = torch.from_numpy(d["b"]).view(FP8)
+    a_s, b_s = torch.from_numpy(d["a_s"]), torch.from_numpy(d["b_s"])
+    for fn in (O.fp8_gemm, O.fp8_gemm_blockwise):
+        c32 = fn(a, a_s, b, b_s, dtype=torch.float32)
+        assert np.array_equal(c32.numpy().view(np.uint32), d["c_f32"].view(np.uint32))
+        c16 = fn(a, a_s, b, b_s, dtype=torch.bfloat16)
+        assert np.array_equal(c16.view(torch.int16).numpy().view(np.uint16), d["c_bf16_bits"])
+    assert np.array_equal(O.fp8_gemm_f64(a, a_s, b, b_s).numpy(), d["c_f32"].astype(np.float64))
+
+
+def test_fp8_gemm_against_float64_and_blockwise():
+    x, w, a, a_s, b, b_s = _rand_problem(48, 200, 512, 11)
+    truth = O.fp8_gemm_f64(a, a_s, b, b_s)
+    c = O.fp8_gemm(a, a_s, b, b_s, dtype=torch.float32).double()
+    cb = O.fp8_gemm_blockwise(a, a_s, b, b_s, dtype=torch.float32).double()
+    scale = truth.abs().max()
+    assert (c - truth).abs().max() <= 1e-5 * scale
+    assert (cb - truth).abs().max() <= 1e-5 * scale
+    # and it approximates the unquantized product at the level the reference reports
+    ref = x.float() @ w.float().t()
+    assert (c.float() - ref).abs().mean() < 0.05 * ref.abs().mean() + 1e-3
+
+
+def test_fp8_gemm_one_hot_rows_and_single_scale_block():
+    N, K = 256, 256
+    g = torch.Generator().manual_seed(2)
+    b = torch.randint(0, 0x77, (N, K), generator=g, dtype=torch.uint8).view(FP8)
+    b_s = torch.tensor([[1.0, 0.5], [0.25, 2.0]])
+    a = torch.zeros(4, K).to(FP8)
+    hot = [3, 127, 128, 255]
+    for r, k in enumerate(hot):
+        a[r, k] = torch.tensor(1.0).to(FP8)
+    a_s = torch.tensor([[1.0, 1.0], [2.0, 1.0], [1.0, 4.0], [1.0, 0.5]])
+    c = O.fp8_gemm(a, a_s, b, b_s, dtype=torch.float32)
+    bd = O.weight_dequant(b, b_s, dtype=torch.float32)
+    for r, k in enumerate(hot):
+        assert torch.equal(c[r], bd[:, k] * a_s[r, k // 128])
+    # perturbing one (n-block, k-block) weight scale changes only that output stripe
+    b_s2 = b_s.clone()
+    b_s2[1, 0] = 8.0
+    a2 = torch.randint(0, 0x60, (8, K), generator=g, dtype=torch.uint8).view(FP8)
+    a2_s = torch.ones(8, 2)
+    d = O.fp8_gemm(a2, a2_s, b, b_s2, dtype=torch.float32) - O.fp8_gemm(a2, a2_s, b, b_s, dtype=torch.float32)
+    assert torch.count_nonzero(d[:, :128]) == 0 and torch.count_nonzero(d[:, 128:]) > 0
+
+
+# ------------------------------------------------------------------ DeepLinear dialect
+def test_quant_input_layout_padding_and_eps():
+    g = torch.Generator().manual_seed(4)
+    M, K = 6, 300
+    x = torch.randn(M, K, generator=g).bfloat16()
+    y, s, y_t, s_t = O.quant_input(x, True)
+    assert y_t is None and s_t is None
+    assert tuple(y.shape) == (8, 512) and tuple(s.shape) == (8, 4) and s.stride() == (1, 8)
+    yb = u8(y)
+    assert np.all(yb[M:] == 0) and np.all(yb[:, 384:] == 0) and np.all(yb[:M, K:384] == 0)
+    eps_scale = (np.float32(1e-8) / np.float32(448)).astype(np.float32)
+    assert np.all(s.numpy()[M:] == eps_scale) and np.all(s.numpy()[:, 3] == eps_scale)
+    xf = x.float().numpy()
+    amax = np.abs(xf[:, :128]).max(axis=1)
+    s_np = ((np.minimum(amax, np.float32(1e4)) + np.float32(1e-8)) / np.float32(448)).astype(np.float32)
+    assert np.array_equal(s.numpy()[:M, 0].view(np.uint32), s_np.view(np.uint32))
+    assert np.array_equal(yb[:M, :128], F.encode_rne_sat((xf[:, :128] / s_np[:, None]).astype(np.float32)))
+
+
+def test_quant_input_saturates_beyond_clamp():
+    x = torch.zeros(4, 256, dtype=torch.bfloat16)
+    x[0, 0] = 3e4
+    x[0, 1] = -2e4
+    x[0, 2] = 5e3
+    y, s, _, _ = O.quant_input(x, True)
+    b = u8(y)[0]
+    assert b[0] == 0x7E and b[1] == 0xFE
+    sc = (np.float32(1e4) + np.float32(1e-8)) / np.float32(448)
+    assert s[0, 0].item() == sc
+    assert b[2] == F.encode_rne(np.array([np.float32(5e3) / sc], np.float32))[0]
+
+
+def test_quant_weight_blocks_padding_transpose():
+    g = torch.Generator().manual_seed(6)
+    N, K = 200, 300
+    w = (torch.randn(N, K, generator=g) * 0.02).bfloat16()
+    y, s, y_t, s_t = O.quant_weight(w, False)
+    assert tuple(y.shape) == (256, 512) and tuple(s.shape) == (2, 4)
+    assert tuple(y_t.shape) == (512, 256) and tuple(s_t.shape) == (4, 2)
+    assert torch.equal(y_t.view(torch.uint8), y.view(torch.uint8).t()) and torch.equal(s_t, s.t())
+    y1, s1, _, _ = O.quant_weight(w, True)
+    assert tuple(y1.shape) == (256, 512)
+    wf = w.float().numpy()
+    blk = wf[128:200, 256:300]
+    amax = np.abs(blk).max()
+    sc = ((np.float32(amax) + np.float32(1e-8)) / np.float32(448)).astype(np.float32)
+    assert s1[1, 2].item() == sc
+    assert sc != np.float32(amax) / np.float32(448)  # the eps is not a no-op at this magnitude
+    assert np.array_equal(u8(y1)[128:200, 256:300], F.encode_rne_sat((blk / sc).astype(np.float32)))
+    assert np.all(u8(y1)[200:] == 0)
+
+
+def test_weight_quant_block_matches_act_quant_on_uniform_rows():
+    # a 128x128 block whose rows all share the same absmax quantizes like 128 act_quant groups
+    g = torch.Generator().manual_seed(8)
+    w = torch.randn(128, 128, generator=g).bfloat16()
+    w[:, 0] = 7.0
+    w = w.clamp(-7, 7)
+    yb, sb = O.weight_quant_block(w)
+    ya, sa = O.act_quant(w)
+    assert torch.equal(sa, sb.expand(128, 1)) and np.array_equal(u8(ya), u8(yb))
+
+
+def test_quant_grad_output_is_row_and_column_quant():
+    g = torch.Generator().manual_seed(9)
+    dy = torch.randn(256, 256, generator=g).bfloat16()
+    y, s, y_t, s_t = O.quant_grad_output(dy)
+    y_r, s_r, _, _ = O.quant_input(dy, True)
+    assert np.array_equal(u8(y), u8(y_r)) and torch.equal(s.contiguous(), s_r.contiguous())
+    y_c, s_c, _, _ = O.quant_input(dy.t().contiguous(), True)
+    assert np.array_equal(u8(y_t), u8(y_c)) and torch.equal(s_t.contiguous(), s_c.contiguous())
+
+
+def test_add_bias_and_deep_linear_composition():
+    g = torch.Generator().manual_seed(10)
+    x = torch.randn(2, 4, 256, generator=g).bfloat16()
+    w = (torch.randn(128, 256, generator=g) * 0.05).bfloat16()
+    bias = torch.randn(128, generator=g).bfloat16()
+    out = O.deep_linear_forward(x, w, bias)
+    assert tuple(out.shape) == (2, 4, 128) and out.dtype == torch.bfloat16
+    ref = torch.nn.functional.linear(x.float(), w.float(), bias.float())
+    assert (out.float() - ref).abs().mean() < 0.03
+    nb = O.deep_linear_forward(x, w, None)
+    assert torch.equal(out, O.add_bias(nb, bias))
