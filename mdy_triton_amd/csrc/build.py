@@ -17,6 +17,8 @@ LIB = os.path.join(HERE, "libmdyfp8.so")
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA results go to plain VGPRs: the GEMM folds them with v_fma_f32, which cannot read AGPRs
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
     "-Wno-unused-command-line-argument",
 ]
 

@@ -7,18 +7,24 @@
 //
 // Main kernel (K % 128 == 0):
 //   * one workgroup owns a BM x BN tile of C; per 128-wide K block the A and B
-//     panels (BM x 128 and BN x 128 bytes) are staged in LDS, double buffered;
+//     panels (BM x 128 and BN x 128 bytes) and the BM activation scales are
+//     copied global -> LDS by `buffer_load ... lds` (no registers involved),
+//     double buffered, one barrier per K block.  The buffer descriptors cover
+//     exactly the rows of the tile, so rows past M or N read as zero;
 //   * LDS rows are 128 bytes; the eight 16-byte chunks of a row are XOR-swizzled
-//     with (row & 7) ^ (row>>3 & 1) so that both the 16-byte staging writes and the
-//     ds_read_b128 fragment reads are bank-conflict free;
+//     with (row & 7) ^ (row>>3 & 1): each DMA lane fetches the permuted chunk,
+//     the ds_read_b128 fragment reads are bank-conflict free;
 //   * v_mfma_f32_16x16x128_f8f6f4 consumes a whole 128-deep scale block per
 //     instruction.  The B rows go in as the MFMA "A" operand and the A rows as
 //     its "B" operand, so a lane ends up with 4 consecutive n of one m: the
 //     per-block scale a_s[m,kb]*b_s[n/128,kb] is ONE value per lane and
 //     sub-tile, and the epilogue stores 8 contiguous bytes per lane;
-//   * each MFMA starts from C = 0; its 4 results are folded into the fp32 master
-//     accumulator with v_fma_f32 (the promotion the reference does on its
-//     CUDA cores at offical_kernel.py:86);
+//   * each MFMA starts from C = 0 and writes plain VGPRs; its 4 results are folded
+//     into the fp32 master accumulator with v_fma_f32 a few MFMAs later (the
+//     promotion the reference does at offical_kernel.py:86), so the VALU work
+//     runs in the shadow of the matrix pipe;
+//   * the smaller fragment set of the wave tile is held in registers for the
+//     whole K block, the other one is streamed through a two-deep register queue;
 //   * workgroup ids are remapped so that the 32 workgroups that share an XCD's L2
 //     cover a compact 4 x 8 block of tiles.
 // Small-M kernel (M <= 64): weight streaming, one workgroup per 16 columns, waves
@@ -53,38 +59,63 @@ __device__ __forceinline__ void store4(OUT* c, int64_t ldc, int m, int n, int M,
     }
 }
 
+// raw buffer descriptor: base, byte range, no stride, no swizzle
+__device__ __forceinline__ intx4 make_rsrc(const void* base, uint32_t bytes) {
+    const uint64_t p = reinterpret_cast<uint64_t>(base);
+    intx4 r;
+    r[0] = (int)(uint32_t)p;
+    r[1] = (int)((uint32_t)(p >> 32) & 0xFFFFu);
+    r[2] = (int)bytes;
+    r[3] = 0x00020000;
+    return r;
+}
+__device__ __forceinline__ uint32_t lds_addr(const void* p) {
+    return (uint32_t)(uintptr_t)((__attribute__((address_space(3))) const void*)p);
+}
+// 64 lanes x 16 bytes, global (descriptor base + voff + soff) -> LDS (lds + lane*16).
+// Issued as inline asm so that the copy stays asynchronous: the kernel waits for it
+// with an explicit vmcnt(0) + barrier at the end of the K block, nowhere else.
+// rsrc, soff and lds must be wave-uniform.
+__device__ __forceinline__ void dma16(const intx4& rsrc, int voff, int soff, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
+                 :: "v"(voff), "s"(rsrc), "s"(soff), "s"(lds) : "memory");
+}
+__device__ __forceinline__ void dma4(const intx4& rsrc, int voff, int soff, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dword %0, %1, %2 offen lds"
+                 :: "v"(voff), "s"(rsrc), "s"(soff), "s"(lds) : "memory");
+}
+
 // BM x BN block tile, WGM x WGN waves, each wave (BM/WGM) x (BN/WGN).
+// as_bytes = byte size of the addressed part of a_s (host computed, < 2^31).
 template <int BM, int BN, int WGM, int WGN, typename OUT>
 __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
-    const uint8_t* __restrict__ a, const float* __restrict__ a_s, int64_t as_rs, int64_t as_cs,
+    const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
     const uint16_t* __restrict__ bias, int M, int N, int K, int tiles_m, int tiles_n) {
-    constexpr int T = WGM * WGN * 64;
-    constexpr int WM = BM / WGM, WN = BN / WGN;
-    constexpr int TI = WM / 16, TJ = WN / 16;
-    constexpr int A_CHUNKS = BM * 8 / T, B_CHUNKS = BN * 8 / T;
-    static_assert(BM * 8 % T == 0 && BN * 8 % T == 0, "tile/threads mismatch");
-    static_assert(WN % 16 == 0 && WM % 16 == 0, "wave tile must be a multiple of 16");
+    constexpr int WAVES = WGM * WGN;
+    constexpr int WM = BM / WGM, WN = BN / WGN, TI = WM / 16, TJ = WN / 16;
+    constexpr int PASS_ROWS = WAVES * 8;  // rows copied by one DMA instruction of every wave
+    constexpr int A_PASSES = BM / PASS_ROWS, B_PASSES = BN / PASS_ROWS;
+    constexpr int S_WAVES = BM / 64;      // waves that also copy the activation scales
+    constexpr int DEPTH = 4;              // MFMAs in flight before their results are folded
+    static_assert(BM % PASS_ROWS == 0 && BN % PASS_ROWS == 0 && PASS_ROWS % 16 == 0, "tile/threads mismatch");
+    static_assert(WN <= 128 && 128 % WN == 0 && S_WAVES <= WAVES, "one weight-scale block per wave column");
+    constexpr bool HOLD_A = TI <= TJ;
+    constexpr int NH = HOLD_A ? TI : TJ, NS = HOLD_A ? TJ : TI;
 
-    __shared__ __attribute__((aligned(16))) uint8_t lds_a[2][BM * 128];
-    __shared__ __attribute__((aligned(16))) uint8_t lds_b[2][BN * 128];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a[2][BM * 128];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_b[2][BN * 128];
+    __shared__ __attribute__((aligned(256))) float lds_s[2][BM];
 
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
+    const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WGN, wn = wave % WGN;
 
-    // ---- XCD-aware tile order: consecutive ids land on different XCDs (8 of them);
-    // give each XCD a contiguous run of tiles, walked in groups of 4 tile rows.
+    // ---- XCD-aware tile order: consecutive workgroup ids land on different XCDs (8 of
+    // them); give each XCD a contiguous run of tiles, walked in groups of 4 tile rows.
     int pid = blockIdx.x;
     const int ntiles = tiles_m * tiles_n;
-    {
-        const int per_xcd = (ntiles + 7) / 8;
-        const int xcd = pid & 7, local = pid >> 3;
-        int t = xcd * per_xcd + local;
-        if (ntiles % 8 != 0) t = pid;  // irregular counts: keep the plain order
-        pid = t;
-    }
+    if (ntiles % 8 == 0) pid = (pid & 7) * (ntiles >> 3) + (pid >> 3);
     constexpr int GM = 4;
     const int group = pid / (GM * tiles_n);
     const int first_m = group * GM;
@@ -92,57 +123,37 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
     const int tm = first_m + (pid % (GM * tiles_n)) % gsz;
     const int tn = (pid % (GM * tiles_n)) / gsz;
     const int m0 = tm * BM, n0 = tn * BN;
-
     const int KB = K >> 7;
 
-    // ---- staging: thread -> (row, chunk) of the panels
-    const uint8_t* a_src[A_CHUNKS];
-    int a_dst[A_CHUNKS];
-#pragma unroll
-    for (int i = 0; i < A_CHUNKS; ++i) {
-        const int q = tid + T * i, row = q >> 3, ch = q & 7;
-        const int gr = min(m0 + row, M - 1);
-        a_src[i] = a + (int64_t)gr * K + ch * 16;
-        a_dst[i] = row * 128 + ((ch ^ swz(row)) << 4);
-    }
-    const uint8_t* b_src[B_CHUNKS];
-    int b_dst[B_CHUNKS];
-#pragma unroll
-    for (int i = 0; i < B_CHUNKS; ++i) {
-        const int q = tid + T * i, row = q >> 3, ch = q & 7;
-        const int gr = min(n0 + row, N - 1);
-        b_src[i] = b + (int64_t)gr * K + ch * 16;
-        b_dst[i] = row * 128 + ((ch ^ swz(row)) << 4);
-    }
+    // ---- DMA: descriptors limited to the rows of this tile, so that the M and N tails read 0
+    const intx4 ra = make_rsrc(a + (size_t)m0 * K, (uint32_t)min(BM, M - m0) * (uint32_t)K);
+    const intx4 rb = make_rsrc(b + (size_t)n0 * K, (uint32_t)min(BN, N - n0) * (uint32_t)K);
+    const intx4 rs = make_rsrc(a_s, as_bytes);
+    const int prow = wave * 8 + (lane >> 3);                          // row inside a pass
+    const int voff = prow * K + (((lane & 7) ^ swz(prow)) << 4);      // permuted chunk of that row
+    const int s_voff = min(m0 + wave * 64 + lane, M - 1) * as_rs * 4;
+    const uint32_t la_base = lds_addr(&lds_a[0][0]) + wave * 1024;
+    const uint32_t lb_base = lds_addr(&lds_b[0][0]) + wave * 1024;
+    const uint32_t ls_base = lds_addr(&lds_s[0][0]) + wave * 256;
 
-    // ---- fragment read offsets: lane -> row (lane%16) and the 32-byte K slice (lane/16)
+    auto dma_tile = [&](int kb, int buf) {
+        if (wave < S_WAVES) dma4(rs, s_voff, kb * as_cs * 4, ls_base + buf * (BM * 4));
+#pragma unroll
+        for (int i = 0; i < A_PASSES; ++i)
+            dma16(ra, voff, i * PASS_ROWS * K + kb * 128, la_base + buf * (BM * 128) + i * PASS_ROWS * 128);
+#pragma unroll
+        for (int i = 0; i < B_PASSES; ++i)
+            dma16(rb, voff, i * PASS_ROWS * K + kb * 128, lb_base + buf * (BN * 128) + i * PASS_ROWS * 128);
+    };
+
+    // ---- fragment reads: lane -> row (lane%16) and the 32-byte K slice (lane/16) of a 16-row sub-tile
     const int frow = lane & 15, fk = lane >> 4;
-    int a_off[TI][2], b_off[TJ][2];
-#pragma unroll
-    for (int i = 0; i < TI; ++i) {
-        const int row = wm * WM + i * 16 + frow;
-        a_off[i][0] = row * 128 + (((2 * fk) ^ swz(row)) << 4);
-        a_off[i][1] = row * 128 + (((2 * fk + 1) ^ swz(row)) << 4);
-    }
-#pragma unroll
-    for (int j = 0; j < TJ; ++j) {
-        const int row = wn * WN + j * 16 + frow;
-        b_off[j][0] = row * 128 + (((2 * fk) ^ swz(row)) << 4);
-        b_off[j][1] = row * 128 + (((2 * fk + 1) ^ swz(row)) << 4);
-    }
-
-    // ---- scales: this lane's m for sub-tile i is m0 + wm*WM + 16*i + lane%16
-    const float* as_ptr[TI];
-#pragma unroll
-    for (int i = 0; i < TI; ++i) {
-        const int m = min(m0 + wm * WM + i * 16 + frow, M - 1);
-        as_ptr[i] = a_s + (int64_t)m * as_rs;
-    }
-    const int sKB = KB;  // row stride of b_s
-    // sub-tile j covers n0 + wn*WN + 16*j .. +15, inside one 128-block
-    int bs_row[TJ];
-#pragma unroll
-    for (int j = 0; j < TJ; ++j) bs_row[j] = min(n0 + wn * WN + 16 * j, N - 1) >> 7;
+    const int a_rd0 = (wm * WM + frow) * 128 + (((2 * fk) ^ swz(frow)) << 4);
+    const int a_rd1 = (wm * WM + frow) * 128 + (((2 * fk + 1) ^ swz(frow)) << 4);
+    const int b_rd0 = (wn * WN + frow) * 128 + (((2 * fk) ^ swz(frow)) << 4);
+    const int b_rd1 = (wn * WN + frow) * 128 + (((2 * fk + 1) ^ swz(frow)) << 4);
+    const int s_rd = wm * WM + frow;
+    const float* bs_row = b_s + (size_t)(min(n0 + wn * WN, N - 1) >> 7) * KB;
 
     floatx4 acc[TI][TJ];
 #pragma unroll
@@ -150,66 +161,60 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
 #pragma unroll
         for (int j = 0; j < TJ; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    // ---- prologue: stage K block 0
-    intx4 ra[A_CHUNKS], rb[B_CHUNKS];
-#pragma unroll
-    for (int i = 0; i < A_CHUNKS; ++i) ra[i] = *reinterpret_cast<const intx4*>(a_src[i]);
-#pragma unroll
-    for (int i = 0; i < B_CHUNKS; ++i) rb[i] = *reinterpret_cast<const intx4*>(b_src[i]);
-#pragma unroll
-    for (int i = 0; i < A_CHUNKS; ++i) *reinterpret_cast<intx4*>(&lds_a[0][a_dst[i]]) = ra[i];
-#pragma unroll
-    for (int i = 0; i < B_CHUNKS; ++i) *reinterpret_cast<intx4*>(&lds_b[0][b_dst[i]]) = rb[i];
+    auto read_frag = [&](const uint8_t* base, int rd0, int rd1, int idx) {
+        const intx4 lo = *reinterpret_cast<const intx4*>(base + rd0 + idx * 2048);
+        const intx4 hi = *reinterpret_cast<const intx4*>(base + rd1 + idx * 2048);
+        return intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    };
+
+    dma_tile(0, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
     for (int kb = 0; kb < KB; ++kb) {
         const int cur = kb & 1;
-        const bool has_next = kb + 1 < KB;
-        if (has_next) {
+        if (kb + 1 < KB) dma_tile(kb + 1, cur ^ 1);
+        const uint8_t* la = lds_a[cur];
+        const uint8_t* lb = lds_b[cur];
+        const float* ls = lds_s[cur];
+        const uint8_t* lh = HOLD_A ? la : lb;    // held operand
+        const uint8_t* lx = HOLD_A ? lb : la;    // streamed operand
+        const int h0 = HOLD_A ? a_rd0 : b_rd0, h1 = HOLD_A ? a_rd1 : b_rd1;
+        const int x0 = HOLD_A ? b_rd0 : a_rd0, x1 = HOLD_A ? b_rd1 : a_rd1;
+        const float sb = bs_row[kb];
+        intx8 fh[NH];
 #pragma unroll
-            for (int i = 0; i < A_CHUNKS; ++i) ra[i] = *reinterpret_cast<const intx4*>(a_src[i] + (int64_t)(kb + 1) * 128);
+        for (int h = 0; h < NH; ++h) fh[h] = read_frag(lh, h0, h1, h);
+        float sc[TI];
 #pragma unroll
-            for (int i = 0; i < B_CHUNKS; ++i) rb[i] = *reinterpret_cast<const intx4*>(b_src[i] + (int64_t)(kb + 1) * 128);
-        }
-        // combined scale per (i, distinct b_s row)
-        float sa[TI];
+        for (int i = 0; i < TI; ++i) sc[i] = ls[s_rd + i * 16] * sb;
+        intx8 fx[2];
+        fx[0] = read_frag(lx, x0, x1, 0);
+        floatx4 p[DEPTH + 1];
+        constexpr int NT = TI * TJ;
 #pragma unroll
-        for (int i = 0; i < TI; ++i) sa[i] = as_ptr[i][(int64_t)kb * as_cs];
-        float sb[TJ];
-#pragma unroll
-        for (int j = 0; j < TJ; ++j) sb[j] = b_s[(int64_t)bs_row[j] * sKB + kb];
-
-        intx8 fa[TI];
-#pragma unroll
-        for (int i = 0; i < TI; ++i) {
-            const intx4 lo = *reinterpret_cast<const intx4*>(&lds_a[cur][a_off[i][0]]);
-            const intx4 hi = *reinterpret_cast<const intx4*>(&lds_a[cur][a_off[i][1]]);
-            fa[i] = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        }
-#pragma unroll
-        for (int j = 0; j < TJ; ++j) {
-            const intx4 lo = *reinterpret_cast<const intx4*>(&lds_b[cur][b_off[j][0]]);
-            const intx4 hi = *reinterpret_cast<const intx4*>(&lds_b[cur][b_off[j][1]]);
-            const intx8 fb = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-#pragma unroll
-            for (int i = 0; i < TI; ++i) {
+        for (int t = 0; t < NT + DEPTH; ++t) {
+            if (t < NT) {
+                const int si = t / NH, h = t % NH;
+                if (h == 0 && si + 1 < NS) fx[(si + 1) & 1] = read_frag(lx, x0, x1, si + 1);
+                const intx8 fa_ = HOLD_A ? fh[h] : fx[si & 1];
+                const intx8 fb_ = HOLD_A ? fx[si & 1] : fh[h];
                 const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
                 // rows of the MFMA = n (B panel), columns = m (A panel)
-                const floatx4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa[i], zero, 0, 0, 0, 0, 0, 0);
-                const float sc = sa[i] * sb[j];
-                acc[i][j][0] = __builtin_fmaf(p[0], sc, acc[i][j][0]);
-                acc[i][j][1] = __builtin_fmaf(p[1], sc, acc[i][j][1]);
-                acc[i][j][2] = __builtin_fmaf(p[2], sc, acc[i][j][2]);
-                acc[i][j][3] = __builtin_fmaf(p[3], sc, acc[i][j][3]);
+                p[t % (DEPTH + 1)] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb_, fa_, zero, 0, 0, 0, 0, 0, 0);
             }
+            if (t >= DEPTH) {
+                const int u = t - DEPTH, si = u / NH, h = u % NH;
+                const int i = HOLD_A ? h : si, j = HOLD_A ? si : h;
+                const floatx4 q = p[u % (DEPTH + 1)];
+                acc[i][j][0] = __builtin_fmaf(q[0], sc[i], acc[i][j][0]);
+                acc[i][j][1] = __builtin_fmaf(q[1], sc[i], acc[i][j][1]);
+                acc[i][j][2] = __builtin_fmaf(q[2], sc[i], acc[i][j][2]);
+                acc[i][j][3] = __builtin_fmaf(q[3], sc[i], acc[i][j][3]);
+            }
+            __builtin_amdgcn_sched_barrier(0);  // keep the MFMA / FMA / ds_read interleaving as written
         }
-        if (has_next) {
-            const int nxt = cur ^ 1;
-#pragma unroll
-            for (int i = 0; i < A_CHUNKS; ++i) *reinterpret_cast<intx4*>(&lds_a[nxt][a_dst[i]]) = ra[i];
-#pragma unroll
-            for (int i = 0; i < B_CHUNKS; ++i) *reinterpret_cast<intx4*>(&lds_b[nxt][b_dst[i]]) = rb[i];
-        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the next K block has landed in LDS
         __syncthreads();
     }
 
@@ -339,21 +344,26 @@ __global__ __launch_bounds__(256) void fp8_gemm_scalar_kernel(const uint8_t* __r
 }
 
 template <int BM, int BN, int WGM, int WGN, typename OUT>
-static int launch_mfma(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, const uint8_t* b,
-                       const float* b_s, OUT* c, const uint16_t* bias, int M, int N, int K, hipStream_t stream) {
+static int launch_mfma(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, uint32_t as_bytes,
+                       const uint8_t* b, const float* b_s, OUT* c, const uint16_t* bias, int M, int N, int K,
+                       hipStream_t stream) {
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     dim3 grid((unsigned)(tiles_m * tiles_n)), block(WGM * WGN * 64);
-    hipLaunchKernelGGL((fp8_gemm_mfma_kernel<BM, BN, WGM, WGN, OUT>), grid, block, 0, stream, a, a_s, as_rs, as_cs, b,
-                       b_s, c, bias, M, N, K, tiles_m, tiles_n);
+    hipLaunchKernelGGL((fp8_gemm_mfma_kernel<BM, BN, WGM, WGN, OUT>), grid, block, 0, stream, a, a_s, (int)as_rs,
+                       (int)as_cs, as_bytes, b, b_s, c, bias, M, N, K, tiles_m, tiles_n);
     return (int)hipGetLastError();
 }
 
 template <typename OUT>
 static int dispatch(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, const uint8_t* b,
                     const float* b_s, OUT* c, const uint16_t* bias, int M, int N, int K, hipStream_t stream) {
+    const int KB = (K + 127) / 128;
+    // byte extent of the activation scales as the MFMA kernel addresses them
+    const int64_t as_extent = ((int64_t)(M - 1) * as_rs + (int64_t)(KB - 1) * as_cs + 1) * 4;
     const bool mfma_ok = (K % 128 == 0) && ((reinterpret_cast<uintptr_t>(a) & 15) == 0) &&
                          ((reinterpret_cast<uintptr_t>(b) & 15) == 0);
-    if (!mfma_ok) {
+    const bool big_ok = mfma_ok && K <= (1 << 22) && as_rs >= 0 && as_cs >= 0 && as_extent < ((int64_t)1 << 31);
+    if (!mfma_ok || (M > 64 && !big_ok)) {
         dim3 grid((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16));
         hipLaunchKernelGGL((fp8_gemm_scalar_kernel<OUT>), grid, dim3(256), 0, stream, a, a_s, as_rs, as_cs, b, b_s, c,
                            bias, M, N, K);
@@ -372,8 +382,9 @@ static int dispatch(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t a
         return (int)hipGetLastError();
     }
     const long tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-    if (tiles256 >= 128) return launch_mfma<256, 128, 2, 2, OUT>(a, a_s, as_rs, as_cs, b, b_s, c, bias, M, N, K, stream);
-    return launch_mfma<128, 128, 2, 2, OUT>(a, a_s, as_rs, as_cs, b, b_s, c, bias, M, N, K, stream);
+    if (tiles256 >= 200)
+        return launch_mfma<256, 256, 2, 4, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, stream);
+    return launch_mfma<128, 128, 2, 2, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, stream);
 }
 
 int launch_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,

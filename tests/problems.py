@@ -18,6 +18,11 @@ def activations(kind: str, M: int, K: int, seed: int) -> torch.Tensor:
     return x.bfloat16()
 
 
+def weights_bf16(N: int, K: int, seed: int) -> torch.Tensor:
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(N, K, generator=g) * 0.02).bfloat16()
+
+
 def weights(N: int, K: int, seed: int):
     """bf16 N(0, 0.02) weights, block-quantized 128x128 (rows padded for the quantizer
     only); returns (w_bf16 [N,K], wq e4m3fn [N,K], ws fp32 [ceil(N/128), K/128])."""

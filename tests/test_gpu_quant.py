@@ -175,7 +175,7 @@ def test_quant_input_strided_rows_and_saturation():
 @pytest.mark.parametrize("N,K,only_forward,seed", [(1024, 1024, True, 0), (1536, 7168, True, 1), (200, 300, True, 2),
                                                    (200, 300, False, 3), (512, 256, False, 4), (129, 257, False, 5)])
 def test_quant_weight_bit_exact(N, K, only_forward, seed):
-    w, _, _ = P.weights(N, K, seed)
+    w = P.weights_bf16(N, K, seed)
     ref = O.quant_weight(w, only_forward)
     got = m.quant_weight(w.to(DEV), only_forward)
     for r, g in zip(ref, got):
