@@ -1,0 +1,286 @@
+#!/usr/bin/env python3
+"""Benchmark of the block-wise FP8 linear path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3] [--table]
+
+One "step" is one pass of the hot path over one batch of synthetic input that is
+already resident in HBM: act_quant(X) followed by fp8_gemm(Xq, Xs, Wq, Ws) -> bf16,
+i.e. the FP8 linear forward with a pre-quantized weight.  The default workload is
+the headline shape of the benchmark definition: DeepSeek-V3 dense MLP up/gate,
+X[4096, 7168] bf16 ~ N(0,1), W[18432, 7168] e4m3fn with 128x128 fp32 block scales.
+
+Prints ONE JSON line on stdout:
+  value        whole-step throughput in TFLOP/s (2*M*N*K / step time, quantizer included)
+  roofline     the dominant kernel (fp8_gemm): algorithmic FLOPs per launch / its
+               average launch duration, measured with HIP events on the launch stream
+               inside the timed region, against the dense FP8 MFMA peak
+  kernels      the same for act_quant and weight_dequant against the HBM peak
+               (algorithmic bytes: 3.03125*M*K and 3*N*K + 4*ceil(N/128)*ceil(K/128)),
+               each timed alone, cold cache (a 512 MiB buffer is rewritten before every launch)
+  cpu_baseline the CPU oracle (dequantize + fp32 matmul, torch CPU ops) on a bounded
+               sample of the same workload, on the host cores of this box
+With --table a per-kernel table for every benchmark configuration goes to stderr.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP8_TFLOPS = 5000.0   # MI355X dense FP8 MFMA, published
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E, published
+
+# HBM bytes per fp8_gemm launch at the C3 shape, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (KiB per dispatch, scaled by the same counters read on a plain copy kernel of known size);
+# the runs are summarised in profiles/fp8_gemm_C3_hbm_traffic.txt.  None = not measured.
+GEMM_C3_HBM_TRAFFIC_BYTES = None
+
+WORKLOADS = {
+    # name: (activation kind, M, N, K, description)
+    "C1": ("normal", 128, 1024, 1024, "CPU reference case: X[128,1024], W[1024,1024]"),
+    "C2": ("outliers", 4096, 1536, 7168, "DeepSeek-V3 attention q_a proj: X[4096,7168] (1% outliers x10), W[1536,7168]"),
+    "C3": ("normal", 4096, 18432, 7168, "DeepSeek-V3 dense MLP up/gate: X[4096,7168], W[18432,7168] (headline GEMM shape)"),
+    "C4": ("heavy", 4096, 7168, 18432, "DeepSeek-V3 dense MLP down: X[4096,18432] heavy-tailed, W[7168,18432]"),
+}
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="C3", choices=sorted(WORKLOADS))
+    ap.add_argument("--table", action="store_true", help="also print a per-kernel table for all configurations to stderr")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="first run one plain 256 MiB device-to-device copy kernel (counter calibration for rocprofv3 --pmc)")
+    return ap.parse_args()
+
+
+def make_inputs(torch, kind, M, N, K, seed, dev):
+    """Synthetic tensors of the configuration, generated on the device (values follow the
+    benchmark definition; the parity tests use CPU-generated seeded inputs instead)."""
+    g = torch.Generator(device=dev).manual_seed(seed)
+    x = torch.randn(M, K, generator=g, device=dev)
+    if kind == "outliers":
+        x = torch.where(torch.rand(M, K, generator=g, device=dev) < 0.01, x * 10, x)
+    elif kind == "heavy":
+        x = x * torch.randn(M, K, generator=g, device=dev).abs()
+    x = x.bfloat16()
+    w = (torch.randn(N, K, generator=g, device=dev) * 0.02).bfloat16()
+    return x, w
+
+
+class ColdTimer:
+    """HIP-event timing of single launches on the current stream with a cache flush before each."""
+
+    def __init__(self, torch, dev):
+        self.torch = torch
+        self.flush = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
+
+    def run(self, fn, reps, cold=True):
+        torch = self.torch
+        fn()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(reps):
+            if cold:
+                self.flush.add_(1)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1) * 1e3)
+        ts.sort()
+        return ts[len(ts) // 2], sum(ts) / len(ts)
+
+
+def cpu_baseline(torch, kind, M, N, K, xq, xs, wq, ws):
+    """The CPU oracle (dequantize activations + dequantize weights + fp32 matmul -> bf16) on a
+    bounded sample: `rows` activation rows (all of them up to 4096) against the full weight,
+    one pass.  If rows < M the row-proportional parts are extrapolated linearly."""
+    from oracle import oracle as O
+    torch.set_num_threads(os.cpu_count() or 1)
+    cores = torch.get_num_threads()
+    rows = min(M, 4096)
+    a = xq[:rows].cpu()
+    a_s = xs[:rows].cpu()
+    b = wq.cpu()
+    b_s = ws.cpu()
+    t0 = time.perf_counter()
+    bd = O.weight_dequant(b, b_s, dtype=torch.float32)
+    t1 = time.perf_counter()
+    ad = O.dequant_rows(a, a_s)
+    t2 = time.perf_counter()
+    c = (ad @ bd.t()).to(torch.bfloat16)
+    t3 = time.perf_counter()
+    t_w, t_a, t_mm = t1 - t0, t2 - t1, t3 - t2
+    full = t_w + (t_a + t_mm) * (M / rows)
+    model = ""
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    return {
+        "value": round(2.0 * M * N * K / full / 1e12, 4),
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": ("%d of %d activation rows x full W[%d,%d]: weight dequant %.2f s (once), act dequant %.3f s, "
+                   "fp32 matmul %.2f s; row-proportional parts extrapolated to %d rows -> %.1f s per step; cpu: %s"
+                   % (rows, M, N, K, t_w, t_a, t_mm, M, full, model)),
+        "checksum": float(c.float().abs().mean()),
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the path shards by N or K "
+              "without changing the kernels); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (torch.cuda.is_available() is False)", file=sys.stderr)
+        sys.exit(2)
+    import mdy_triton_amd as m
+    from mdy_triton_amd.fp8 import quant_weight  # noqa: F401  (weight side is prepared once, untimed)
+    from oracle import oracle as O
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    kind, M, N, K, desc = WORKLOADS[args.workload]
+    x, w = make_inputs(torch, kind, M, N, K, 0, dev)
+    # weight: block-quantized once with the official-dialect quantizer (amax/448, no eps)
+    wq = torch.empty(N, K, dtype=torch.float8_e4m3fn, device=dev)
+    ws = torch.empty((N + 127) // 128, K // 128, dtype=torch.float32, device=dev)
+    from mdy_triton_amd import _lib
+    _lib.check(_lib.load().mdy_weight_quant(w.data_ptr(), wq.data_ptr(), ws.data_ptr(), None, None, N, K, K, 1,
+                                            N, K, 0, None), "weight_quant")
+    torch.cuda.synchronize()
+
+    def step():
+        xq, xs = m.act_quant(x)
+        return xq, xs, m.fp8_gemm(xq, xs, wq, ws, out_dtype=torch.bfloat16)
+
+    if args.calib_copy:
+        src = torch.full((64 << 20,), 1.0, dtype=torch.float32, device=dev)   # 256 MiB
+        dst = torch.empty_like(src)
+        dst.copy_(src)                                                          # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    # ---- timed region: exactly `steps` steps; HIP events bracket every fp8_gemm launch
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        xq, xs = m.act_quant(x)
+        ev[i][0].record()
+        out = m.fp8_gemm(xq, xs, wq, ws, out_dtype=torch.bfloat16)
+        ev[i][1].record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    gemm_us = sum(a.elapsed_time(b) for a, b in ev) * 1e3 / args.steps
+    flops = 2.0 * M * N * K
+
+    # ---- the two HBM-bound kernels, each alone, cold cache
+    timer = ColdTimer(torch, dev)
+    aq_us, _ = timer.run(lambda: m.act_quant(x), 30)
+    wd_us, _ = timer.run(lambda: m.weight_dequant(wq, ws, out_dtype=torch.bfloat16), 30)
+    gemm_cold_us, _ = timer.run(lambda: m.fp8_gemm(xq, xs, wq, ws, out_dtype=torch.bfloat16), 15)
+    aq_bytes = 3.03125 * M * K
+    wd_bytes = 3.0 * N * K + 4.0 * ((N + 127) // 128) * (K // 128)
+
+    # ---- parity spot check of this very run against the oracle (a few rows)
+    rows = torch.tensor([0, M // 2, M - 1])
+    ref = O.fp8_gemm(xq[rows.to(dev)].cpu(), xs[rows.to(dev)].cpu(), wq.cpu(), ws.cpu(), dtype=torch.bfloat16)
+    parity_ok = bool(torch.allclose(out[rows.to(dev)].float().cpu(), ref.float(), rtol=1e-2, atol=1e-2))
+    yq_ref, s_ref = O.act_quant(x[rows.to(dev)].cpu())
+    parity_ok = parity_ok and bool(torch.equal(xq[rows.to(dev)].cpu().view(torch.uint8), yq_ref.view(torch.uint8))) \
+        and bool(torch.equal(xs[rows.to(dev)].cpu(), s_ref))
+
+    achieved = flops / (gemm_us * 1e-6) / 1e12
+    result = {
+        "metric": "fp8_gemm TFLOPS + % FP8 MFMA peak; act_quant/dequant GB/s + % HBM, 1 GPU",
+        "value": round(flops / (ms_per_step * 1e-3) / 1e12, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8_e4m3fn x fp8_e4m3fn -> fp32 accumulate -> bf16",
+        "data": "synthetic",
+        "config": {"workload": "%s %s; step = act_quant + fp8_gemm (pre-quantized weight)" % (args.workload, desc),
+                   "M": M, "N": N, "K": K},
+        "roofline": {"bound": "mfma", "kernel": "fp8_gemm", "achieved": round(achieved, 2), "peak": PEAK_FP8_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP8_TFLOPS, 4),
+                     "launch_us": round(gemm_us, 2), "flops_per_launch": flops,
+                     "traffic": GEMM_C3_HBM_TRAFFIC_BYTES if args.workload == "C3" else None},
+        "kernels": {
+            "fp8_gemm_cold": {"us": round(gemm_cold_us, 2), "TFLOP/s": round(flops / gemm_cold_us / 1e6, 2),
+                              "frac_mfma_peak": round(flops / gemm_cold_us / 1e6 / PEAK_FP8_TFLOPS, 4)},
+            "act_quant": {"us": round(aq_us, 2), "bytes": aq_bytes, "GB/s": round(aq_bytes / aq_us / 1e3, 1),
+                          "frac_hbm_peak": round(aq_bytes / aq_us / 1e3 / PEAK_HBM_GBS, 4)},
+            "weight_dequant": {"us": round(wd_us, 2), "bytes": wd_bytes, "GB/s": round(wd_bytes / wd_us / 1e3, 1),
+                               "frac_hbm_peak": round(wd_bytes / wd_us / 1e3 / PEAK_HBM_GBS, 4)},
+        },
+        "parity_spot_check": parity_ok,
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(torch, kind, M, N, K, xq, xs, wq, ws)
+
+    if args.table:
+        table(torch, m, timer, dev)
+    print(json.dumps(result))
+
+
+def table(torch, m, timer, dev):
+    """Per-kernel table for every configuration (stderr)."""
+    FP8 = torch.float8_e4m3fn
+
+    def line(name, us, work, unit, peak):
+        rate = work / us / (1e6 if unit == "TFLOP/s" else 1e3)
+        print("%-46s %9.1f us %10.2f %-8s %5.1f %% of peak" % (name, us, rate, unit, 100 * rate / peak), file=sys.stderr)
+
+    for name, (kind, M, N, K, _) in WORKLOADS.items():
+        x, w = make_inputs(torch, kind, M, N, K, 1, dev)
+        wq, ws, _, _ = m.quant_weight(w)
+        xq, xs = m.act_quant(x)
+        line("%s act_quant %dx%d" % (name, M, K), timer.run(lambda: m.act_quant(x), 20)[0], 3.03125 * M * K, "GB/s", PEAK_HBM_GBS)
+        line("%s weight_dequant %dx%d" % (name, N, K), timer.run(lambda: m.weight_dequant(wq, ws, out_dtype=torch.bfloat16), 20)[0],
+             3.0 * N * K + 4.0 * ((N + 127) // 128) * (K // 128), "GB/s", PEAK_HBM_GBS)
+        line("%s fp8_gemm %dx%dx%d" % (name, M, N, K), timer.run(lambda: m.fp8_gemm(xq, xs, wq, ws, out_dtype=torch.bfloat16), 10)[0],
+             2.0 * M * N * K, "TFLOP/s", PEAK_FP8_TFLOPS)
+    for M in (1, 16, 64):
+        for (N, K) in ((7168, 2048), (2048, 7168)):
+            a = torch.randint(0, 120, (M, K), dtype=torch.uint8, device=dev).view(FP8)
+            b = torch.randint(0, 120, (N, K), dtype=torch.uint8, device=dev).view(FP8)
+            a_s = torch.rand(M, K // 128, device=dev)
+            b_s = torch.rand(N // 128, K // 128, device=dev)
+            byts = M * K + N * K + 4 * M * K / 128 + 4 * (N // 128) * (K // 128) + 2 * M * N
+
+            def many():
+                for _ in range(20):
+                    m.fp8_gemm(a, a_s, b, b_s, out_dtype=torch.bfloat16)
+            us = timer.run(many, 10, cold=False)[0] / 20
+            line("C5 fp8_gemm M=%d N=%d K=%d (warm, back-to-back)" % (M, N, K), us, byts, "GB/s", PEAK_HBM_GBS)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,7 +1,5 @@
 """Tensor plumbing shared by the operator modules: device checks, raw pointers,
 the current HIP stream.  PyTorch is used for memory and streams only."""
-import contextlib
-
 import torch
 
 from . import _lib
@@ -28,14 +26,25 @@ def stream_ptr(device):
     return torch.cuda.current_stream(device).cuda_stream
 
 
-@contextlib.contextmanager
+class _NoSwitch:
+    __slots__ = ()
+
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
 def on_device(device):
-    """Make `device` current for the launch (kernels go to the current device)."""
+    """Context that makes `device` current for the launch (kernels go to the current
+    device); free when it already is."""
     if torch.cuda.current_device() == device.index:
-        yield
-    else:
-        with torch.cuda.device(device):
-            yield
+        return _NO_SWITCH
+    return torch.cuda.device(device)
 
 
 def out_code(dtype):

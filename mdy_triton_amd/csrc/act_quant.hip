@@ -13,6 +13,7 @@
 //     element is x*r corrected by two FMAs (bit-identical to x / scale, proven
 //     exhaustively over bf16 x bf16); groups whose amax is tiny, above 1e4
 //     (DeepLinear dialect, needs the saturating cast) or non-finite divide plainly;
+//   * loads and stores are non-temporal (every byte is touched once);
 //   * v_cvt_pk_fp8_f32 x4 -> one 8-byte store per lane; lane 0 of the row stores
 //     the scale at a caller-given (row, column) stride so that both the row-major
 //     [M, K/128] layout and the column-major padded [K/128][PM] layout come out
@@ -84,7 +85,7 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restri
         if (row < M && col < K) {
             const uint16_t* p = x + (int64_t)row * x_row_stride + col;
             if (VEC) {
-                raw[r] = *reinterpret_cast<const uint4*>(p);  // K % 8 == 0: all 8 columns in range
+                raw[r] = load_nt16(p);  // K % 8 == 0: all 8 columns in range
             } else {
                 uint32_t w[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
@@ -112,7 +113,7 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restri
         float scale;
         const uint2 packed = quantize8<MODE>(f, amax, scale);
         if (row < PM && col_in_out) {
-            *reinterpret_cast<uint2*>(y + (int64_t)row * PK + col) = packed;
+            store_nt8(y + (int64_t)row * PK + col, packed);
             if ((lane & 15) == 0) s[(int64_t)row * s_row_stride + (int64_t)(col >> 7) * s_col_stride] = scale;
         }
     }

@@ -66,6 +66,27 @@ __device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float 
     return (uint32_t)w;
 }
 
+// Streaming (non-temporal) vector accesses: the quantizers and the dequantizer touch every
+// byte exactly once, so they bypass cache allocation; measured 1.25-1.5x over plain accesses.
+typedef unsigned uintx4_t __attribute__((ext_vector_type(4)));
+typedef unsigned uintx2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint4 load_nt16(const void* p) {
+    const uintx4_t v = __builtin_nontemporal_load(static_cast<const uintx4_t*>(p));
+    return make_uint4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ uint2 load_nt8(const void* p) {
+    const uintx2_t v = __builtin_nontemporal_load(static_cast<const uintx2_t*>(p));
+    return make_uint2(v[0], v[1]);
+}
+__device__ __forceinline__ void store_nt16(void* p, const uint4& v) {
+    const uintx4_t u = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(u, static_cast<uintx4_t*>(p));
+}
+__device__ __forceinline__ void store_nt8(void* p, const uint2& v) {
+    const uintx2_t u = {v.x, v.y};
+    __builtin_nontemporal_store(u, static_cast<uintx2_t*>(p));
+}
+
 __device__ __forceinline__ uint32_t pack2_bf16(float a, float b) {
     floatx2 f = {a, b};
     bf16x2 h = __builtin_convertvector(f, bf16x2);

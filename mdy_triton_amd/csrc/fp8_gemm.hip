@@ -41,6 +41,8 @@ __device__ __forceinline__ void store4(OUT* c, int64_t ldc, int m, int n, int M,
     if (m >= M || n >= N) return;
     OUT* p = c + (int64_t)m * ldc + n;
     if (vec_ok && n + 3 < N) {
+        // plain (cached) stores: the 8-byte pieces of a line written by different instructions are
+        // merged in L2; non-temporal stores measured ~5 % slower here
         if (sizeof(OUT) == 2) {
             *reinterpret_cast<uint2*>(p) = make_uint2(pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]));
         } else {

@@ -8,7 +8,8 @@
 // bytes (one 8-byte load), expands them with v_cvt_pk_f32_fp8, multiplies by the
 // scale of its 128x128 block (one scalar-ish load per lane, same address for 16
 // neighbouring lanes, L1/L2 resident) and writes 8 bf16 as one 16-byte store, so
-// a wave's store instruction covers 1 KiB of contiguous output.  Each wave walks
+// a wave's store instruction covers 1 KiB of contiguous output.  All tile accesses are
+// non-temporal (no cache allocation for data touched once).  Each wave walks
 // kWdRows rows of a 512-column stripe to keep several loads in flight.
 //
 // HBM traffic per element: 1 B in + 2 B out (+ 4 B per 16384 elements of scale).
@@ -39,7 +40,7 @@ __global__ __launch_bounds__(256) void weight_dequant_kernel(const uint8_t* __re
         if (row < N) {
             const uint8_t* p = x + (int64_t)row * K + col;
             if (VEC) {
-                raw[r] = *reinterpret_cast<const uint2*>(p);
+                raw[r] = load_nt8(p);
             } else {
                 uint32_t w[2] = {0u, 0u};
 #pragma unroll
@@ -65,7 +66,7 @@ __global__ __launch_bounds__(256) void weight_dequant_kernel(const uint8_t* __re
             if (VEC) {
                 uint4 o = make_uint4(pack2_bf16(f[0], f[1]), pack2_bf16(f[2], f[3]), pack2_bf16(f[4], f[5]),
                                      pack2_bf16(f[6], f[7]));
-                *reinterpret_cast<uint4*>(q) = o;
+                store_nt16(q, o);
             } else {
 #pragma unroll
                 for (int i = 0; i < 8; ++i)
@@ -73,8 +74,8 @@ __global__ __launch_bounds__(256) void weight_dequant_kernel(const uint8_t* __re
             }
         } else {
             if (VEC) {
-                reinterpret_cast<float4*>(q)[0] = make_float4(f[0], f[1], f[2], f[3]);
-                reinterpret_cast<float4*>(q)[1] = make_float4(f[4], f[5], f[6], f[7]);
+                store_nt16(q, make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3])));
+                store_nt16(q + 4, make_uint4(__float_as_uint(f[4]), __float_as_uint(f[5]), __float_as_uint(f[6]), __float_as_uint(f[7])));
             } else {
 #pragma unroll
                 for (int i = 0; i < 8; ++i)

@@ -42,7 +42,7 @@ __global__ __launch_bounds__(256) void weight_quant_kernel(const uint16_t* __res
         uint32_t wd[4] = {0u, 0u, 0u, 0u};
         if (row < N && c0 < K) {
             if (VEC) {
-                const uint4 v = *reinterpret_cast<const uint4*>(w + (int64_t)row * w_row_stride + c0);
+                const uint4 v = load_nt16(w + (int64_t)row * w_row_stride + c0);
                 wd[0] = v.x; wd[1] = v.y; wd[2] = v.z; wd[3] = v.w;
             } else {
 #pragma unroll
@@ -93,7 +93,7 @@ __global__ __launch_bounds__(256) void weight_quant_kernel(const uint16_t* __res
         o.x = pack4_e4m3(q[0], q[1], q[2], q[3]);
         o.y = pack4_e4m3(q[4], q[5], q[6], q[7]);
         const int row = rbase + 16 * i;  // < PN because PN % 128 == 0
-        *reinterpret_cast<uint2*>(y + (int64_t)row * PK + c0) = o;
+        store_nt8(y + (int64_t)row * PK + c0, o);
         if (y_t) *reinterpret_cast<uint2*>(&tile[(t >> 4) + 16 * i][(t & 15) * 8]) = o;
     }
     if (y_t) {
@@ -109,7 +109,7 @@ __global__ __launch_bounds__(256) void weight_quant_kernel(const uint16_t* __res
                 lo |= (uint32_t)tile[nn + j][kk] << (8 * j);
                 hi |= (uint32_t)tile[nn + 4 + j][kk] << (8 * j);
             }
-            *reinterpret_cast<uint2*>(y_t + (int64_t)(bk * 128 + kk) * PN + bn * 128 + nn) = make_uint2(lo, hi);
+            store_nt8(y_t + (int64_t)(bk * 128 + kk) * PN + bn * 128 + nn, make_uint2(lo, hi));
         }
     }
 }
