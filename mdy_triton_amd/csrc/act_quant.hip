@@ -24,9 +24,9 @@
 
 namespace mdy {
 
-constexpr int kAqRowsPerWave = 4;
+constexpr int kAqRowsPerWave = 2;
 constexpr int kAqWaves = 4;
-constexpr int kAqRowsPerBlock = kAqRowsPerWave * kAqWaves;  // 16 rows x 512 columns per block
+constexpr int kAqRowsPerBlock = kAqRowsPerWave * kAqWaves;  // 8 rows x 512 columns per block
 
 __device__ __forceinline__ float row16_max(float v) {
     // butterfly over the 16 lanes of a DPP row: xor 1, xor 2 (quad_perm), then
@@ -66,7 +66,7 @@ __device__ __forceinline__ uint2 quantize8(const float (&f)[8], float amax, floa
     return out;
 }
 
-// grid.x = ceil(PK / 512), grid.y = ceil(PM / 16), block = 256
+// grid.x = ceil(PK / 512), grid.y = ceil(PM / 8), block = 256
 template <int MODE, bool VEC>
 __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ y,
                                                          float* __restrict__ s, int M, int K, int64_t x_row_stride,

@@ -27,8 +27,8 @@
 //     whole K block, the other one is streamed through a two-deep register queue;
 //   * workgroup ids are remapped so that the 32 workgroups that share an XCD's L2
 //     cover a compact 4 x 8 block of tiles.
-// Small-M kernel (M <= 64): weight streaming, one workgroup per 16 columns, waves
-// split K and reduce through LDS.  Scalar kernel: any other shape/alignment.
+// Small-M kernel (M <= 64): weight streaming, one workgroup of 8 waves per 16 columns,
+// waves split K (next block prefetched) and reduce through LDS.  Scalar kernel: any other shape/alignment.
 #include "common.h"
 
 namespace mdy {
@@ -240,18 +240,24 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// Small-M kernel: M <= 16*MT rows.  One workgroup (4 waves) per 16 output
-// columns; wave w handles K blocks w, w+4, ...; B fragments come straight from
-// global memory (each row slice is one full 128-byte line), A fragments too (A is
-// tiny and L2 resident).  Partial sums are reduced through LDS.
+// Small-M kernel: M <= 16*MT rows (decode / routed-expert shapes).  Pure weight
+// streaming: one workgroup of 8 waves per 16 output columns; wave w takes K blocks
+// w, w+8, ... and keeps the loads of the next block in flight while the MFMAs of
+// the current one run; B fragments come straight from global memory (each row
+// slice of a K block is one full 128-byte line, read once, non-temporal), A
+// fragments too (A is tiny and L2 resident).  Partial sums are reduced through LDS.
 // ---------------------------------------------------------------------------
+constexpr int kSmWaves = 8;
+
 template <int MT, typename OUT>
-__global__ __launch_bounds__(256) void fp8_gemm_smallm_kernel(const uint8_t* __restrict__ a,
-                                                               const float* __restrict__ a_s, int64_t as_rs,
-                                                               int64_t as_cs, const uint8_t* __restrict__ b,
-                                                               const float* __restrict__ b_s, OUT* __restrict__ c,
-                                                               const uint16_t* __restrict__ bias, int M, int N, int K) {
-    __shared__ float red[4][MT][64][4];
+__global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_kernel(const uint8_t* __restrict__ a,
+                                                                          const float* __restrict__ a_s, int64_t as_rs,
+                                                                          int64_t as_cs, const uint8_t* __restrict__ b,
+                                                                          const float* __restrict__ b_s,
+                                                                          OUT* __restrict__ c,
+                                                                          const uint16_t* __restrict__ bias, int M,
+                                                                          int N, int K) {
+    __shared__ float red[kSmWaves][MT][64][4];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int frow = lane & 15, fk = lane >> 4;
@@ -260,24 +266,50 @@ __global__ __launch_bounds__(256) void fp8_gemm_smallm_kernel(const uint8_t* __r
     const int nrow = min(n0 + frow, N - 1);
     const uint8_t* bp = b + (int64_t)nrow * K + fk * 32;
     const float* bsp = b_s + (int64_t)(n0 >> 7) * KB;
+    const uint8_t* ap[MT];
+    const float* asp[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int m = min(i * 16 + frow, M - 1);
+        ap[i] = a + (int64_t)m * K + fk * 32;
+        asp[i] = a_s + (int64_t)m * as_rs;
+    }
 
     floatx4 acc[MT];
 #pragma unroll
     for (int i = 0; i < MT; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    for (int kb = wave; kb < KB; kb += 4) {
-        const intx4 blo = *reinterpret_cast<const intx4*>(bp + (int64_t)kb * 128);
-        const intx4 bhi = *reinterpret_cast<const intx4*>(bp + (int64_t)kb * 128 + 16);
-        const intx8 fb = intx8{blo[0], blo[1], blo[2], blo[3], bhi[0], bhi[1], bhi[2], bhi[3]};
-        const float sb = bsp[kb];
+    // everything one K block needs: B fragment, MT A fragments, MT activation scales, the weight scale
+    struct Operands {
+        uint4 blo, bhi;
+        intx4 alo[MT], ahi[MT];
+        float sa[MT];
+        float sb;
+    };
+    auto load_block = [&](int kb, Operands& o) {
+        o.blo = load_nt16(bp + (int64_t)kb * 128);
+        o.bhi = load_nt16(bp + (int64_t)kb * 128 + 16);
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
-            const int m = min(i * 16 + frow, M - 1);
-            const uint8_t* ap = a + (int64_t)m * K + (int64_t)kb * 128 + fk * 32;
-            const intx4 alo = *reinterpret_cast<const intx4*>(ap);
-            const intx4 ahi = *reinterpret_cast<const intx4*>(ap + 16);
-            const intx8 fa = intx8{alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
-            const float sc = a_s[(int64_t)m * as_rs + (int64_t)kb * as_cs] * sb;
+            o.alo[i] = *reinterpret_cast<const intx4*>(ap[i] + (int64_t)kb * 128);
+            o.ahi[i] = *reinterpret_cast<const intx4*>(ap[i] + (int64_t)kb * 128 + 16);
+            o.sa[i] = asp[i][(int64_t)kb * as_cs];
+        }
+        o.sb = bsp[kb];
+    };
+    Operands cur, nxt;
+    int kb = wave;
+    if (kb < KB) load_block(kb, cur);
+    for (; kb < KB; kb += kSmWaves) {
+        const bool more = kb + kSmWaves < KB;
+        if (more) load_block(kb + kSmWaves, nxt);   // in flight while this block's MFMAs run
+        const intx8 fb = intx8{(int)cur.blo.x, (int)cur.blo.y, (int)cur.blo.z, (int)cur.blo.w,
+                               (int)cur.bhi.x, (int)cur.bhi.y, (int)cur.bhi.z, (int)cur.bhi.w};
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const intx8 fa = intx8{cur.alo[i][0], cur.alo[i][1], cur.alo[i][2], cur.alo[i][3],
+                                   cur.ahi[i][0], cur.ahi[i][1], cur.ahi[i][2], cur.ahi[i][3]};
+            const float sc = cur.sa[i] * cur.sb;
             const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
             const floatx4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, zero, 0, 0, 0, 0, 0, 0);
             acc[i][0] = __builtin_fmaf(p[0], sc, acc[i][0]);
@@ -285,28 +317,32 @@ __global__ __launch_bounds__(256) void fp8_gemm_smallm_kernel(const uint8_t* __r
             acc[i][2] = __builtin_fmaf(p[2], sc, acc[i][2]);
             acc[i][3] = __builtin_fmaf(p[3], sc, acc[i][3]);
         }
+        if (more) cur = nxt;
     }
 #pragma unroll
     for (int i = 0; i < MT; ++i)
 #pragma unroll
         for (int e = 0; e < 4; ++e) red[wave][i][lane][e] = acc[i][e];
     __syncthreads();
-    if (wave == 0) {
+    if (wave < MT) {
+        // wave i reduces row sub-tile i (fixed order, so results do not depend on timing)
+        const int i = wave;
         const bool vec_ok = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
+        float v[4];
 #pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            float v[4];
+        for (int e = 0; e < 4; ++e) {
+            float t = 0.0f;
+#pragma unroll
+            for (int w = 0; w < kSmWaves; ++w) t += red[w][i][lane][e];
+            v[e] = t;
+        }
+        const int m = i * 16 + frow, n = n0 + 4 * fk;
+        if (bias != nullptr) {
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-                v[e] = (red[0][i][lane][e] + red[1][i][lane][e]) + (red[2][i][lane][e] + red[3][i][lane][e]);
-            const int m = i * 16 + frow, n = n0 + 4 * fk;
-            if (bias != nullptr) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (n + e < N) v[e] += bf16_one(bias[n + e]);
-            }
-            store4<OUT>(c, N, m, n, M, N, v, vec_ok);
+                if (n + e < N) v[e] += bf16_one(bias[n + e]);
         }
+        store4<OUT>(c, N, m, n, M, N, v, vec_ok);
     }
 }
 
@@ -374,7 +410,7 @@ static int dispatch(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t a
     if (M <= 64) {
         dim3 grid((unsigned)((N + 15) / 16));
 #define MDY_SM(MT)                                                                                                 \
-    hipLaunchKernelGGL((fp8_gemm_smallm_kernel<MT, OUT>), grid, dim3(256), 0, stream, a, a_s, as_rs, as_cs, b, b_s, \
+    hipLaunchKernelGGL((fp8_gemm_smallm_kernel<MT, OUT>), grid, dim3(kSmWaves * 64), 0, stream, a, a_s, as_rs, as_cs, b, b_s, \
                        c, bias, M, N, K)
         if (M <= 16) MDY_SM(1);
         else if (M <= 32) MDY_SM(2);

@@ -17,7 +17,7 @@
 
 namespace mdy {
 
-constexpr int kWdRows = 4;           // rows per wave (independent loads in flight)
+constexpr int kWdRows = 2;           // rows per wave (independent loads in flight)
 constexpr int kWdWaves = 4;          // waves per block
 constexpr int kWdCols = 64 * 8;      // columns per wave pass
 
