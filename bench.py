@@ -36,8 +36,10 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E, published
 
 # HBM bytes per fp8_gemm launch at the C3 shape, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (KiB per dispatch, scaled by the same counters read on a plain copy kernel of known size);
-# the runs are summarised in profiles/fp8_gemm_C3_hbm_traffic.txt.  None = not measured.
-GEMM_C3_HBM_TRAFFIC_BYTES = None
+# the runs are summarised in profiles/bench_C3_hbm_traffic.txt: FETCH_SIZE 407 706 KiB x 1.9997 (copy-kernel
+# calibration) = 834.9 MB read, WRITE_SIZE 150 687 KiB x 1.0 = 154.3 MB written; algorithmic bytes are 313 MB
+# (the A and B panels are re-fetched by the eight XCD-local L2s).
+GEMM_C3_HBM_TRAFFIC_BYTES = 989.2e6
 
 WORKLOADS = {
     # name: (activation kind, M, N, K, description)
