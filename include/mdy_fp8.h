@@ -79,6 +79,27 @@ int mdy_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t, in
                      int64_t w_row_stride, int64_t w_col_stride, int64_t PN, int64_t PK, int mode,
                      void* stream);
 
+/* Training-time quantizer: row-wise 1x128 quantization of x AND the quantized transpose,
+ * one read of x.  DeepLinear dialect only (clamp 1e4 + eps 1e-8, saturating cast).
+ * Replaces quant_grad_output (fp8.py:46-77, kernel :13-44) with t_mode = MDY_T_COLUMN and
+ * quant_input(only_forward=False) (fp8.py:122-161, kernel branch :115-120) with
+ * t_mode = MDY_T_BLOCK.
+ *
+ *   x    bf16 [M, K], element (m, k) at x[m * x_row_stride + k * x_col_stride]
+ *   y    e4m3fn [PM, PK] row-major, PM % 128 == 0, PK % 128 == 0, padding reads as 0
+ *   s    fp32, scale of row m, K-group kb at s[kb * PM + m]          ([PK/128, PM] row-major)
+ *   y_t  e4m3fn [PK, PM] row-major: y_t[k, m] = x[m, k] / scale_t
+ *   s_t  MDY_T_COLUMN: one scale per column k and 128-row group a, at s_t[a * PK + k]
+ *                      ([PM/128, PK] row-major; the reference returns its transpose view)
+ *        MDY_T_BLOCK:  one scale per 128x128 tile, at s_t[(k/128) * (PM/128) + m/128]
+ *                      ([PK/128, PM/128] row-major)
+ */
+#define MDY_T_COLUMN 0
+#define MDY_T_BLOCK 1
+int mdy_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
+                        int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int t_mode,
+                        void* stream);
+
 /* 128x128 block weight dequantizer: y[n,k] = fp32(x[n,k]) * s[n/128, k/128].
  * Replaces weight_dequant (offical_kernel.py:46-53, kernel :31-43).
  *   x e4m3fn [N, K] row-major; s fp32 [ceil(N/128), ceil(K/128)] row-major;

@@ -3,7 +3,7 @@ mdy666/mdy_triton, rebuilt for AMD MI355X (gfx950) as hand-written HIP kernels
 behind a C ABI.  Importing the package does not load the library; the first
 operator call does, and raises if it has not been built."""
 from .offical_kernel import act_quant, fp8_gemm, weight_dequant  # noqa: F401
-from .fp8 import DeepLinear, add_bias, fp8_matmul, quant_input, quant_weight  # noqa: F401
+from .fp8 import DeepLinear, add_bias, fp8_matmul, quant_grad_output, quant_input, quant_weight  # noqa: F401
 
-__all__ = ["act_quant", "weight_dequant", "fp8_gemm", "quant_input", "quant_weight", "fp8_matmul", "add_bias",
+__all__ = ["act_quant", "weight_dequant", "fp8_gemm", "quant_input", "quant_weight", "quant_grad_output", "fp8_matmul", "add_bias",
            "DeepLinear"]

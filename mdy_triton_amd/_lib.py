@@ -23,6 +23,7 @@ _int = ctypes.c_int
 SIGNATURES = {
     "mdy_act_quant": [_p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p],
     "mdy_weight_quant": [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p],
+    "mdy_quant_transpose": [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p],
     "mdy_weight_dequant": [_p, _p, _p, _i64, _i64, _int, _p],
     "mdy_fp8_gemm_nt": [_p, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p],
     "mdy_add_bias": [_p, _p, _i64, _i64, _p],

@@ -89,6 +89,23 @@ int mdy_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t, in
                     "weight_quant");
 }
 
+int mdy_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
+                        int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int t_mode, void* stream) {
+    if (t_mode != MDY_T_COLUMN && t_mode != MDY_T_BLOCK) return fail(MDY_E_DTYPE, "quant_transpose: unknown t_mode %d", t_mode);
+    if (M < 0 || K < 0 || PM < M || PK < K || PM > kMaxDim || PK > kMaxDim)
+        return fail(MDY_E_SHAPE, "quant_transpose: need 0 <= M <= PM, 0 <= K <= PK");
+    if (PM % 128 != 0 || PK % 128 != 0) return fail(MDY_E_SHAPE, "quant_transpose: PM=%lld, PK=%lld must be multiples of 128", (long long)PM, (long long)PK);
+    if (PM / 128 > 65535) return fail(MDY_E_SHAPE, "quant_transpose: PM too large");
+    if (PM == 0 || PK == 0) return 0;
+    if (!y || !s || !y_t || !s_t || (!x && M > 0 && K > 0)) return fail(MDY_E_NULL, "quant_transpose: null pointer");
+    if (!aligned(y, 8) || !aligned(y_t, 8)) return fail(MDY_E_ALIGN, "quant_transpose: y / y_t must be 8-byte aligned");
+    if (!aligned(x, 2) || !aligned(s, 4) || !aligned(s_t, 4)) return fail(MDY_E_ALIGN, "quant_transpose: x/s/s_t misaligned for their element type");
+    if (int e = check_device()) return e;
+    return launched(mdy::launch_quant_transpose(x, y, s, y_t, s_t, M, K, x_row_stride, x_col_stride, PM, PK, t_mode,
+                                                static_cast<hipStream_t>(stream)),
+                    "quant_transpose");
+}
+
 int mdy_weight_dequant(const void* x, const float* s, void* y, int64_t N, int64_t K, int out_dtype, void* stream) {
     if (out_dtype != MDY_DT_BF16 && out_dtype != MDY_DT_F32) return fail(MDY_E_DTYPE, "weight_dequant: unknown out_dtype %d", out_dtype);
     if (N < 0 || K < 0 || N > kMaxDim || K > kMaxDim) return fail(MDY_E_SHAPE, "weight_dequant: bad shape");

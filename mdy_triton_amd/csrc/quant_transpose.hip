@@ -1,0 +1,197 @@
+// Training-time quantizer: one pass over a bf16 matrix produces
+//   (1) the row-wise 1x128 quantization y[PM,PK] with scales s[kb*PM + m]      (as the forward quantizer), and
+//   (2) the quantized TRANSPOSE y_t[PK,PM], scaled either per 128x1 column group (t_mode 0) or per
+//       128x128 block (t_mode 1),
+// both in the DeepLinear dialect (scale = (min(amax,1e4) + 1e-8) / 448, saturating cast).
+//
+// Restates _quant_grad_output_kernel (/root/reference/triton_kernels/dpsk_fp8linear/fp8.py:13-44;
+// t_mode 0: second half at :40-44 quantizes along axis 0 and stores ST[off_n + pid_m*PN]) and the
+// training branch of _quant_input_kernel (fp8.py:115-120; t_mode 1: one scale per 128x128 tile, the
+// max of the rows' clamped+eps maxima, stored ST[pid_n*num_programs(0) + pid_m]).
+//
+// One 256-thread block per 128x128 tile, the tile stays in registers (read once).  Thread t owns
+// columns (t%16)*8..+7 of rows t/16 + 16*i: row maxima by DPP inside 16-lane rows, column maxima by
+// a per-thread max over its 8 rows followed by an LDS reduction over the 16 row groups.  Quotients
+// use the reciprocal + 2-FMA form (bit-identical to IEEE division for every finite amax in this
+// dialect); groups whose amax exceeds the 1e4 clamp or is not finite divide plainly and clamp.
+// The transposed bytes go through a padded LDS tile so that both outputs are written row-contiguously.
+#include "common.h"
+
+namespace mdy {
+
+__device__ __forceinline__ float qt_row16_max(float v) {
+    int i = __float_as_int(v);
+    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0xB1, 0xF, 0xF, true))));
+    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0x4E, 0xF, 0xF, true))));
+    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0x141, 0xF, 0xF, true))));
+    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0x140, 0xF, 0xF, true))));
+    return __int_as_float(i);
+}
+
+// x / s in the DeepLinear dialect.  FAST (amax <= 1e4, so |x/s| <= 448 needs no clamp) uses the
+// reciprocal form; otherwise an IEEE division saturated at +-448 (NaN kept).
+template <bool FAST>
+__device__ __forceinline__ float qt_quot(float x, float s, float r) {
+    if (FAST) return fast_quotient(x, s, r);
+    return sat_for_mode<1>(x / s);
+}
+
+template <int TMODE, bool VEC>
+__global__ __launch_bounds__(256) void quant_transpose_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ y,
+                                                               float* __restrict__ s, uint8_t* __restrict__ y_t,
+                                                               float* __restrict__ s_t, int M, int K,
+                                                               int64_t x_row_stride, int64_t x_col_stride, int PM,
+                                                               int PK) {
+    __shared__ float col_part[16][128];   // per row group (t/16) partial column maxima
+    __shared__ float col_amax[128];
+    __shared__ float blk_part[4];
+    __shared__ __attribute__((aligned(16))) uint8_t tile[128][128 + 16];
+
+    const int t = threadIdx.x;
+    const int lane = t & 63, wave = t >> 6;
+    const int bm = blockIdx.y, bk = blockIdx.x;
+    const int cl = (t & 15) * 8;          // first local column of this thread
+    const int rg = t >> 4;                // row group 0..15
+    const int c0 = bk * 128 + cl;
+
+    float f[8][8];
+    float rmax[8];
+    float cmax[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) cmax[j] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int row = bm * 128 + rg + 16 * i;
+        uint32_t wd[4] = {0u, 0u, 0u, 0u};
+        if (row < M && c0 < K) {
+            if (VEC) {
+                const uint4 v = load_nt16(x + (int64_t)row * x_row_stride + c0);
+                wd[0] = v.x; wd[1] = v.y; wd[2] = v.z; wd[3] = v.w;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (c0 + j < K)
+                        wd[j >> 1] |= (uint32_t)x[(int64_t)row * x_row_stride + (int64_t)(c0 + j) * x_col_stride]
+                                      << ((j & 1) * 16);
+            }
+        }
+        float m = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            f[i][2 * j] = bf16_lo(wd[j]);
+            f[i][2 * j + 1] = bf16_hi(wd[j]);
+            m = fmaxf(fmaxf(fabsf(f[i][2 * j]), fabsf(f[i][2 * j + 1])), m);
+            cmax[2 * j] = fmaxf(cmax[2 * j], fabsf(f[i][2 * j]));
+            cmax[2 * j + 1] = fmaxf(cmax[2 * j + 1], fabsf(f[i][2 * j + 1]));
+        }
+        rmax[i] = qt_row16_max(m);
+    }
+
+    // ---- (1) row-wise quantization straight from registers
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int row = bm * 128 + rg + 16 * i;     // < PM
+        const float sc = group_scale<1>(rmax[i]);
+        const float r = 1.0f / sc;
+        float q[8];
+        if (rmax[i] <= 1e4f) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) q[j] = qt_quot<true>(f[i][j], sc, r);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) q[j] = qt_quot<false>(f[i][j], sc, r);
+        }
+        store_nt8(y + (int64_t)row * PK + c0, make_uint2(pack4_e4m3(q[0], q[1], q[2], q[3]), pack4_e4m3(q[4], q[5], q[6], q[7])));
+        if ((t & 15) == 0) s[(int64_t)bk * PM + row] = sc;
+    }
+
+    // ---- (2) scales of the transposed copy
+    float tamax[8];   // amax that scales this thread's 8 columns in the transposed copy
+    if (TMODE == 0) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) col_part[rg][cl + j] = cmax[j];
+        __syncthreads();
+        if (t < 128) {
+            float m = 0.0f;
+#pragma unroll
+            for (int g = 0; g < 16; ++g) m = fmaxf(m, col_part[g][t]);
+            col_amax[t] = m;
+            // logical s_t[k, a]: stored [A][PK]
+            s_t[(int64_t)bm * PK + bk * 128 + t] = group_scale<1>(m);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 8; ++j) tamax[j] = col_amax[cl + j];
+    } else {
+        float m = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) m = fmaxf(m, rmax[i]);
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+        if (lane == 0) blk_part[wave] = m;
+        __syncthreads();
+        const float bmax = fmaxf(fmaxf(blk_part[0], blk_part[1]), fmaxf(blk_part[2], blk_part[3]));
+        if (t == 0) s_t[(int64_t)bk * (PM >> 7) + bm] = group_scale<1>(bmax);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) tamax[j] = bmax;
+    }
+    float tsc[8], tr[8];
+    bool tfast = true;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        tsc[j] = group_scale<1>(tamax[j]);
+        tr[j] = 1.0f / tsc[j];
+        tfast = tfast && (tamax[j] <= 1e4f);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        float q[8];
+        if (tfast) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) q[j] = qt_quot<true>(f[i][j], tsc[j], tr[j]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) q[j] = qt_quot<false>(f[i][j], tsc[j], tr[j]);
+        }
+        *reinterpret_cast<uint2*>(&tile[rg + 16 * i][cl]) =
+            make_uint2(pack4_e4m3(q[0], q[1], q[2], q[3]), pack4_e4m3(q[4], q[5], q[6], q[7]));
+    }
+    __syncthreads();
+    // y_t[k][m]: thread owns output columns (t%16)*8..+7 (m) of output rows t/16 + 16*i (k)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int kk = rg + 16 * i;
+        uint32_t lo = 0u, hi = 0u;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            lo |= (uint32_t)tile[cl + j][kk] << (8 * j);
+            hi |= (uint32_t)tile[cl + 4 + j][kk] << (8 * j);
+        }
+        store_nt8(y_t + (int64_t)(bk * 128 + kk) * PM + bm * 128 + cl, make_uint2(lo, hi));
+    }
+}
+
+int launch_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
+                           int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int t_mode,
+                           hipStream_t stream) {
+    if (PM == 0 || PK == 0) return 0;
+    dim3 grid((unsigned)(PK / 128), (unsigned)(PM / 128));
+    dim3 block(256);
+    const bool vec = (x_col_stride == 1) && (K % 8 == 0) && (x_row_stride % 8 == 0) &&
+                     ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+    const uint16_t* xp = static_cast<const uint16_t*>(x);
+    uint8_t* yp = static_cast<uint8_t*>(y);
+    uint8_t* ytp = static_cast<uint8_t*>(y_t);
+#define MDY_QT(TM, VEC)                                                                                          \
+    hipLaunchKernelGGL((quant_transpose_kernel<TM, VEC>), grid, block, 0, stream, xp, yp, s, ytp, s_t, (int)M, \
+                       (int)K, x_row_stride, x_col_stride, (int)PM, (int)PK)
+    if (t_mode == 0) {
+        if (vec) MDY_QT(0, true); else MDY_QT(0, false);
+    } else {
+        if (vec) MDY_QT(1, true); else MDY_QT(1, false);
+    }
+#undef MDY_QT
+    return (int)hipGetLastError();
+}
+
+}  // namespace mdy

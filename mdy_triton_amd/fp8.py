@@ -17,18 +17,51 @@ def _cdiv(a: int, b: int) -> int:
     return (a + b - 1) // b
 
 
+def _quant_transpose(x: torch.Tensor, t_mode: int, who: str):
+    """Shared launcher of the two training-time quantizers (row-wise copy + quantized transpose)."""
+    if x.dim() != 2:
+        raise ValueError("%s expects a 2-D tensor" % who)
+    if x.dtype != torch.bfloat16:
+        raise TypeError("%s expects bfloat16, got %s" % (who, x.dtype))
+    dev = require_gpu(x)
+    M, K = x.shape
+    PM, PN = _cdiv(M, 256) * 256, _cdiv(K, 256) * 256
+    A, B = PM // 128, PN // 128
+    y = torch.empty(PM, PN, device=dev, dtype=FP8)
+    s = torch.empty(B, PM, device=dev, dtype=torch.float32)
+    y_t = torch.empty(PN, PM, device=dev, dtype=FP8)
+    s_t = torch.empty((A, PN) if t_mode == 0 else (B, A), device=dev, dtype=torch.float32)
+    with on_device(dev):
+        check(lib().mdy_quant_transpose(ptr(x), ptr(y), ptr(s), ptr(y_t), ptr(s_t), M, K, x.stride(0), x.stride(1),
+                                        PM, PN, t_mode, stream_ptr(dev)), who)
+    return y, s.transpose(0, 1), y_t, s_t
+
+
+def quant_grad_output(x: torch.Tensor):
+    """Output-gradient quantizer of the backward pass (fp8.py:46-77).
+
+    x [M, N] bf16, any strides.  Returns (y, s, y_t, s_t) with PM = cdiv(M,256)*256,
+    PN = cdiv(N,256)*256: y [PM, PN] quantized along N in groups of 128, s logical
+    [PM, PN/128] with strides (1, PM); y_t [PN, PM] quantized along M in groups of
+    128, s_t logical [PN, PM/128] with strides (1, PN).
+    """
+    y, s, y_t, s_t = _quant_transpose(x, 0, "quant_grad_output")
+    return y, s, y_t, s_t.transpose(0, 1)
+
+
 def quant_input(x: torch.Tensor, only_forward: bool = True):
     """1x128 activation quantizer with clamp(amax, 0, 1e4) + 1e-8 (fp8.py:122-161).
 
     x [M, K] bf16, last dim unit-strided or not (a non-unit column stride is
-    copied first).  Returns (y, s, y_t, s_t):
-      y [PM, PN] e4m3fn, PN = cdiv(K,256)*256, PM = cdiv(M,4)*4;
-      s logical [PM, PN/128] with strides (1, PM) (column-major, as fp8.py:134,161).
-    Only only_forward=True is implemented: the transposed outputs belong to the
-    backward pass.
+    copied first in the forward-only case).  Returns (y, s, y_t, s_t):
+      y [PM, PN] e4m3fn, PN = cdiv(K,256)*256, PM = cdiv(M,4)*4 (cdiv(M,256)*256 when
+      only_forward=False);
+      s logical [PM, PN/128] with strides (1, PM) (column-major, as fp8.py:134,161);
+      with only_forward=False also y_t [PN, PM], the transposed copy quantized per
+      128x128 block, and its scales s_t [PN/128, PM/128]; otherwise None, None.
     """
     if not only_forward:
-        raise NotImplementedError("quant_input(only_forward=False): the backward-pass outputs are not built yet")
+        return _quant_transpose(x, 1, "quant_input")
     if x.dim() != 2:
         raise ValueError("quant_input expects a 2-D tensor")
     if x.dtype != torch.bfloat16:
@@ -124,33 +157,64 @@ def fp8_matmul(qa: torch.Tensor, sa: torch.Tensor, qb: torch.Tensor, sb: torch.T
 
 
 class _DeepLinear(torch.autograd.Function):
-    """Forward of fp8.py:313-328: flatten, quantize input and weight, GEMM, bias, view back.
+    """fp8.py:313-344: forward = flatten, quantize input and weight, GEMM, bias, view back;
+    backward = quantize the output gradient both ways, dgrad = dy . W, wgrad = dy^T . x,
+    both as block-scaled FP8 GEMMs on the transposed copies saved by the forward.
 
-    The bias add is folded into the GEMM epilogue (same fp32 add, one rounding less
-    than GEMM->bf16->add->bf16 only when a bias is present; see `fuse_bias`).
+    The GEMMs run on the unpadded row counts (the quantizers pad rows to 4/128/256, the
+    padding is never multiplied), so shapes that are not multiples of 256 work and no
+    result is sliced.  The bias add can be folded into the GEMM epilogue (`fuse_bias`).
     """
 
     @staticmethod
     def forward(ctx, input, weight, bias, is_grad_enable, weight_cache=None, fuse_bias=False):
         inp_shape = input.shape
         x = input.reshape(-1, input.size(-1))
-        q_inp, s_inp, _, _ = quant_input(x, only_forward=True)
+        M, K = x.shape
+        N = weight.size(0)
+        need_dgrad = bool(is_grad_enable and input.requires_grad)
+        need_wgrad = bool(is_grad_enable and weight.requires_grad)
+        # fp8.py:318: the transposed input copy is only needed for wgrad
+        q_inp, s_inp, q_inp_t, s_inp_t = quant_input(x, only_forward=not need_wgrad)
         if weight_cache is not None:
-            q_weight, s_weight = weight_cache
+            q_weight, s_weight, q_weight_t, s_weight_t = weight_cache
         else:
-            q_weight, s_weight, _, _ = quant_weight(weight, only_forward=True)
-        out = fp8_matmul(q_inp, s_inp, q_weight, s_weight, bias=bias if fuse_bias else None)
+            q_weight, s_weight, q_weight_t, s_weight_t = quant_weight(weight, only_forward=not need_dgrad)
+        if need_dgrad and q_weight_t is None:
+            raise RuntimeError("DeepLinear: the cached weight has no transposed copy but dgrad is required")
+        if is_grad_enable:
+            ctx.inp_shape = inp_shape
+            ctx.dims = (M, N, K)
+            ctx.quantized = (q_inp_t, s_inp_t, q_weight_t, s_weight_t)
+            ctx.has_bias = bias is not None
+        out = fp8_matmul(q_inp[:M], s_inp[:M], q_weight[:N], s_weight[:_cdiv(N, 128)],
+                         bias=bias if fuse_bias else None)
         if bias is not None and not fuse_bias:
             add_bias(out, bias)
-        return out.view(*inp_shape[:-1], -1)
+        return out.view(*inp_shape[:-1], N)
 
     @staticmethod
     def backward(ctx, grad_output):
-        raise NotImplementedError("DeepLinear backward (quant_grad_output + dgrad/wgrad GEMMs) is not built yet")
+        q_inp_t, s_inp_t, q_weight_t, s_weight_t = ctx.quantized
+        M, N, K = ctx.dims
+        dy = grad_output.reshape(-1, N)
+        if dy.dtype != torch.bfloat16:
+            dy = dy.to(torch.bfloat16)
+        q_dy, s_dy, q_dy_t, s_dy_t = quant_grad_output(dy)
+        dgrad = wgrad = grad_bias = None
+        if ctx.needs_input_grad[0]:
+            # [M, PN] . [K, PN]^T, contraction over the (zero-padded) output features
+            dgrad = fp8_matmul(q_dy[:M], s_dy[:M], q_weight_t[:K], s_weight_t[:_cdiv(K, 128)]).view(*ctx.inp_shape)
+        if ctx.needs_input_grad[1]:
+            # [N, PM] . [K, PM]^T, contraction over the (zero-padded) tokens
+            wgrad = fp8_matmul(q_dy_t[:N], s_dy_t[:N], q_inp_t[:K], s_inp_t[:_cdiv(K, 128)])
+        if ctx.has_bias and ctx.needs_input_grad[2]:
+            grad_bias = dy.sum(0)
+        return dgrad, wgrad, grad_bias, None, None, None
 
 
 class DeepLinear(torch.nn.Linear):
-    """nn.Linear whose forward runs the block-wise FP8 path (fp8.py:347-349).
+    """nn.Linear whose forward and backward run the block-wise FP8 path (fp8.py:347-349).
 
     The bf16 master weight is quantized per 128x128 block; the result is cached
     and reused until the weight tensor changes (its version counter or storage),
@@ -162,16 +226,17 @@ class DeepLinear(torch.nn.Linear):
     cache_weight = True
     fuse_bias = False
 
-    def _quantized_weight(self):
+    def _quantized_weight(self, with_transpose: bool):
         w = self.weight
         key = (w.data_ptr(), w._version, tuple(w.shape), w.device)
         cached = getattr(self, "_wq_cache", None)
-        if cached is not None and cached[0] == key:
+        if cached is not None and cached[0] == key and (cached[1][2] is not None or not with_transpose):
             return cached[1]
-        q, s, _, _ = quant_weight(w.detach(), only_forward=True)
-        self._wq_cache = (key, (q, s))
-        return q, s
+        quantized = quant_weight(w.detach(), only_forward=not with_transpose)
+        self._wq_cache = (key, quantized)
+        return quantized
 
     def forward(self, input):
-        cache = self._quantized_weight() if self.cache_weight else None
-        return _DeepLinear.apply(input, self.weight, self.bias, torch.is_grad_enabled(), cache, self.fuse_bias)
+        grad = torch.is_grad_enabled()
+        cache = self._quantized_weight(grad and input.requires_grad) if self.cache_weight else None
+        return _DeepLinear.apply(input, self.weight, self.bias, grad, cache, self.fuse_bias)

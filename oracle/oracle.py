@@ -262,12 +262,37 @@ def fp8_matmul(qa, sa, qb, sb) -> torch.Tensor:
 
 def deep_linear_forward(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
     """Composition of fp8.py:313-328: flatten, quant_input, quant_weight,
-    fp8_matmul, add_bias, view back."""
+    fp8_matmul, add_bias, view back.  Rows and columns the quantizers added as
+    padding are dropped before the bias (the reference's own view only works
+    when there are none: M % 4 == 0 and N % 128 == 0)."""
     shape = x.shape
     x2 = x.reshape(-1, shape[-1])
     qa, sa, _, _ = quant_input(x2, True)
     qb, sb, _, _ = quant_weight(weight, True)
-    out = fp8_matmul(qa, sa, qb, sb)
+    out = fp8_matmul(qa, sa, qb, sb)[:x2.size(0), :weight.size(0)].contiguous()
     if bias is not None:
         out = add_bias(out, bias)
     return out.view(*shape[:-1], -1)
+
+
+def deep_linear_backward(x: torch.Tensor, weight: torch.Tensor, grad_output: torch.Tensor, has_bias: bool = True):
+    """Composition of fp8.py:331-344 on the tensors the forward saved (:318-321):
+    dgrad = fp8_matmul(q(dy), q_t(W)), wgrad = fp8_matmul(q_t(dy), q_t(x)), grad_bias = dy.sum(0).
+
+    The reference multiplies the padded operands and views the result with the input's
+    shape, which only works when no padding was added; here the padded rows and columns
+    are dropped, which is the same thing for shapes that are multiples of 256.
+    """
+    shape = x.shape
+    x2 = x.reshape(-1, shape[-1])
+    M, K = x2.shape
+    N = weight.size(0)
+    dy = grad_output.reshape(-1, N)
+    _, _, q_inp_t, s_inp_t = quant_input(x2, False)
+    _, _, q_w_t, s_w_t = quant_weight(weight, False)
+    q_dy, s_dy, q_dy_t, s_dy_t = quant_grad_output(dy)
+    dgrad = fp8_matmul(q_dy, s_dy, q_w_t, s_w_t)[:M, :K].reshape(shape)
+    wgrad = fp8_matmul(q_dy_t, s_dy_t, q_inp_t, s_inp_t)[:N, :K]
+    # torch's bf16 sum accumulates in fp32 and rounds once (fp8.py:343)
+    grad_bias = dy.detach().cpu().float().sum(0).to(dy.dtype) if has_bias else None
+    return dgrad, wgrad, grad_bias

@@ -23,6 +23,16 @@ def close(got, ref):
     return torch.allclose(got.float().cpu(), ref.float(), rtol=RTOL, atol=ATOL)
 
 
+def close_biased(got, ref, bias):
+    """The GEMM tolerance applied where it belongs when a bias follows: the relative part is taken of the
+    GEMM result before the bias (ref - bias), since a one-ulp difference there survives a cancelling bias."""
+    if bias is None:
+        return close(got, ref)
+    ref = ref.float()
+    mag = torch.maximum(ref.abs(), (ref - bias.float().cpu()).abs())
+    return bool(((got.float().cpu() - ref).abs() <= ATOL + RTOL * mag).all())
+
+
 def quantized_problem(kind, M, N, K, seed):
     x = P.activations(kind, M, K, seed)
     a, a_s = O.act_quant(x)
@@ -193,9 +203,9 @@ def test_deep_linear_forward(shape, N, bias):
         lin.fuse_bias = True
         out_fused = lin(x.to(DEV))
     assert out.shape == (*shape[:-1], N) and out.dtype == torch.bfloat16
-    assert close(out, ref)
+    assert close_biased(out, ref, lin.bias.detach() if bias else None)
     assert torch.equal(out, out_again) and torch.equal(out, out_nocache)
-    assert close(out_fused, ref)
+    assert close_biased(out_fused, ref, lin.bias.detach() if bias else None)
     # sanity band against the unquantized layer (the reference prints ~0.017 mean abs error at d=4096)
     full = torch.nn.functional.linear(x.float(), lin.weight.detach().float().cpu(),
                                       lin.bias.detach().float().cpu() if bias else None)
@@ -210,3 +220,56 @@ def test_deep_linear_cache_follows_weight_updates():
         lin.weight.mul_(2)
         y1 = lin(x)
     assert torch.allclose(y1.float(), 2 * y0.float(), rtol=2e-2, atol=1e-3) and not torch.equal(y0, y1)
+
+
+# ------------------------------------------------------------------ DeepLinear backward
+@pytest.mark.parametrize("bias", [True, False])
+@pytest.mark.parametrize("shape,N", [((2, 128, 256), 256), ((512, 1024), 768), ((3, 50, 300), 200), ((1024, 7168), 1536)])
+def test_deep_linear_backward(shape, N, bias):
+    g = torch.Generator().manual_seed(sum(shape) + N + 1)
+    K = shape[-1]
+    w = (torch.randn(N, K, generator=g) * 0.02).bfloat16()
+    b = torch.randn(N, generator=g).bfloat16() if bias else None
+    x = torch.randn(*shape, generator=g).bfloat16()
+    dy = torch.randn(*shape[:-1], N, generator=g).bfloat16()
+    ref_out = O.deep_linear_forward(x, w, b)
+    ref_dx, ref_dw, ref_db = O.deep_linear_backward(x, w, dy, bias)
+
+    lin = m.DeepLinear(K, N, bias=bias, dtype=torch.bfloat16)
+    with torch.no_grad():
+        lin.weight.copy_(w)
+        if bias:
+            lin.bias.copy_(b)
+    lin = lin.to(DEV)
+    for cache in (True, False):
+        lin.cache_weight = cache
+        lin.zero_grad()
+        xg = x.to(DEV).requires_grad_(True)
+        out = lin(xg)
+        out.backward(dy.to(DEV))
+        assert close_biased(out, ref_out, b)
+        assert xg.grad.shape == x.shape and xg.grad.dtype == torch.bfloat16
+        assert lin.weight.grad.shape == (N, K) and lin.weight.grad.dtype == torch.bfloat16
+        assert close(xg.grad, ref_dx)
+        assert close(lin.weight.grad, ref_dw)
+        if bias:
+            assert torch.allclose(lin.bias.grad.float().cpu(), ref_db.float(), rtol=1e-2, atol=1e-2)
+    # sanity band against the unquantized gradients
+    xf, dyf = x.float().reshape(-1, K), dy.float().reshape(-1, N)
+    dref, wref = (dyf @ w.float()).reshape(x.shape), dyf.t() @ xf
+    assert (xg.grad.float().cpu() - dref).abs().mean() < 0.06 * dref.abs().mean()
+    assert (lin.weight.grad.float().cpu() - wref).abs().mean() < 0.06 * wref.abs().mean()
+
+
+def test_deep_linear_backward_partial_requirements():
+    lin = m.DeepLinear(256, 256, bias=True, dtype=torch.bfloat16, device=DEV)
+    x = torch.randn(64, 256, device=DEV).bfloat16()
+    out = lin(x)                                  # input needs no gradient: only wgrad and grad_bias
+    out.sum().backward()                          # the incoming gradient is an expanded (stride-0) tensor
+    assert lin.weight.grad is not None and lin.bias.grad is not None
+    ref = O.deep_linear_backward(x.cpu(), lin.weight.detach().cpu(), torch.ones(64, 256).bfloat16())
+    assert close(lin.weight.grad, ref[1])
+    lin.weight.requires_grad_(False); lin.bias.requires_grad_(False)
+    xg = x.clone().requires_grad_(True)
+    lin(xg).sum().backward()                      # only dgrad
+    assert close(xg.grad, ref[0])

@@ -171,6 +171,75 @@ def test_quant_input_strided_rows_and_saturation():
     assert torch.equal(s.cpu(), s_ref) and np.array_equal(u8(y), u8(y_ref))
 
 
+# ------------------------------------------------------------------ training-time quantizers
+def _same_quant(got, ref):
+    for g_, r_ in zip(got, ref):
+        assert g_.shape == r_.shape and g_.stride() == r_.stride()
+        if r_.dtype == FP8:
+            assert np.array_equal(u8(g_), u8(r_))
+        else:
+            assert torch.equal(g_.cpu().contiguous(), r_.contiguous())
+
+
+@pytest.mark.parametrize("M,K,seed", [(256, 256, 0), (512, 1024, 1), (130, 300, 2), (1, 7, 3), (4096, 7168, 4),
+                                      (257, 129, 5)])
+def test_quant_input_training_bit_exact(M, K, seed):
+    x = P.activations("outliers", M, K, seed)
+    _same_quant(m.quant_input(x.to(DEV), False), O.quant_input(x, False))
+
+
+@pytest.mark.parametrize("M,N,seed", [(256, 256, 0), (1024, 512, 1), (130, 200, 2), (3, 5, 3), (4096, 1536, 4),
+                                      (385, 127, 5)])
+def test_quant_grad_output_bit_exact(M, N, seed):
+    dy = P.activations("outliers", M, N, seed)
+    _same_quant(m.quant_grad_output(dy.to(DEV)), O.quant_grad_output(dy))
+
+
+def test_training_quantizers_strides_and_saturation():
+    big = P.activations("normal", 300, 1024, 8)
+    big[0, 130] = 3e4; big[5, 131] = -2e4; big[140, 700] = 1.5e4      # beyond the 1e4 clamp: plain division + saturation
+    for view in (lambda t: t[:, 128:128 + 520], lambda t: t.t(), lambda t: t[::2, 1::3], lambda t: t[:1].expand(40, 1024)):
+        x = view(big)
+        for fn_g, fn_o in ((lambda t: m.quant_input(t, False), lambda t: O.quant_input(t, False)),
+                           (m.quant_grad_output, O.quant_grad_output)):
+            got, ref = fn_g(view(big.to(DEV))), fn_o(x)
+            for g_, r_ in zip(got, ref):
+                if r_.dtype == FP8:
+                    assert np.array_equal(u8(g_), u8(r_))
+                else:
+                    assert torch.equal(g_.cpu().contiguous(), r_.contiguous())
+
+
+def test_training_quantizers_ignore_nan_in_the_group_max():
+    """As in the forward quantizer: a NaN element stays NaN in both copies, its row, column and block
+    are scaled by the max of the finite values."""
+    x = P.activations("normal", 256, 256, 13)
+    x[3, 200] = float("nan")
+    xz = x.clone(); xz[3, 200] = 0.0
+    for fn_g, fn_o in ((lambda t: m.quant_input(t, False), lambda t: O.quant_input(t, False)),
+                       (m.quant_grad_output, O.quant_grad_output)):
+        (y, s, y_t, s_t), (y_r, s_r, yt_r, st_r) = fn_g(x.to(DEV)), fn_o(xz)
+        assert torch.equal(s.cpu().contiguous(), s_r.contiguous()) and torch.equal(s_t.cpu().contiguous(), st_r.contiguous())
+        got, got_t = u8(y), u8(y_t)
+        assert (got[3, 200] & 0x7F) == 0x7F and (got_t[200, 3] & 0x7F) == 0x7F
+        got[3, 200] = 0; got_t[200, 3] = 0
+        assert np.array_equal(got, u8(y_r)) and np.array_equal(got_t, u8(yt_r))
+
+
+def test_quant_transpose_abi_rejects_bad_arguments():
+    L = _lib.load()
+    x = torch.zeros(256, 256, dtype=torch.bfloat16, device=DEV)
+    y = torch.empty(256, 256, dtype=torch.uint8, device=DEV)
+    s = torch.empty(2, 256, dtype=torch.float32, device=DEV)
+    args = lambda **kw: [kw.get("x", x.data_ptr()), kw.get("y", y.data_ptr()), s.data_ptr(), kw.get("y_t", y.data_ptr()),
+                         s.data_ptr(), 256, 256, 256, 1, kw.get("PM", 256), kw.get("PK", 256), kw.get("t_mode", 0), None]
+    assert L.mdy_quant_transpose(*args(t_mode=2)) == -4
+    assert L.mdy_quant_transpose(*args(PM=200)) == -2
+    assert L.mdy_quant_transpose(*args(PK=384 + 64)) == -2
+    assert L.mdy_quant_transpose(*args(y_t=None)) == -1
+    assert L.mdy_quant_transpose(*args(y=y.data_ptr() + 4)) == -3
+
+
 # ------------------------------------------------------------------ quant_weight
 @pytest.mark.parametrize("N,K,only_forward,seed", [(1024, 1024, True, 0), (1536, 7168, True, 1), (200, 300, True, 2),
                                                    (200, 300, False, 3), (512, 256, False, 4), (129, 257, False, 5)])

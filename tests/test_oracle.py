@@ -248,3 +248,60 @@ def test_add_bias_and_deep_linear_composition():
     assert (out.float() - ref).abs().mean() < 0.03
     nb = O.deep_linear_forward(x, w, None)
     assert torch.equal(out, O.add_bias(nb, bias))
+
+
+def test_quant_input_training_outputs():
+    # the transposed copy is a 128x128 block quantization: it must coincide with the block weight quantizer's
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(256, 512, generator=g).bfloat16()
+    x[3, 5] = 2e4                                      # beyond the clamp: saturates in both
+    y, s, y_t, s_t = O.quant_input(x, False)
+    y1, s1, _, _ = O.quant_input(x, True)
+    assert np.array_equal(u8(y), u8(y1)) and torch.equal(s.contiguous(), s1.contiguous())
+    _, _, w_t, ws_t = O.quant_weight(x, False)
+    assert tuple(y_t.shape) == (512, 256) and tuple(s_t.shape) == (4, 2)
+    assert np.array_equal(u8(y_t), u8(w_t)) and torch.equal(s_t, ws_t)
+    # ragged: rows padded to 256, padding bytes 0, padded tiles carry the eps scale
+    xr = torch.randn(130, 300, generator=g).bfloat16()
+    y, s, y_t, s_t = O.quant_input(xr, False)
+    assert tuple(y.shape) == (256, 512) and tuple(y_t.shape) == (512, 256) and tuple(s_t.shape) == (4, 2)
+    assert np.all(u8(y_t)[300:] == 0) and np.all(u8(y_t)[:, 130:] == 0)
+    assert s_t[3, 0].item() == np.float32(1e-8) / np.float32(448)
+    # brute force of one tile: block (rows 128..129, cols 256..299)
+    blk = xr.float().numpy()[128:130, 256:300]
+    sc = ((np.abs(blk).max() + np.float32(1e-8)) / np.float32(448)).astype(np.float32)
+    assert s_t[2, 1].item() == sc
+    assert np.array_equal(u8(y_t)[256:300, 128:130], F.encode_rne_sat((blk / sc).astype(np.float32)).T)
+
+
+def test_quant_grad_output_ragged_layout():
+    g = torch.Generator().manual_seed(12)
+    dy = torch.randn(130, 200, generator=g).bfloat16()
+    y, s, y_t, s_t = O.quant_grad_output(dy)
+    assert tuple(y.shape) == (256, 256) and tuple(s.shape) == (256, 2) and s.stride() == (1, 256)
+    assert tuple(y_t.shape) == (256, 256) and tuple(s_t.shape) == (256, 2) and s_t.stride() == (1, 256)
+    d = dy.float().numpy()
+    # column 7, rows 128..129 form one group of the transposed copy
+    col = d[128:130, 7]
+    sc = ((np.abs(col).max() + np.float32(1e-8)) / np.float32(448)).astype(np.float32)
+    assert s_t[7, 1].item() == sc
+    assert np.array_equal(u8(y_t)[7, 128:130], F.encode_rne_sat((col / sc).astype(np.float32)))
+    assert np.all(u8(y_t)[200:] == 0) and np.all(u8(y_t)[:, 130:] == 0)
+
+
+def test_deep_linear_backward_close_to_unquantized_gradients():
+    g = torch.Generator().manual_seed(13)
+    x = torch.randn(2, 128, 256, generator=g).bfloat16()
+    w = (torch.randn(256, 256, generator=g) * 0.05).bfloat16()
+    dy = torch.randn(2, 128, 256, generator=g).bfloat16()
+    dgrad, wgrad, gb = O.deep_linear_backward(x, w, dy)
+    xf = x.float().reshape(-1, 256); dyf = dy.float().reshape(-1, 256)
+    dref = (dyf @ w.float()).reshape(x.shape)
+    wref = dyf.t() @ xf
+    assert tuple(dgrad.shape) == tuple(x.shape) and tuple(wgrad.shape) == (256, 256)
+    assert (dgrad.float() - dref).abs().mean() < 0.05 * dref.abs().mean()
+    assert (wgrad.float() - wref).abs().mean() < 0.05 * wref.abs().mean()
+    assert gb.dtype == torch.bfloat16 and torch.equal(gb, dyf.sum(0).bfloat16())
+    # transposed operands really are transposes: swapping x and dy roles transposes wgrad
+    _, wgrad2, _ = O.deep_linear_backward(dy.reshape(-1, 256), w, x.reshape(-1, 256))
+    assert (wgrad2.float().t() - wref).abs().mean() < 0.05 * wref.abs().mean()
