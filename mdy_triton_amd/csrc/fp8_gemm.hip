@@ -93,7 +93,7 @@ template <int BM, int BN, int WGM, int WGN, typename OUT>
 __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
-    const uint16_t* __restrict__ bias, int M, int N, int K, int tiles_m, int tiles_n) {
+    const uint16_t* __restrict__ bias, int M, int N, int K, int ldc, int tiles_m, int tiles_n) {
     constexpr int WAVES = WGM * WGN;
     constexpr int WM = BM / WGM, WN = BN / WGN, TI = WM / 16, TJ = WN / 16;
     constexpr int PASS_ROWS = WAVES * 8;  // rows copied by one DMA instruction of every wave
@@ -221,7 +221,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
     }
 
     // ---- epilogue: lane holds c[m][n..n+3], m = .. + lane%16, n = .. + 4*(lane/16)
-    const bool vec_ok = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
+    const bool vec_ok = (ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
 #pragma unroll
     for (int i = 0; i < TI; ++i) {
         const int m = m0 + wm * WM + i * 16 + frow;
@@ -234,7 +234,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
                 for (int e = 0; e < 4; ++e)
                     if (n + e < N) v[e] += bf16_one(bias[n + e]);
             }
-            store4<OUT>(c, N, m, n, M, N, v, vec_ok);
+            store4<OUT>(c, ldc, m, n, M, N, v, vec_ok);
         }
     }
 }
@@ -384,12 +384,32 @@ __global__ __launch_bounds__(256) void fp8_gemm_scalar_kernel(const uint8_t* __r
 template <int BM, int BN, int WGM, int WGN, typename OUT>
 static int launch_mfma(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, uint32_t as_bytes,
                        const uint8_t* b, const float* b_s, OUT* c, const uint16_t* bias, int M, int N, int K,
-                       hipStream_t stream) {
+                       int ldc, hipStream_t stream) {
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     dim3 grid((unsigned)(tiles_m * tiles_n)), block(WGM * WGN * 64);
     hipLaunchKernelGGL((fp8_gemm_mfma_kernel<BM, BN, WGM, WGN, OUT>), grid, block, 0, stream, a, a_s, (int)as_rs,
-                       (int)as_cs, as_bytes, b, b_s, c, bias, M, N, K, tiles_m, tiles_n);
+                       (int)as_cs, as_bytes, b, b_s, c, bias, M, N, K, ldc, tiles_m, tiles_n);
     return (int)hipGetLastError();
+}
+
+constexpr int kCUs = 256;   // workgroups of the big tile that run at once (one per CU)
+
+// How many 256-wide tile columns the 256x256 kernel should take when the tile count is not a
+// multiple of the CU count: if the last, partly filled round holds at most half a round of
+// tiles, those columns are better cut into 128x256 tiles (twice as many workgroups, each ~0.6x
+// the time), which fills the machine for one short round instead of half-filling a long one.
+// Returns tiles_n when no split pays.
+static int main_tile_columns(int tiles_m, int tiles_n) {
+    const long total = (long)tiles_m * tiles_n;
+    const long full_rounds = total / kCUs;
+    if (full_rounds < 1 || total % kCUs == 0) return tiles_n;
+    const int cols_main = (int)(full_rounds * kCUs / tiles_m);
+    if (cols_main <= 0 || cols_main >= tiles_n) return tiles_n;
+    const long rounds_main = ((long)cols_main * tiles_m + kCUs - 1) / kCUs;
+    const long rem_small = 2L * (tiles_n - cols_main) * tiles_m;
+    const double cost_split = (double)rounds_main + 0.6 * (double)((rem_small + kCUs - 1) / kCUs);
+    const double cost_plain = (double)((total + kCUs - 1) / kCUs);
+    return cost_split < cost_plain - 0.05 ? cols_main : tiles_n;
 }
 
 template <typename OUT>
@@ -420,9 +440,19 @@ static int dispatch(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t a
         return (int)hipGetLastError();
     }
     const long tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-    if (tiles256 >= 200)
-        return launch_mfma<256, 256, 2, 4, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, stream);
-    return launch_mfma<128, 128, 2, 2, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, stream);
+    if (tiles256 >= 200) {
+        const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
+        const int cols_main = main_tile_columns(tiles_m, tiles_n);
+        const int n_main = cols_main < tiles_n ? cols_main * 256 : N;
+        int rc = launch_mfma<256, 256, 2, 4, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, n_main, K, N,
+                                                  stream);
+        if (rc != 0 || n_main == N) return rc;
+        // remaining columns as 128x256 tiles; n_main is a multiple of 256, so every pointer below keeps its alignment
+        return launch_mfma<128, 256, 2, 4, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b + (size_t)n_main * K,
+                                                b_s + (size_t)(n_main >> 7) * KB, c + n_main,
+                                                bias ? bias + n_main : nullptr, M, N - n_main, K, N, stream);
+    }
+    return launch_mfma<128, 128, 2, 2, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
 }
 
 int launch_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,

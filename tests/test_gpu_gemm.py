@@ -72,6 +72,24 @@ def test_gemm_exact_integer_cases_all_kernels(M, N, K):
     assert torch.equal(got.cpu().double(), c)
 
 
+@pytest.mark.parametrize("M,N,K", [(4000, 4328, 256), (3590, 4608, 384), (4096, 4352, 128)])
+def test_gemm_exact_integer_big_tiles_and_split_launch(M, N, K):
+    """>= 200 tiles of 256x256: the big-tile kernel runs, and because the tile count is not a multiple
+    of the CU count the last tile columns go to a second launch with 128x256 tiles (ragged M and N edges
+    in both)."""
+    test_gemm_exact_integer_cases_all_kernels(M, N, K)
+
+
+def test_gemm_split_launch_with_bias_bf16():
+    M, N, K = 4096, 4352, 256
+    a, a_s, wq, ws = quantized_problem("normal", M, N, K, 21)
+    bias = torch.randn(N, generator=torch.Generator().manual_seed(3)).bfloat16()
+    rows = torch.arange(0, M, 61)
+    ref = O.fp8_gemm(a[rows].contiguous(), a_s[rows].contiguous(), wq, ws, dtype=torch.bfloat16, bias=bias)
+    got = m.fp8_gemm(a.to(DEV), a_s.to(DEV), wq.to(DEV), ws.to(DEV), out_dtype=torch.bfloat16, bias=bias.to(DEV))
+    assert close_biased(got[rows.to(DEV)], ref, bias)
+
+
 @pytest.mark.parametrize("M", [1, 5, 16, 17, 33, 64])
 def test_gemm_small_m_exact(M):
     test_gemm_exact_integer_cases_all_kernels(M, 272, 384)
