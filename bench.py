@@ -269,6 +269,22 @@ def table(torch, m, timer, dev):
              3.0 * N * K + 4.0 * ((N + 127) // 128) * (K // 128), "GB/s", PEAK_HBM_GBS)
         line("%s fp8_gemm %dx%dx%d" % (name, M, N, K), timer.run(lambda: m.fp8_gemm(xq, xs, wq, ws, out_dtype=torch.bfloat16), 10)[0],
              2.0 * M * N * K, "TFLOP/s", PEAK_FP8_TFLOPS)
+    # training-time operators at the C3 shapes (DeepLinear dialect): bytes = 2 in + 1 out + 1 transposed out per element
+    kind, M, N, K, _ = WORKLOADS["C3"]
+    x, w = make_inputs(torch, kind, M, N, K, 2, dev)
+    dy = torch.randn(M, N, device=dev, dtype=torch.bfloat16)
+    line("C3 quant_input(train) %dx%d" % (M, K), timer.run(lambda: m.quant_input(x, False), 20)[0], 4.0 * M * K, "GB/s", PEAK_HBM_GBS)
+    line("C3 quant_grad_output %dx%d" % (M, N), timer.run(lambda: m.quant_grad_output(dy), 20)[0], 4.0 * M * N, "GB/s", PEAK_HBM_GBS)
+    line("C3 quant_weight(train) %dx%d" % (N, K), timer.run(lambda: m.quant_weight(w, False), 20)[0], 4.0 * N * K, "GB/s", PEAK_HBM_GBS)
+    lin = m.DeepLinear(K, N, bias=False, dtype=torch.bfloat16, device=dev)
+    xg = x.clone().requires_grad_(True)
+
+    def train_step():
+        lin.zero_grad(set_to_none=True)
+        xg.grad = None
+        lin(xg).backward(dy)
+    line("C3 DeepLinear fwd+bwd (3 GEMMs + quantizers)", timer.run(train_step, 10)[0], 6.0 * M * N * K, "TFLOP/s", PEAK_FP8_TFLOPS)
+    del lin, xg, dy, x, w
     for M in (1, 16, 64):
         for (N, K) in ((7168, 2048), (2048, 7168)):
             a = torch.randint(0, 120, (M, K), dtype=torch.uint8, device=dev).view(FP8)

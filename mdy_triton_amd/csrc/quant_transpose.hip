@@ -10,11 +10,13 @@
 // max of the rows' clamped+eps maxima, stored ST[pid_n*num_programs(0) + pid_m]).
 //
 // One 256-thread block per 128x128 tile, the tile stays in registers (read once).  Thread t owns
-// columns (t%16)*8..+7 of rows t/16 + 16*i: row maxima by DPP inside 16-lane rows, column maxima by
+// columns (t%16)*8..+7 of the 8 consecutive rows (t/16)*8 + i: row maxima by DPP inside 16-lane rows, column maxima by
 // a per-thread max over its 8 rows followed by an LDS reduction over the 16 row groups.  Quotients
 // use the reciprocal + 2-FMA form (bit-identical to IEEE division for every finite amax in this
 // dialect); groups whose amax exceeds the 1e4 clamp or is not finite divide plainly and clamp.
-// The transposed bytes go through a padded LDS tile so that both outputs are written row-contiguously.
+// Because a thread's rows are consecutive, its 8 bytes of one column are 8 consecutive bytes of a row of the
+// transposed tile: the transpose goes through a padded LDS tile with 8-byte writes and 8-byte reads, and both
+// outputs are written row-contiguously.
 #include "common.h"
 
 namespace mdy {
@@ -45,7 +47,7 @@ __global__ __launch_bounds__(256) void quant_transpose_kernel(const uint16_t* __
     __shared__ float col_part[16][128];   // per row group (t/16) partial column maxima
     __shared__ float col_amax[128];
     __shared__ float blk_part[4];
-    __shared__ __attribute__((aligned(16))) uint8_t tile[128][128 + 16];
+    __shared__ __attribute__((aligned(16))) uint8_t tile[128][128 + 8];   // [k][m], transposed
 
     const int t = threadIdx.x;
     const int lane = t & 63, wave = t >> 6;
@@ -61,7 +63,7 @@ __global__ __launch_bounds__(256) void quant_transpose_kernel(const uint16_t* __
     for (int j = 0; j < 8; ++j) cmax[j] = 0.0f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        const int row = bm * 128 + rg + 16 * i;
+        const int row = bm * 128 + rg * 8 + i;
         uint32_t wd[4] = {0u, 0u, 0u, 0u};
         if (row < M && c0 < K) {
             if (VEC) {
@@ -90,7 +92,7 @@ __global__ __launch_bounds__(256) void quant_transpose_kernel(const uint16_t* __
     // ---- (1) row-wise quantization straight from registers
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        const int row = bm * 128 + rg + 16 * i;     // < PM
+        const int row = bm * 128 + rg * 8 + i;      // < PM
         const float sc = group_scale<1>(rmax[i]);
         const float r = 1.0f / sc;
         float q[8];
@@ -143,6 +145,9 @@ __global__ __launch_bounds__(256) void quant_transpose_kernel(const uint16_t* __
         tr[j] = 1.0f / tsc[j];
         tfast = tfast && (tamax[j] <= 1e4f);
     }
+    uint32_t tb[8][2];   // [column j][rows 0..3 | 4..7] quantized bytes of the transposed copy
+#pragma unroll
+    for (int j = 0; j < 8; ++j) tb[j][0] = tb[j][1] = 0u;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         float q[8];
@@ -153,21 +158,20 @@ __global__ __launch_bounds__(256) void quant_transpose_kernel(const uint16_t* __
 #pragma unroll
             for (int j = 0; j < 8; ++j) q[j] = qt_quot<false>(f[i][j], tsc[j], tr[j]);
         }
-        *reinterpret_cast<uint2*>(&tile[rg + 16 * i][cl]) =
-            make_uint2(pack4_e4m3(q[0], q[1], q[2], q[3]), pack4_e4m3(q[4], q[5], q[6], q[7]));
+        const uint32_t lo = pack4_e4m3(q[0], q[1], q[2], q[3]), hi = pack4_e4m3(q[4], q[5], q[6], q[7]);
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            tb[j][i >> 2] |= (((j < 4 ? lo : hi) >> (8 * (j & 3))) & 0xFFu) << (8 * (i & 3));
     }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) *reinterpret_cast<uint2*>(&tile[cl + j][rg * 8]) = make_uint2(tb[j][0], tb[j][1]);
     __syncthreads();
     // y_t[k][m]: thread owns output columns (t%16)*8..+7 (m) of output rows t/16 + 16*i (k)
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         const int kk = rg + 16 * i;
-        uint32_t lo = 0u, hi = 0u;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            lo |= (uint32_t)tile[cl + j][kk] << (8 * j);
-            hi |= (uint32_t)tile[cl + 4 + j][kk] << (8 * j);
-        }
-        store_nt8(y_t + (int64_t)(bk * 128 + kk) * PM + bm * 128 + cl, make_uint2(lo, hi));
+        const uint2 v = *reinterpret_cast<const uint2*>(&tile[kk][cl]);
+        store_nt8(y_t + (int64_t)(bk * 128 + kk) * PM + bm * 128 + cl, v);
     }
 }
 

@@ -7,11 +7,12 @@
 // (/root/reference/triton_kernels/deepseekv3/fp8_kernel.py:88-122; plain amax/448).
 //
 // One 256-thread block per 128x128 tile.  Thread t owns columns (t%16)*8..+7 of
-// rows t/16 + 16*i, i = 0..7: eight 16-byte loads kept in registers (the tile is
+// rows (t/16)*8 + i, i = 0..7: eight 16-byte loads kept in registers (the tile is
 // read from HBM exactly once), absmax by DPP inside 16-lane rows, ds_swizzle-free
 // cross-row reduction with __shfl_xor, four wave results combined through LDS.
 // The quotient is the same reciprocal + 2-FMA form as the activation quantizer.
-// The transposed copy goes through a padded LDS byte tile.
+// The transposed copy goes through a padded LDS tile: a thread's 8 consecutive rows of one column are 8
+// consecutive bytes of a transposed row (8-byte LDS writes and reads).
 //
 // HBM traffic per element: 2 B in + 1 B out (+ 1 B for the transposed copy).
 #include "common.h"
@@ -24,7 +25,7 @@ __global__ __launch_bounds__(256) void weight_quant_kernel(const uint16_t* __res
                                                             float* __restrict__ s_t, int N, int K, int64_t w_row_stride,
                                                             int64_t w_col_stride, int PN, int PK) {
     __shared__ float wave_max[4];
-    __shared__ __attribute__((aligned(16))) uint8_t tile[128][128 + 16];
+    __shared__ __attribute__((aligned(16))) uint8_t tile[128][128 + 8];   // [k][n], transposed
 
     const int t = threadIdx.x;
     const int lane = t & 63;
@@ -32,13 +33,13 @@ __global__ __launch_bounds__(256) void weight_quant_kernel(const uint16_t* __res
     const int bn = blockIdx.y;  // block row (along N)
     const int bk = blockIdx.x;  // block column (along K)
     const int c0 = bk * 128 + (t & 15) * 8;
-    const int rbase = bn * 128 + (t >> 4);
+    const int rbase = bn * 128 + (t >> 4) * 8;
 
     float f[8][8];
     float m = 0.0f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        const int row = rbase + 16 * i;
+        const int row = rbase + i;
         uint32_t wd[4] = {0u, 0u, 0u, 0u};
         if (row < N && c0 < K) {
             if (VEC) {
@@ -73,6 +74,9 @@ __global__ __launch_bounds__(256) void weight_quant_kernel(const uint16_t* __res
         s[(int64_t)bn * (PK >> 7) + bk] = sc;
         if (s_t) s_t[(int64_t)bk * (PN >> 7) + bn] = sc;
     }
+    uint32_t tb[8][2];   // [column j][rows 0..3 | 4..7] bytes of the transposed copy
+#pragma unroll
+    for (int j = 0; j < 8; ++j) tb[j][0] = tb[j][1] = 0u;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         float q[8];
@@ -92,24 +96,23 @@ __global__ __launch_bounds__(256) void weight_quant_kernel(const uint16_t* __res
         uint2 o;
         o.x = pack4_e4m3(q[0], q[1], q[2], q[3]);
         o.y = pack4_e4m3(q[4], q[5], q[6], q[7]);
-        const int row = rbase + 16 * i;  // < PN because PN % 128 == 0
+        const int row = rbase + i;  // < PN because PN % 128 == 0
         store_nt8(y + (int64_t)row * PK + c0, o);
-        if (y_t) *reinterpret_cast<uint2*>(&tile[(t >> 4) + 16 * i][(t & 15) * 8]) = o;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            tb[j][i >> 2] |= (((j < 4 ? o.x : o.y) >> (8 * (j & 3))) & 0xFFu) << (8 * (i & 3));
     }
     if (y_t) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            *reinterpret_cast<uint2*>(&tile[(t & 15) * 8 + j][(t >> 4) * 8]) = make_uint2(tb[j][0], tb[j][1]);
         __syncthreads();
         // y_t[k][n]: thread owns output columns (t%16)*8..+7 (n) of output rows t/16 + 16*i (k)
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int kk = (t >> 4) + 16 * i;
             const int nn = (t & 15) * 8;
-            uint32_t lo = 0u, hi = 0u;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                lo |= (uint32_t)tile[nn + j][kk] << (8 * j);
-                hi |= (uint32_t)tile[nn + 4 + j][kk] << (8 * j);
-            }
-            store_nt8(y_t + (int64_t)(bk * 128 + kk) * PN + bn * 128 + nn, make_uint2(lo, hi));
+            store_nt8(y_t + (int64_t)(bk * 128 + kk) * PN + bn * 128 + nn, *reinterpret_cast<const uint2*>(&tile[kk][nn]));
         }
     }
 }
