@@ -285,6 +285,16 @@ def table(torch, m, timer, dev):
         lin(xg).backward(dy)
     line("C3 DeepLinear fwd+bwd (3 GEMMs + quantizers)", timer.run(train_step, 10)[0], 6.0 * M * N * K, "TFLOP/s", PEAK_FP8_TFLOPS)
     del lin, xg, dy, x, w
+    # SwiGLU in front of the MLP-down quantizer (C4's activation): fused vs the reference's two passes
+    Ms, Ns = 4096, 18432
+    ug = (torch.randn(Ms, 2 * Ns, device=dev) * 1.5).to(torch.bfloat16)
+    line("C4 silu_act_quant fused %dx%d" % (Ms, Ns), timer.run(lambda: m.silu_act_quant(ug), 20)[0], 5.03125 * Ms * Ns, "GB/s", PEAK_HBM_GBS)
+
+    def unfused():
+        m.act_quant(m.silu_fwd(ug))
+    line("C4 silu_fwd + act_quant (2 passes) %dx%d" % (Ms, Ns), timer.run(unfused, 20)[0], 9.03125 * Ms * Ns, "GB/s", PEAK_HBM_GBS)
+    line("C4 silu_fwd %dx%d" % (Ms, Ns), timer.run(lambda: m.silu_fwd(ug), 20)[0], 6.0 * Ms * Ns, "GB/s", PEAK_HBM_GBS)
+    del ug
     for M in (1, 16, 64):
         for (N, K) in ((7168, 2048), (2048, 7168)):
             a = torch.randint(0, 120, (M, K), dtype=torch.uint8, device=dev).view(FP8)

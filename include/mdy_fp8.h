@@ -100,6 +100,33 @@ int mdy_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t,
                         int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int t_mode,
                         void* stream);
 
+/* SwiGLU, alone or fused with the 1x128 activation quantizer that feeds the next GEMM.
+ *   act[m, n] = bf16( silu(gate[m, n]) * up[m, n] ), silu(g) = g / (1 + exp(-g)) in fp32;
+ *   (y, s)    = 1x128 quantization of act (the bf16-rounded value) as mdy_act_quant would produce it.
+ * Replaces silu_fwd (triton_kernels/deepseekv3/fp8_kernel.py:384-402, kernel :315-344; the same kernel
+ * is triton_kernels/megatron_patchs/swiglu.py:6-36) and the silu_fwd + act_quant pair of the FP8 MLP
+ * (fp8_kernel.py:447-450, 500-515) in one pass.
+ *
+ *   x    bf16 [M, 2N], row m at x + m * x_row_stride; gate_first = 0: columns [0,N) are `up` and [N,2N)
+ *        `gate` (the reference's order 'up-gate'); gate_first = 1: the other way round ('gate-up')
+ *   act  bf16 [M, N] row-major or NULL
+ *   y    e4m3fn [PM, PN] row-major or NULL (then s, PM, PN, strides and mode are ignored);
+ *        PM >= M, PN >= N, PN % 128 == 0, padding quantizes as 0
+ *   s    fp32, scale of (row m, group kb) at s[m * s_row_stride + kb * s_col_stride]
+ *   mode MDY_QUANT_OFFICIAL or MDY_QUANT_DEEPLINEAR
+ * At least one of act, y must be given.
+ */
+int mdy_swiglu(const void* x, void* act, void* y, float* s, int64_t M, int64_t N, int64_t x_row_stride,
+               int gate_first, int64_t PM, int64_t PN, int64_t s_row_stride, int64_t s_col_stride, int mode,
+               void* stream);
+
+/* Backward of SwiGLU: dx[m, up] = silu(gate) * dy, dx[m, gate] = (sig + silu * (1 - sig)) * up * dy.
+ * Replaces silu_bwd (fp8_kernel.py:404-421, kernel :346-382).
+ *   x bf16 [M, 2N] (row stride x_row_stride), dy bf16 [M, N] row-major, dx bf16 [M, 2N] row-major.
+ */
+int mdy_swiglu_bwd(const void* x, const void* dy, void* dx, int64_t M, int64_t N, int64_t x_row_stride,
+                   int gate_first, void* stream);
+
 /* 128x128 block weight dequantizer: y[n,k] = fp32(x[n,k]) * s[n/128, k/128].
  * Replaces weight_dequant (offical_kernel.py:46-53, kernel :31-43).
  *   x e4m3fn [N, K] row-major; s fp32 [ceil(N/128), ceil(K/128)] row-major;

@@ -5,5 +5,7 @@ operator call does, and raises if it has not been built."""
 from .offical_kernel import act_quant, fp8_gemm, weight_dequant  # noqa: F401
 from .fp8 import DeepLinear, add_bias, fp8_matmul, quant_grad_output, quant_input, quant_weight  # noqa: F401
 
-__all__ = ["act_quant", "weight_dequant", "fp8_gemm", "quant_input", "quant_weight", "quant_grad_output", "fp8_matmul", "add_bias",
+from .fp8_kernel import silu_act_quant, silu_bwd, silu_fwd, triton_silu, weight_quant_block  # noqa: F401
+
+__all__ = ["silu_fwd", "silu_bwd", "triton_silu", "silu_act_quant", "weight_quant_block", "act_quant", "weight_dequant", "fp8_gemm", "quant_input", "quant_weight", "quant_grad_output", "fp8_matmul", "add_bias",
            "DeepLinear"]

@@ -106,6 +106,44 @@ int mdy_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t,
                     "quant_transpose");
 }
 
+int mdy_swiglu(const void* x, void* act, void* y, float* s, int64_t M, int64_t N, int64_t x_row_stride, int gate_first,
+               int64_t PM, int64_t PN, int64_t s_row_stride, int64_t s_col_stride, int mode, void* stream) {
+    if (M < 0 || N < 0 || M > kMaxDim || 2 * N > kMaxDim) return fail(MDY_E_SHAPE, "swiglu: bad shape M=%lld N=%lld", (long long)M, (long long)N);
+    if (!act && !y) return fail(MDY_E_NULL, "swiglu: neither act nor y given");
+    if (y) {
+        if (mode != MDY_QUANT_OFFICIAL && mode != MDY_QUANT_DEEPLINEAR) return fail(MDY_E_DTYPE, "swiglu: unknown mode %d", mode);
+        if (PM < M || PN < N || PM > kMaxDim || PN > kMaxDim) return fail(MDY_E_SHAPE, "swiglu: need M <= PM, N <= PN");
+        if (PN % 128 != 0) return fail(MDY_E_SHAPE, "swiglu: PN=%lld is not a multiple of 128", (long long)PN);
+        if (PM == 0 || PN == 0) return 0;
+        if (!s) return fail(MDY_E_NULL, "swiglu: y given without s");
+        if (!aligned(y, 8) || !aligned(s, 4)) return fail(MDY_E_ALIGN, "swiglu: y must be 8-byte, s 4-byte aligned");
+        if ((PM + 7) / 8 > 65535) return fail(MDY_E_SHAPE, "swiglu: PM too large");
+    } else {
+        if (M == 0 || N == 0) return 0;
+        if ((M + 7) / 8 > 65535) return fail(MDY_E_SHAPE, "swiglu: M too large");
+    }
+    if (!x && M > 0 && N > 0) return fail(MDY_E_NULL, "swiglu: null x");
+    if (M > 0 && x_row_stride < 2 * N) return fail(MDY_E_SHAPE, "swiglu: x_row_stride=%lld < 2N=%lld", (long long)x_row_stride, (long long)(2 * N));
+    if (!aligned(x, 2) || (act && !aligned(act, 2))) return fail(MDY_E_ALIGN, "swiglu: x/act misaligned for bf16");
+    if (int e = check_device()) return e;
+    return launched(mdy::launch_swiglu(x, act, y, s, M, N, x_row_stride, gate_first != 0, PM, PN, s_row_stride, s_col_stride,
+                                       mode, static_cast<hipStream_t>(stream)),
+                    "swiglu");
+}
+
+int mdy_swiglu_bwd(const void* x, const void* dy, void* dx, int64_t M, int64_t N, int64_t x_row_stride, int gate_first,
+                   void* stream) {
+    if (M < 0 || N < 0 || M > kMaxDim || 2 * N > kMaxDim) return fail(MDY_E_SHAPE, "swiglu_bwd: bad shape");
+    if ((M + 7) / 8 > 65535) return fail(MDY_E_SHAPE, "swiglu_bwd: M too large");
+    if (M == 0 || N == 0) return 0;
+    if (!x || !dy || !dx) return fail(MDY_E_NULL, "swiglu_bwd: null pointer");
+    if (x_row_stride < 2 * N) return fail(MDY_E_SHAPE, "swiglu_bwd: x_row_stride < 2N");
+    if (!aligned(x, 2) || !aligned(dy, 2) || !aligned(dx, 2)) return fail(MDY_E_ALIGN, "swiglu_bwd: misaligned pointer");
+    if (int e = check_device()) return e;
+    return launched(mdy::launch_swiglu_bwd(x, dy, dx, M, N, x_row_stride, gate_first != 0, static_cast<hipStream_t>(stream)),
+                    "swiglu_bwd");
+}
+
 int mdy_weight_dequant(const void* x, const float* s, void* y, int64_t N, int64_t K, int out_dtype, void* stream) {
     if (out_dtype != MDY_DT_BF16 && out_dtype != MDY_DT_F32) return fail(MDY_E_DTYPE, "weight_dequant: unknown out_dtype %d", out_dtype);
     if (N < 0 || K < 0 || N > kMaxDim || K > kMaxDim) return fail(MDY_E_SHAPE, "weight_dequant: bad shape");

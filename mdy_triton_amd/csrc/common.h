@@ -105,6 +105,11 @@ int launch_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t,
 int launch_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
                            int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int t_mode,
                            hipStream_t stream);
+int launch_swiglu(const void* x, void* act, void* y, float* s, int64_t M, int64_t N, int64_t x_row_stride,
+                  int gate_first, int64_t PM, int64_t PN, int64_t s_row_stride, int64_t s_col_stride, int mode,
+                  hipStream_t stream);
+int launch_swiglu_bwd(const void* x, const void* dy, void* dx, int64_t M, int64_t N, int64_t x_row_stride,
+                      int gate_first, hipStream_t stream);
 int launch_weight_dequant(const void* x, const float* s, void* y, int64_t N, int64_t K, int out_dtype,
                           hipStream_t stream);
 int launch_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,

@@ -296,3 +296,38 @@ def deep_linear_backward(x: torch.Tensor, weight: torch.Tensor, grad_output: tor
     # torch's bf16 sum accumulates in fp32 and rounds once (fp8.py:343)
     grad_bias = dy.detach().cpu().float().sum(0).to(dy.dtype) if has_bias else None
     return dgrad, wgrad, grad_bias
+
+
+# ----------------------------------------------------------------------------
+# SwiGLU before the down projection (floating point: compared with a tolerance)
+# ----------------------------------------------------------------------------
+def _split_up_gate(x: torch.Tensor, order: str):
+    assert order in ("up-gate", "gate-up")
+    N = x.size(-1) // 2
+    xf = x.detach().cpu().float()
+    first, second = xf[..., :N], xf[..., N:]
+    return (first, second) if order == "up-gate" else (second, first)     # fp8_kernel.py:327-332
+
+
+def silu_fwd(x: torch.Tensor, order: str = "up-gate") -> torch.Tensor:
+    """y = (gate * sigmoid(gate)) * up in fp32, rounded once to x.dtype (fp8_kernel.py:335-344)."""
+    up, gate = _split_up_gate(x, order)
+    return ((gate * torch.sigmoid(gate)) * up).to(x.dtype)
+
+
+def silu_bwd(dy: torch.Tensor, x: torch.Tensor, order: str = "up-gate") -> torch.Tensor:
+    """fp8_kernel.py:369-382: dup = act*dy, dgate = (sig + act*(1-sig)) * (up*dy), each rounded to dy.dtype."""
+    up, gate = _split_up_gate(x, order)
+    d = dy.detach().cpu().float().reshape(up.shape)
+    sig = torch.sigmoid(gate)
+    act = sig * gate
+    dup = (act * d).to(dy.dtype)
+    dgate = ((sig + act * (1 - sig)) * (up * d)).to(dy.dtype)
+    return torch.cat([dup, dgate] if order == "up-gate" else [dgate, dup], dim=-1)
+
+
+def silu_act_quant(x: torch.Tensor, order: str = "up-gate"):
+    """The unfused pair of the FP8 MLP (fp8_kernel.py:447-450): act = silu_fwd(x); act_quant(act)."""
+    act = silu_fwd(x, order)
+    y, s = act_quant(act.contiguous())
+    return y, s, act

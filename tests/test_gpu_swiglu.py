@@ -1,0 +1,114 @@
+"""GPU parity of SwiGLU and of its fusion with the activation quantizer.
+
+silu is floating point (exp / reciprocal differ between implementations by about one fp32 ulp), so the
+bf16 activation is compared with the CPU oracle to within one bf16 ulp (rtol 2^-7) and the two must agree
+bit for bit on all but a small fraction of elements; the quantizer part of the fused kernel is integer-exact:
+its bytes and scales must equal the oracle quantizer applied to the kernel's own bf16 activation."""
+import numpy as np
+import pytest
+import torch
+
+import mdy_triton_amd as m
+from mdy_triton_amd import _lib
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+FP8 = torch.float8_e4m3fn
+ULP = 2.0 ** -7      # one bf16 ulp, relative
+
+
+def u8(t):
+    return t.contiguous().view(torch.uint8).cpu().numpy()
+
+
+def up_gate(M, N2, seed, scale=2.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(M, N2, generator=g) * scale).bfloat16()
+
+
+def within_ulp(got, ref, ulps=1):
+    got, ref = got.float().cpu(), ref.float()
+    ok = (got - ref).abs() <= ulps * ULP * ref.abs() + 1e-30
+    same = (got == ref) | (got.isnan() & ref.isnan())
+    return bool((ok | same).all()), float((~same).float().mean())
+
+
+@pytest.mark.parametrize("order", ["up-gate", "gate-up"])
+@pytest.mark.parametrize("M,N2", [(128, 512), (37, 1000), (4096, 4096), (5, 22)])
+def test_silu_fwd(M, N2, order):
+    x = up_gate(M, N2, M + N2)
+    ok, frac = within_ulp(m.silu_fwd(x.to(DEV), order), O.silu_fwd(x, order))
+    assert ok and frac < 2e-3
+
+
+def test_silu_fwd_leading_dims_strides_and_extremes():
+    x = up_gate(6 * 8, 512, 3).reshape(6, 8, 512)
+    x[0, 0, :8] = torch.tensor([0.0, -0.0, 80.0, -80.0, 1e4, -1e4, 3e38, -3e38]).bfloat16()
+    x[0, 0, 256:264] = torch.tensor([5.0, -5.0, 100.0, -100.0, -200.0, 200.0, 1.0, -1.0]).bfloat16()
+    got = m.silu_fwd(x.to(DEV))
+    assert got.shape == (6, 8, 256)
+    ok, frac = within_ulp(got, O.silu_fwd(x))
+    assert ok
+    big = up_gate(40, 1024, 4)
+    ok, _ = within_ulp(m.silu_fwd(big.to(DEV)[:, 256:768]), O.silu_fwd(big[:, 256:768]))     # row stride 1024
+    assert ok
+    assert m.silu_fwd(torch.empty(0, 256, dtype=torch.bfloat16, device=DEV)).shape == (0, 128)
+
+
+@pytest.mark.parametrize("order", ["up-gate", "gate-up"])
+@pytest.mark.parametrize("M,N2", [(128, 512), (33, 600), (2048, 4096)])
+def test_silu_bwd_and_autograd(M, N2, order):
+    x = up_gate(M, N2, M + 7)
+    dy = up_gate(M, N2 // 2, M + 8, 1.0)
+    ok, frac = within_ulp(m.silu_bwd(dy.to(DEV), x.to(DEV), order), O.silu_bwd(dy, x, order), ulps=2)
+    assert ok and frac < 5e-3
+    xg = x.to(DEV).requires_grad_(True)
+    m.triton_silu(xg, order).backward(dy.to(DEV))
+    ok, _ = within_ulp(xg.grad, O.silu_bwd(dy, x, order), ulps=2)
+    assert ok
+
+
+@pytest.mark.parametrize("order", ["up-gate", "gate-up"])
+@pytest.mark.parametrize("M,N2", [(128, 512), (4096, 2 * 2048), (3, 256), (100, 2 * 18432)])
+def test_silu_act_quant_official(M, N2, order):
+    x = up_gate(M, N2, M + N2 + 1)
+    y, s, act = m.silu_act_quant(x.to(DEV), order, return_act=True)
+    ok, frac = within_ulp(act, O.silu_fwd(x, order))
+    assert ok and frac < 2e-3
+    y_ref, s_ref = O.act_quant(act.cpu())                       # the quantizer part is exact
+    assert torch.equal(s.cpu(), s_ref) and np.array_equal(u8(y), u8(y_ref))
+    y2, s2 = m.silu_act_quant(x.to(DEV), order)                 # same bytes when the activation is not written
+    assert torch.equal(y2.view(torch.uint8), y.view(torch.uint8)) and torch.equal(s2, s)
+    assert torch.equal(act, m.silu_fwd(x.to(DEV), order))
+    # against the fully unfused oracle: scales within one bf16 ulp of the group maximum
+    _, s_o, _ = O.silu_act_quant(x, order)
+    assert torch.allclose(s.cpu(), s_o, rtol=ULP, atol=0)
+
+
+def test_silu_act_quant_deeplinear_layout_and_zero_groups():
+    x = up_gate(6, 2 * 300, 11)
+    y, s, act = m.silu_act_quant(x.to(DEV), return_act=True, dialect="deeplinear")
+    y_ref, s_ref, _, _ = O.quant_input(act.cpu(), True)
+    assert y.shape == y_ref.shape == (8, 512) and s.shape == s_ref.shape and s.stride() == s_ref.stride()
+    assert torch.equal(s.cpu(), s_ref) and np.array_equal(u8(y), u8(y_ref))
+    # an all-zero group in the official dialect: s = 0, bytes NaN (as act_quant)
+    z = torch.zeros(2, 512, dtype=torch.bfloat16)
+    yz, sz = m.silu_act_quant(z.to(DEV))
+    assert torch.count_nonzero(sz) == 0 and np.all((u8(yz) & 0x7F) == 0x7F)
+
+
+def test_swiglu_abi_rejects_bad_arguments():
+    L = _lib.load()
+    x = torch.zeros(8, 512, dtype=torch.bfloat16, device=DEV)
+    act = torch.empty(8, 256, dtype=torch.bfloat16, device=DEV)
+    y = torch.empty(8, 256, dtype=torch.uint8, device=DEV)
+    s = torch.empty(8, 2, dtype=torch.float32, device=DEV)
+    assert L.mdy_swiglu(x.data_ptr(), None, None, None, 8, 256, 512, 0, 0, 0, 0, 0, 0, None) == -1
+    assert L.mdy_swiglu(x.data_ptr(), None, y.data_ptr(), None, 8, 256, 512, 0, 8, 256, 2, 1, 0, None) == -1
+    assert L.mdy_swiglu(x.data_ptr(), None, y.data_ptr(), s.data_ptr(), 8, 256, 512, 0, 8, 200, 2, 1, 0, None) == -2
+    assert L.mdy_swiglu(x.data_ptr(), None, y.data_ptr(), s.data_ptr(), 8, 256, 512, 0, 8, 256, 2, 1, 7, None) == -4
+    assert L.mdy_swiglu(x.data_ptr(), act.data_ptr(), None, None, 8, 256, 500, 0, 0, 0, 0, 0, 0, None) == -2
+    assert L.mdy_swiglu_bwd(x.data_ptr(), None, x.data_ptr(), 8, 256, 512, 0, None) == -1
+    with pytest.raises(AssertionError):
+        m.silu_fwd(x, "gate_up")

@@ -305,3 +305,26 @@ def test_deep_linear_backward_close_to_unquantized_gradients():
     # transposed operands really are transposes: swapping x and dy roles transposes wgrad
     _, wgrad2, _ = O.deep_linear_backward(dy.reshape(-1, 256), w, x.reshape(-1, 256))
     assert (wgrad2.float().t() - wref).abs().mean() < 0.05 * wref.abs().mean()
+
+
+def test_silu_matches_torch_functional_and_autograd():
+    g = torch.Generator().manual_seed(14)
+    x = (torch.randn(16, 512, generator=g) * 2).bfloat16()
+    for order in ("up-gate", "gate-up"):
+        up, gate = (x[:, :256], x[:, 256:]) if order == "up-gate" else (x[:, 256:], x[:, :256])
+        ref = (torch.nn.functional.silu(gate.float()) * up.float())
+        act = O.silu_fwd(x, order)
+        assert act.dtype == torch.bfloat16 and (act.float() - ref).abs().max() <= 2.0 ** -8 * ref.abs().max()
+        xf = x.float().requires_grad_(True)
+        upf, gatef = (xf[:, :256], xf[:, 256:]) if order == "up-gate" else (xf[:, 256:], xf[:, :256])
+        dy = torch.randn(16, 256, generator=g).bfloat16()
+        (torch.nn.functional.silu(gatef) * upf).backward(dy.float())
+        dx = O.silu_bwd(dy, x, order)
+        assert (dx.float() - xf.grad).abs().max() <= 2.0 ** -7 * xf.grad.abs().max()
+    y, s, act = O.silu_act_quant(x)
+    y2, s2 = O.act_quant(act)
+    assert torch.equal(s, s2) and np.array_equal(u8(y), u8(y2))
+    # closed forms: silu(0) = 0, silu(large) = identity, silu(-large) = -large * exp(-large)
+    e = torch.tensor([[1.0, 1.0, 1.0, 0.0, 60.0, -60.0]]).bfloat16()
+    got = O.silu_fwd(e).tolist()[0]
+    assert got[:2] == [0.0, 60.0] and abs(got[2] / (-60.0 * np.exp(-60.0)) - 1) < 2.0 ** -8
