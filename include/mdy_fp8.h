@@ -87,7 +87,9 @@ int mdy_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t, in
  *
  *   x    bf16 [M, K], element (m, k) at x[m * x_row_stride + k * x_col_stride]
  *   y    e4m3fn [PM, PK] row-major, PM % 128 == 0, PK % 128 == 0, padding reads as 0
- *   s    fp32, scale of row m, K-group kb at s[kb * PM + m]          ([PK/128, PM] row-major)
+ *   s    fp32, scale of row m, K-group kb at s[kb * s_kb_stride + m]; s_kb_stride >= PM (= PM for the
+ *        [PK/128, PM] buffer of quant_input / quant_grad_output; the total row count when the rows are one
+ *        expert group of a larger matrix, group_per_token_cast_to_fp8 at megatron_patchs/fp8_matmul.py:218-247)
  *   y_t  e4m3fn [PK, PM] row-major: y_t[k, m] = x[m, k] / scale_t
  *   s_t  MDY_T_COLUMN: one scale per column k and 128-row group a, at s_t[a * PK + k]
  *                      ([PM/128, PK] row-major; the reference returns its transpose view)
@@ -97,8 +99,8 @@ int mdy_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t, in
 #define MDY_T_COLUMN 0
 #define MDY_T_BLOCK 1
 int mdy_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
-                        int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int t_mode,
-                        void* stream);
+                        int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int64_t s_kb_stride,
+                        int t_mode, void* stream);
 
 /* SwiGLU, alone or fused with the 1x128 activation quantizer that feeds the next GEMM.
  *   act[m, n] = bf16( silu(gate[m, n]) * up[m, n] ), silu(g) = g / (1 + exp(-g)) in fp32;
@@ -152,6 +154,26 @@ int mdy_weight_dequant(const void* x, const float* s, void* y, int64_t N, int64_
 int mdy_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
                     const void* b, const float* b_s, void* c, const void* bias, int64_t M, int64_t N,
                     int64_t K, int out_dtype, void* stream);
+
+/* Grouped (mixture-of-experts) block-scaled FP8 GEMM, NT layout: the rows of a are split into G
+ * consecutive groups of m_splits[g] rows and group g is multiplied with its own weight,
+ *   c[m, n] = sum_kb (sum_{k in kb} a[m,k] * b[g,n,k]) * a_s[m,kb] * b_s[g, n/128, kb]  (+ bias[g, n])
+ * for the rows m of group g.  Replaces fp8_grouped_matmul
+ * (triton_kernels/megatron_patchs/fp8_matmul.py:400-413, i.e.
+ * deep_gemm.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous with the per-row group index built from m_splits).
+ * Group sizes need no alignment (the reference pads them to 256 rows; zero-sized groups are allowed).
+ *
+ *   a        e4m3fn [M, K] row-major, M = sum of m_splits      a_s as in mdy_fp8_gemm_nt
+ *   b        e4m3fn [G, N, K] row-major                        b_s fp32 [G, ceil(N/128), ceil(K/128)]
+ *   c        [M, N] row-major of out_dtype                     bias bf16 [G, N] or NULL
+ *   m_splits HOST pointer to G non-negative row counts (read before the call returns); G <= 256 for
+ *            the single-launch MFMA path, larger G or K % 128 != 0 / unaligned operands run one launch
+ *            per group.
+ */
+int mdy_fp8_grouped_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
+                            const void* b, const float* b_s, void* c, const void* bias,
+                            const int64_t* m_splits, int64_t G, int64_t N, int64_t K, int out_dtype,
+                            void* stream);
 
 /* In-place x[m, :] = bf16(fp32(x[m, :]) + fp32(b)) on bf16 x [M, N] row-major, bf16 b [N].
  * Replaces add_bias (fp8.py:297-305, kernel :283-295). */

@@ -7,5 +7,8 @@ from .fp8 import DeepLinear, add_bias, fp8_matmul, quant_grad_output, quant_inpu
 
 from .fp8_kernel import silu_act_quant, silu_bwd, silu_fwd, triton_silu, weight_quant_block  # noqa: F401
 
-__all__ = ["silu_fwd", "silu_bwd", "triton_silu", "silu_act_quant", "weight_quant_block", "act_quant", "weight_dequant", "fp8_gemm", "quant_input", "quant_weight", "quant_grad_output", "fp8_matmul", "add_bias",
+from .megatron_patchs.fp8_matmul import (fp8_grouped_matmul, group_per_token_cast_to_fp8, per_block_cast_to_fp8,  # noqa: F401
+                         per_token_cast_to_fp8)
+
+__all__ = ["per_token_cast_to_fp8", "group_per_token_cast_to_fp8", "per_block_cast_to_fp8", "fp8_grouped_matmul", "silu_fwd", "silu_bwd", "triton_silu", "silu_act_quant", "weight_quant_block", "act_quant", "weight_dequant", "fp8_gemm", "quant_input", "quant_weight", "quant_grad_output", "fp8_matmul", "add_bias",
            "DeepLinear"]

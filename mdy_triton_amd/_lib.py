@@ -23,7 +23,8 @@ _int = ctypes.c_int
 SIGNATURES = {
     "mdy_act_quant": [_p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p],
     "mdy_weight_quant": [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p],
-    "mdy_quant_transpose": [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p],
+    "mdy_quant_transpose": [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p],
+    "mdy_fp8_grouped_gemm_nt": [_p, _p, _i64, _i64, _p, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p],
     "mdy_swiglu": [_p, _p, _p, _p, _i64, _i64, _i64, _int, _i64, _i64, _i64, _i64, _int, _p],
     "mdy_swiglu_bwd": [_p, _p, _p, _i64, _i64, _i64, _int, _p],
     "mdy_weight_dequant": [_p, _p, _p, _i64, _i64, _int, _p],

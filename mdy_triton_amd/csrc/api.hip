@@ -90,18 +90,20 @@ int mdy_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t, in
 }
 
 int mdy_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
-                        int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int t_mode, void* stream) {
+                        int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int64_t s_kb_stride, int t_mode,
+                        void* stream) {
     if (t_mode != MDY_T_COLUMN && t_mode != MDY_T_BLOCK) return fail(MDY_E_DTYPE, "quant_transpose: unknown t_mode %d", t_mode);
     if (M < 0 || K < 0 || PM < M || PK < K || PM > kMaxDim || PK > kMaxDim)
         return fail(MDY_E_SHAPE, "quant_transpose: need 0 <= M <= PM, 0 <= K <= PK");
     if (PM % 128 != 0 || PK % 128 != 0) return fail(MDY_E_SHAPE, "quant_transpose: PM=%lld, PK=%lld must be multiples of 128", (long long)PM, (long long)PK);
     if (PM / 128 > 65535) return fail(MDY_E_SHAPE, "quant_transpose: PM too large");
+    if (s_kb_stride < PM) return fail(MDY_E_SHAPE, "quant_transpose: s_kb_stride=%lld < PM=%lld", (long long)s_kb_stride, (long long)PM);
     if (PM == 0 || PK == 0) return 0;
     if (!y || !s || !y_t || !s_t || (!x && M > 0 && K > 0)) return fail(MDY_E_NULL, "quant_transpose: null pointer");
     if (!aligned(y, 8) || !aligned(y_t, 8)) return fail(MDY_E_ALIGN, "quant_transpose: y / y_t must be 8-byte aligned");
     if (!aligned(x, 2) || !aligned(s, 4) || !aligned(s_t, 4)) return fail(MDY_E_ALIGN, "quant_transpose: x/s/s_t misaligned for their element type");
     if (int e = check_device()) return e;
-    return launched(mdy::launch_quant_transpose(x, y, s, y_t, s_t, M, K, x_row_stride, x_col_stride, PM, PK, t_mode,
+    return launched(mdy::launch_quant_transpose(x, y, s, y_t, s_t, M, K, x_row_stride, x_col_stride, PM, PK, s_kb_stride, t_mode,
                                                 static_cast<hipStream_t>(stream)),
                     "quant_transpose");
 }
@@ -170,6 +172,30 @@ int mdy_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int6
     return launched(mdy::launch_fp8_gemm_nt(a, a_s, as_row_stride, as_col_stride, b, b_s, c, bias, M, N, K, out_dtype,
                                             static_cast<hipStream_t>(stream)),
                     "fp8_gemm_nt");
+}
+
+int mdy_fp8_grouped_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,
+                            const float* b_s, void* c, const void* bias, const int64_t* m_splits, int64_t G, int64_t N,
+                            int64_t K, int out_dtype, void* stream) {
+    if (out_dtype != MDY_DT_BF16 && out_dtype != MDY_DT_F32) return fail(MDY_E_DTYPE, "fp8_grouped_gemm_nt: unknown out_dtype %d", out_dtype);
+    if (G < 0 || G > (1 << 20) || N < 0 || K < 1 || N > kMaxDim || K > kMaxDim)
+        return fail(MDY_E_SHAPE, "fp8_grouped_gemm_nt: bad shape G=%lld N=%lld K=%lld", (long long)G, (long long)N, (long long)K);
+    if (G == 0 || N == 0) return 0;
+    if (!m_splits) return fail(MDY_E_NULL, "fp8_grouped_gemm_nt: null m_splits");
+    int64_t M = 0;
+    for (int64_t g = 0; g < G; ++g) {
+        if (m_splits[g] < 0 || m_splits[g] > kMaxDim) return fail(MDY_E_SHAPE, "fp8_grouped_gemm_nt: m_splits[%lld]=%lld", (long long)g, (long long)m_splits[g]);
+        M += m_splits[g];
+    }
+    if (M > kMaxDim || (M + 15) / 16 > 65535 * 16) return fail(MDY_E_SHAPE, "fp8_grouped_gemm_nt: too many rows (%lld)", (long long)M);
+    if (M == 0) return 0;
+    if (!a || !a_s || !b || !b_s || !c) return fail(MDY_E_NULL, "fp8_grouped_gemm_nt: null pointer");
+    if (!aligned(c, out_dtype == MDY_DT_BF16 ? 2 : 4) || !aligned(a_s, 4) || !aligned(b_s, 4) || (bias && !aligned(bias, 2)))
+        return fail(MDY_E_ALIGN, "fp8_grouped_gemm_nt: misaligned pointer");
+    if (int e = check_device()) return e;
+    return launched(mdy::launch_fp8_grouped_gemm_nt(a, a_s, as_row_stride, as_col_stride, b, b_s, c, bias, m_splits, G, M, N, K,
+                                                    out_dtype, static_cast<hipStream_t>(stream)),
+                    "fp8_grouped_gemm_nt");
 }
 
 int mdy_add_bias(void* x, const void* b, int64_t M, int64_t N, void* stream) {

@@ -103,8 +103,8 @@ int launch_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t,
                         int64_t w_row_stride, int64_t w_col_stride, int64_t PN, int64_t PK, int mode,
                         hipStream_t stream);
 int launch_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
-                           int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int t_mode,
-                           hipStream_t stream);
+                           int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int64_t s_kb_stride,
+                           int t_mode, hipStream_t stream);
 int launch_swiglu(const void* x, void* act, void* y, float* s, int64_t M, int64_t N, int64_t x_row_stride,
                   int gate_first, int64_t PM, int64_t PN, int64_t s_row_stride, int64_t s_col_stride, int mode,
                   hipStream_t stream);
@@ -115,6 +115,9 @@ int launch_weight_dequant(const void* x, const float* s, void* y, int64_t N, int
 int launch_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
                        const void* b, const float* b_s, void* c, const void* bias, int64_t M, int64_t N,
                        int64_t K, int out_dtype, hipStream_t stream);
+int launch_fp8_grouped_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
+                               const void* b, const float* b_s, void* c, const void* bias, const int64_t* m_splits,
+                               int64_t G, int64_t M, int64_t N, int64_t K, int out_dtype, hipStream_t stream);
 int launch_add_bias(void* x, const void* b, int64_t M, int64_t N, hipStream_t stream);
 int launch_cast_f32_to_e4m3(const float* x, void* y, int64_t n, int saturate, hipStream_t stream);
 int launch_quotient_selfcheck(uint64_t* out, int amax_lo, int amax_hi, int mode, hipStream_t stream);

@@ -87,13 +87,15 @@ __device__ __forceinline__ void dma4(const intx4& rsrc, int voff, int soff, uint
                  :: "v"(voff), "s"(rsrc), "s"(soff), "s"(lds) : "memory");
 }
 
-// BM x BN block tile, WGM x WGN waves, each wave (BM/WGM) x (BN/WGN).
-// as_bytes = byte size of the addressed part of a_s (host computed, < 2^31).
+// One BM x BN tile of C: WGM x WGN waves, each wave (BM/WGM) x (BN/WGN).
+//   rows m0 .. min(m0+BM, m_end) of a (m_end = end of the matrix, or of the expert group the tile belongs to),
+//   columns n0 .. of b / b_s / bias (already offset to the group's weight), K % 128 == 0.
+// as_bytes = byte size of the addressed part of a_s (host computed, < 2^31); m_total = rows of a_s.
 template <int BM, int BN, int WGM, int WGN, typename OUT>
-__global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
+__device__ __forceinline__ void fp8_gemm_tile(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
-    const uint16_t* __restrict__ bias, int M, int N, int K, int ldc, int tiles_m, int tiles_n) {
+    const uint16_t* __restrict__ bias, int m0, int m_end, int m_total, int n0, int N, int K, int ldc) {
     constexpr int WAVES = WGM * WGN;
     constexpr int WM = BM / WGM, WN = BN / WGN, TI = WM / 16, TJ = WN / 16;
     constexpr int PASS_ROWS = WAVES * 8;  // rows copied by one DMA instruction of every wave
@@ -112,19 +114,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WGN, wn = wave % WGN;
-
-    // ---- XCD-aware tile order: consecutive workgroup ids land on different XCDs (8 of
-    // them); give each XCD a contiguous run of tiles, walked in groups of 4 tile rows.
-    int pid = blockIdx.x;
-    const int ntiles = tiles_m * tiles_n;
-    if (ntiles % 8 == 0) pid = (pid & 7) * (ntiles >> 3) + (pid >> 3);
-    constexpr int GM = 4;
-    const int group = pid / (GM * tiles_n);
-    const int first_m = group * GM;
-    const int gsz = min(tiles_m - first_m, GM);
-    const int tm = first_m + (pid % (GM * tiles_n)) % gsz;
-    const int tn = (pid % (GM * tiles_n)) / gsz;
-    const int m0 = tm * BM, n0 = tn * BN;
+    const int M = m_end;
     const int KB = K >> 7;
 
     // ---- DMA: descriptors limited to the rows of this tile, so that the M and N tails read 0
@@ -133,7 +123,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
     const intx4 rs = make_rsrc(a_s, as_bytes);
     const int prow = wave * 8 + (lane >> 3);                          // row inside a pass
     const int voff = prow * K + (((lane & 7) ^ swz(prow)) << 4);      // permuted chunk of that row
-    const int s_voff = min(m0 + wave * 64 + lane, M - 1) * as_rs * 4;
+    const int s_voff = min(m0 + wave * 64 + lane, m_total - 1) * as_rs * 4;
     const uint32_t la_base = lds_addr(&lds_a[0][0]) + wave * 1024;
     const uint32_t lb_base = lds_addr(&lds_b[0][0]) + wave * 1024;
     const uint32_t ls_base = lds_addr(&lds_s[0][0]) + wave * 256;
@@ -237,6 +227,70 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
             store4<OUT>(c, ldc, m, n, M, N, v, vec_ok);
         }
     }
+}
+
+// Tile order shared by the kernels below: consecutive workgroup ids land on different XCDs (8 of
+// them); give each XCD a contiguous run of tiles, walked in groups of 4 tile rows.
+__device__ __forceinline__ int xcd_contiguous(int pid, int ntiles) {
+    return (ntiles % 8 == 0) ? (pid & 7) * (ntiles >> 3) + (pid >> 3) : pid;
+}
+__device__ __forceinline__ void tile_of(int local, int tiles_m, int tiles_n, int& tm, int& tn) {
+    constexpr int GM = 4;
+    const int group = local / (GM * tiles_n);
+    const int first_m = group * GM;
+    const int gsz = min(tiles_m - first_m, GM);
+    tm = first_m + (local % (GM * tiles_n)) % gsz;
+    tn = (local % (GM * tiles_n)) / gsz;
+}
+
+template <int BM, int BN, int WGM, int WGN, typename OUT>
+__global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
+    const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
+    const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
+    const uint16_t* __restrict__ bias, int M, int N, int K, int ldc, int tiles_m, int tiles_n) {
+    int tm, tn;
+    tile_of(xcd_contiguous(blockIdx.x, tiles_m * tiles_n), tiles_m, tiles_n, tm, tn);
+    fp8_gemm_tile<BM, BN, WGM, WGN, OUT>(a, a_s, as_rs, as_cs, as_bytes, b, b_s, c, bias, tm * BM, M, M, tn * BN, N, K, ldc);
+}
+
+// ---------------------------------------------------------------------------
+// Grouped (mixture-of-experts) GEMM: rows row_start[g] .. row_start[g+1] of a are multiplied with
+// expert g's weight b[g] ([N, K], scales b_s[g]); c has the rows of a.  The table travels as a kernel
+// argument; a workgroup finds its group by binary search over the tile prefix sums.  Tiles never
+// straddle two groups: each group is tiled from its own first row, short last tiles read zeros and
+// store only their own rows.
+// ---------------------------------------------------------------------------
+constexpr int kMaxGroups = 256;
+struct GroupTable {
+    int n_groups;
+    int row_start[kMaxGroups + 1];   // first row of group g; [n_groups] = total rows
+    int tile_start[kMaxGroups + 1];  // tile rows (of BM) before group g
+};
+
+template <int BM, int BN, int WGM, int WGN, typename OUT>
+__global__ __launch_bounds__(WGM* WGN * 64) void fp8_grouped_gemm_kernel(
+    const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
+    const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
+    const uint16_t* __restrict__ bias, int N, int K, int tiles_n, const GroupTable tbl) {
+    const int G = tbl.n_groups;
+    const int pid = xcd_contiguous(blockIdx.x, tbl.tile_start[G] * tiles_n);
+    const int trow = pid / tiles_n;               // position in units of whole tile rows
+    int lo = 0, hi = G - 1;                       // last g with tile_start[g] <= trow (empty groups skipped)
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (tbl.tile_start[mid] <= trow) lo = mid; else hi = mid - 1;
+    }
+    // everything derived from the table is wave-uniform; say so (the copies need scalar descriptors)
+    const int g = __builtin_amdgcn_readfirstlane(lo);
+    const int tiles_m = __builtin_amdgcn_readfirstlane(tbl.tile_start[g + 1] - tbl.tile_start[g]);
+    int tm, tn;
+    tile_of(pid - tbl.tile_start[g] * tiles_n, tiles_m, tiles_n, tm, tn);
+    const int KB = K >> 7, NB = (N + 127) >> 7;
+    const int r0 = __builtin_amdgcn_readfirstlane(tbl.row_start[g]), r1 = __builtin_amdgcn_readfirstlane(tbl.row_start[g + 1]);
+    fp8_gemm_tile<BM, BN, WGM, WGN, OUT>(a, a_s, as_rs, as_cs, as_bytes, b + (size_t)g * N * K,
+                                         b_s + (size_t)g * NB * KB, c, bias ? bias + (size_t)g * N : nullptr,
+                                         __builtin_amdgcn_readfirstlane(r0 + tm * BM), r1,
+                                         __builtin_amdgcn_readfirstlane(tbl.row_start[G]), __builtin_amdgcn_readfirstlane(tn * BN), N, K, N);
 }
 
 // ---------------------------------------------------------------------------
@@ -467,6 +521,73 @@ int launch_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, i
                                   (int)M, (int)N, (int)K, stream);
     return dispatch<float>(ap, a_s, as_row_stride, as_col_stride, bp, b_s, static_cast<float*>(c), biasp, (int)M,
                            (int)N, (int)K, stream);
+}
+
+template <int BM, typename OUT>
+static int launch_grouped(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, uint32_t as_bytes,
+                          const uint8_t* b, const float* b_s, OUT* c, const uint16_t* bias, const int64_t* m_splits,
+                          int G, int N, int K, hipStream_t stream) {
+    GroupTable tbl;
+    tbl.n_groups = G;
+    int row = 0, trow = 0;
+    for (int g = 0; g < G; ++g) {
+        tbl.row_start[g] = row;
+        tbl.tile_start[g] = trow;
+        row += (int)m_splits[g];
+        trow += ((int)m_splits[g] + BM - 1) / BM;
+    }
+    for (int g = G; g <= kMaxGroups; ++g) { tbl.row_start[g] = row; tbl.tile_start[g] = trow; }
+    if (trow == 0) return 0;
+    const int tiles_n = (N + 255) / 256;
+    dim3 grid((unsigned)(trow * tiles_n)), block(512);
+    hipLaunchKernelGGL((fp8_grouped_gemm_kernel<BM, 256, 2, 4, OUT>), grid, block, 0, stream, a, a_s, (int)as_rs, (int)as_cs,
+                       as_bytes, b, b_s, c, bias, N, K, tiles_n, tbl);
+    return (int)hipGetLastError();
+}
+
+template <typename OUT>
+static int dispatch_grouped(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, const uint8_t* b,
+                            const float* b_s, OUT* c, const uint16_t* bias, const int64_t* m_splits, int G, int64_t M,
+                            int N, int K, hipStream_t stream) {
+    const int KB = (K + 127) / 128, NB = (N + 127) / 128;
+    const int64_t as_extent = ((M - 1) * as_rs + (int64_t)(KB - 1) * as_cs + 1) * 4;
+    const bool tiled_ok = (K % 128 == 0) && ((reinterpret_cast<uintptr_t>(a) & 15) == 0) &&
+                          ((reinterpret_cast<uintptr_t>(b) & 15) == 0) && K <= (1 << 22) && as_rs >= 0 && as_cs >= 0 &&
+                          as_extent < ((int64_t)1 << 31) && G <= kMaxGroups;
+    if (tiled_ok) {
+        bool all256 = true;
+        for (int g = 0; g < G; ++g) all256 = all256 && (m_splits[g] % 256 == 0);
+        if (all256)
+            return launch_grouped<256, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, m_splits, G, N, K, stream);
+        return launch_grouped<128, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, m_splits, G, N, K, stream);
+    }
+    // any other shape / alignment: one dense call per group
+    int64_t row = 0;
+    for (int g = 0; g < G; ++g) {
+        const int64_t mg = m_splits[g];
+        if (mg > 0) {
+            int rc = dispatch<OUT>(a + row * K, a_s + row * as_rs, as_rs, as_cs, b + (size_t)g * N * K,
+                                   b_s + (size_t)g * NB * KB, c + row * N, bias ? bias + (size_t)g * N : nullptr, (int)mg, N, K,
+                                   stream);
+            if (rc != 0) return rc;
+        }
+        row += mg;
+    }
+    return 0;
+}
+
+int launch_fp8_grouped_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
+                               const void* b, const float* b_s, void* c, const void* bias, const int64_t* m_splits,
+                               int64_t G, int64_t M, int64_t N, int64_t K, int out_dtype, hipStream_t stream) {
+    if (M == 0 || N == 0 || G == 0) return 0;
+    const uint8_t* ap = static_cast<const uint8_t*>(a);
+    const uint8_t* bp = static_cast<const uint8_t*>(b);
+    const uint16_t* biasp = static_cast<const uint16_t*>(bias);
+    if (out_dtype == 0)
+        return dispatch_grouped<uint16_t>(ap, a_s, as_row_stride, as_col_stride, bp, b_s, static_cast<uint16_t*>(c), biasp,
+                                          m_splits, (int)G, M, (int)N, (int)K, stream);
+    return dispatch_grouped<float>(ap, a_s, as_row_stride, as_col_stride, bp, b_s, static_cast<float*>(c), biasp, m_splits,
+                                   (int)G, M, (int)N, (int)K, stream);
 }
 
 }  // namespace mdy

@@ -1,5 +1,5 @@
 // Training-time quantizer: one pass over a bf16 matrix produces
-//   (1) the row-wise 1x128 quantization y[PM,PK] with scales s[kb*PM + m]      (as the forward quantizer), and
+//   (1) the row-wise 1x128 quantization y[PM,PK] with scales s[kb*s_kb_stride + m]      (as the forward quantizer), and
 //   (2) the quantized TRANSPOSE y_t[PK,PM], scaled either per 128x1 column group (t_mode 0) or per
 //       128x128 block (t_mode 1),
 // both in the DeepLinear dialect (scale = (min(amax,1e4) + 1e-8) / 448, saturating cast).
@@ -43,7 +43,7 @@ __global__ __launch_bounds__(256) void quant_transpose_kernel(const uint16_t* __
                                                                float* __restrict__ s, uint8_t* __restrict__ y_t,
                                                                float* __restrict__ s_t, int M, int K,
                                                                int64_t x_row_stride, int64_t x_col_stride, int PM,
-                                                               int PK) {
+                                                               int PK, int64_t s_kb_stride) {
     __shared__ float col_part[16][128];   // per row group (t/16) partial column maxima
     __shared__ float col_amax[128];
     __shared__ float blk_part[4];
@@ -104,7 +104,7 @@ __global__ __launch_bounds__(256) void quant_transpose_kernel(const uint16_t* __
             for (int j = 0; j < 8; ++j) q[j] = qt_quot<false>(f[i][j], sc, r);
         }
         store_nt8(y + (int64_t)row * PK + c0, make_uint2(pack4_e4m3(q[0], q[1], q[2], q[3]), pack4_e4m3(q[4], q[5], q[6], q[7])));
-        if ((t & 15) == 0) s[(int64_t)bk * PM + row] = sc;
+        if ((t & 15) == 0) s[(int64_t)bk * s_kb_stride + row] = sc;
     }
 
     // ---- (2) scales of the transposed copy
@@ -176,8 +176,8 @@ __global__ __launch_bounds__(256) void quant_transpose_kernel(const uint16_t* __
 }
 
 int launch_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
-                           int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int t_mode,
-                           hipStream_t stream) {
+                           int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int64_t s_kb_stride,
+                           int t_mode, hipStream_t stream) {
     if (PM == 0 || PK == 0) return 0;
     dim3 grid((unsigned)(PK / 128), (unsigned)(PM / 128));
     dim3 block(256);
@@ -188,7 +188,7 @@ int launch_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s
     uint8_t* ytp = static_cast<uint8_t*>(y_t);
 #define MDY_QT(TM, VEC)                                                                                          \
     hipLaunchKernelGGL((quant_transpose_kernel<TM, VEC>), grid, block, 0, stream, xp, yp, s, ytp, s_t, (int)M, \
-                       (int)K, x_row_stride, x_col_stride, (int)PM, (int)PK)
+                       (int)K, x_row_stride, x_col_stride, (int)PM, (int)PK, s_kb_stride)
     if (t_mode == 0) {
         if (vec) MDY_QT(0, true); else MDY_QT(0, false);
     } else {

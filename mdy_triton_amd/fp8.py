@@ -33,7 +33,7 @@ def _quant_transpose(x: torch.Tensor, t_mode: int, who: str):
     s_t = torch.empty((A, PN) if t_mode == 0 else (B, A), device=dev, dtype=torch.float32)
     with on_device(dev):
         check(lib().mdy_quant_transpose(ptr(x), ptr(y), ptr(s), ptr(y_t), ptr(s_t), M, K, x.stride(0), x.stride(1),
-                                        PM, PN, t_mode, stream_ptr(dev)), who)
+                                        PM, PN, PM, t_mode, stream_ptr(dev)), who)
     return y, s.transpose(0, 1), y_t, s_t
 
 

@@ -331,3 +331,76 @@ def silu_act_quant(x: torch.Tensor, order: str = "up-gate"):
     act = silu_fwd(x, order)
     y, s = act_quant(act.contiguous())
     return y, s, act
+
+
+# ----------------------------------------------------------------------------
+# Grouped (mixture-of-experts) operators of megatron_patchs/fp8_matmul.py
+# ----------------------------------------------------------------------------
+def per_token_cast_to_fp8(x: torch.Tensor, output_transpose: bool = False):
+    """fp8_matmul.py:96-135: quant_input's arithmetic; with output_transpose rows pad to 128 (not 256)
+    and the transposed copy is quantized column-wise in groups of 128 rows."""
+    if not output_transpose:
+        return quant_input(x, True)
+    M, N = x.shape
+    PM, PN = _cdiv(M, 128) * 128, _cdiv(N, 256) * 256
+    xp = torch.zeros(PM, PN, dtype=torch.float32)
+    xp[:M, :N] = x.detach().cpu().float()
+    g = xp.reshape(PM, PN // BLOCK, BLOCK)
+    scale = _scale_from_amax(g.abs().amax(-1))
+    y = _cast_sat(g / scale[:, :, None]).reshape(PM, PN)
+    gt = xp.t().contiguous().reshape(PN, PM // BLOCK, BLOCK)
+    scale_t = _scale_from_amax(gt.abs().amax(-1))
+    y_t = _cast_sat(gt / scale_t[:, :, None]).reshape(PN, PM)
+    return y, scale.t().contiguous().t(), y_t, scale_t.t().contiguous().t()
+
+
+def group_per_token_cast_to_fp8(x_all: torch.Tensor, m_splits):
+    """fp8_matmul.py:218-247: rows quantized over the whole matrix (scales [N/128, Mtot] returned
+    transposed), and per group the column-wise quantized transpose."""
+    Mtot, N = x_all.shape
+    ys, ss, yts, sts = [], [], [], []
+    for x in x_all.split(list(m_splits), 0):
+        assert x.size(0) % 256 == 0 and N % 256 == 0
+        if x.size(0) == 0:
+            yts.append(torch.empty(N, 0, dtype=FP8)); sts.append(torch.empty(0, N).t()); continue
+        y, s, y_t, s_t = per_token_cast_to_fp8(x, True)
+        ys.append(y); ss.append(s.contiguous()); yts.append(y_t); sts.append(s_t)
+    y_all = torch.cat(ys, 0)
+    s_all = torch.cat(ss, 0).t().contiguous().t()
+    return y_all, s_all, yts, sts
+
+
+def per_block_cast_to_fp8(ws, output_normal: bool = True, output_transpose: bool = False):
+    """fp8_matmul.py:334-392 for a list of equally shaped weights (stacked along a leading dimension)."""
+    ws = list(ws) if isinstance(ws, (list, tuple)) else [ws]
+    M, N = ws[0].shape
+    BA, BB = (256 if output_transpose else 128), (256 if output_normal else 128)
+    PM, PN = _cdiv(M, BA) * BA, _cdiv(N, BB) * BB
+    A, B = PM // BLOCK, PN // BLOCK
+    ys, ss = [], []
+    for w in ws:
+        wp = torch.zeros(PM, PN, dtype=torch.float32)
+        wp[:M, :N] = w.detach().cpu().float()
+        g = wp.reshape(A, BLOCK, B, BLOCK)
+        scale = _scale_from_amax(g.abs().amax(dim=(1, 3)))
+        ys.append(_cast_sat(g / scale[:, None, :, None]).reshape(PM, PN)); ss.append(scale)
+    y, s = torch.stack(ys), torch.stack(ss)
+    post = (lambda t: t.squeeze(0)) if len(ws) == 1 else (lambda t: t)
+    out = ()
+    if output_normal:
+        out += (post(y), post(s))
+    if output_transpose:
+        out += (post(y.transpose(1, 2).contiguous()), post(s.transpose(1, 2).contiguous()))
+    return out
+
+
+def fp8_grouped_matmul(qa, sa, qb, sb, m_splits, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp8_matmul.py:400-413: row m of group g is multiplied with weight g (one fp8_gemm per group)."""
+    outs, row = [], 0
+    sa = sa.contiguous()
+    for g, mg in enumerate(m_splits):
+        outs.append(fp8_gemm(qa[row:row + mg], sa[row:row + mg], qb[g], sb[g], dtype=torch.bfloat16,
+                             bias=None if bias is None else bias[g]) if mg > 0
+                    else torch.empty(0, qb.size(1), dtype=torch.bfloat16))
+        row += mg
+    return torch.cat(outs, 0)

@@ -1,0 +1,160 @@
+"""GPU parity of the grouped (mixture-of-experts) GEMM and the quantizers around it against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+import mdy_triton_amd as m
+from mdy_triton_amd import _lib
+from oracle import oracle as O
+from tests import problems as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+FP8 = torch.float8_e4m3fn
+RTOL = ATOL = 1e-2     # the GEMM tolerance of the dense path
+
+
+def u8(t):
+    return t.contiguous().view(torch.uint8).cpu().numpy()
+
+
+def same(got, ref):
+    assert got.shape == ref.shape and got.stride() == ref.stride()
+    if ref.dtype == FP8:
+        assert np.array_equal(u8(got), u8(ref))
+    else:
+        assert torch.equal(got.cpu().contiguous(), ref.contiguous())
+
+
+def exact_grouped_case(m_splits, N, K, seed, device_call):
+    """Integer operands and power-of-two scales: every product and partial sum is exact in fp32, so the
+    result must equal the float64 computation bit for bit, group by group."""
+    g = torch.Generator().manual_seed(seed)
+    G, M = len(m_splits), sum(m_splits)
+    KB, NB = K // 128, (N + 127) // 128
+    ai = torch.randint(-4, 5, (M, K), generator=g)
+    bi = torch.randint(-4, 5, (G, N, K), generator=g)
+    ae = torch.randint(-2, 3, (M, KB), generator=g)
+    be = torch.randint(-2, 3, (G, NB, KB), generator=g)
+    ref = torch.zeros(M, N, dtype=torch.float64)
+    row = 0
+    for gi, mg in enumerate(m_splits):
+        for kb in range(KB):
+            part = ai[row:row + mg, kb * 128:(kb + 1) * 128].double() @ bi[gi, :, kb * 128:(kb + 1) * 128].double().t()
+            ref[row:row + mg] += part * torch.exp2((ae[row:row + mg, kb][:, None] + be[gi, torch.arange(N) // 128, kb][None, :]).double())
+        row += mg
+    got = device_call(ai.float().to(FP8).to(DEV), torch.exp2(ae.float()).to(DEV), bi.float().to(FP8).to(DEV),
+                      torch.exp2(be.float()).to(DEV), m_splits)
+    assert torch.equal(got.cpu().double(), ref)
+
+
+def call_f32(qa, sa, qb, sb, m_splits):
+    """fp32 output through the C ABI (the Python wrapper returns bf16 like the reference)."""
+    import ctypes
+    M, K = qa.shape
+    G, N, _ = qb.shape
+    out = torch.full((M, N), float("nan"), device=DEV, dtype=torch.float32)
+    arr = (ctypes.c_int64 * G)(*m_splits)
+    _lib.check(_lib.load().mdy_fp8_grouped_gemm_nt(qa.data_ptr(), sa.data_ptr(), sa.stride(0), sa.stride(1), qb.data_ptr(),
+                                                   sb.data_ptr(), out.data_ptr(), None, ctypes.cast(arr, ctypes.c_void_p), G, N, K, 1,
+                                                   None), "grouped")
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.mark.parametrize("m_splits,N,K", [([256, 512, 0, 256], 520, 384),          # all multiples of 256: 256x256 tiles
+                                          ([100, 0, 1, 300, 129, 128], 776, 256),  # ragged groups: 128x256 tiles, tails everywhere
+                                          ([16] * 32, 2048, 512),                  # decode-like: many tiny groups
+                                          ([3, 5], 40, 128)])
+def test_grouped_gemm_exact_integer(m_splits, N, K):
+    exact_grouped_case(m_splits, N, K, sum(m_splits) + N + K, call_f32)
+
+
+def test_grouped_gemm_exact_integer_per_group_fallback():
+    # more groups than the single-launch table holds, and K not a multiple of 128 is rejected by the MFMA path
+    exact_grouped_case([2] * 300, 48, 128, 7, call_f32)
+
+
+def test_grouped_matmul_against_oracle_with_bias_and_column_major_scales():
+    G, N, K = 6, 1024, 2048
+    m_splits = [256, 64, 0, 500, 1, 203]
+    M = sum(m_splits)
+    x = P.activations("outliers", M, K, 31)
+    g = torch.Generator().manual_seed(32)
+    ws = [(torch.randn(N, K, generator=g) * 0.02).bfloat16() for _ in range(G)]
+    bias = torch.randn(G, N, generator=g).bfloat16()
+    qa, sa, _, _ = m.per_token_cast_to_fp8(x.to(DEV))
+    qb, sb = m.per_block_cast_to_fp8([w.to(DEV) for w in ws])
+    assert qb.shape == (G, N, K) and sb.shape == (G, N // 128, K // 128) and sa.stride() == (1, qa.size(0))
+    ra, rsa, _, _ = O.per_token_cast_to_fp8(x)
+    rb, rsb = O.per_block_cast_to_fp8(ws)
+    same(qa, ra); same(sa, rsa); same(qb, rb); same(sb, rsb)
+    out = m.fp8_grouped_matmul(qa[:M], sa[:M], qb, sb, m_splits)
+    ref = O.fp8_grouped_matmul(ra[:M], rsa[:M], rb, rsb, m_splits)
+    assert out.dtype == torch.bfloat16 and out.shape == (M, N)
+    assert torch.allclose(out.float().cpu(), ref.float(), rtol=RTOL, atol=ATOL)
+    outb = m.fp8_grouped_matmul(qa[:M], sa[:M], qb, sb, m_splits, bias=bias.to(DEV))
+    refb = O.fp8_grouped_matmul(ra[:M], rsa[:M], rb, rsb, m_splits, bias=bias)
+    rows = torch.repeat_interleave(torch.arange(G), torch.tensor(m_splits))
+    mag = torch.maximum(refb.float().abs(), (refb.float() - bias.float()[rows]).abs())
+    assert bool(((outb.float().cpu() - refb.float()).abs() <= ATOL + RTOL * mag).all())
+    buf = torch.empty_like(out)
+    assert m.fp8_grouped_matmul(qa[:M], sa[:M], qb, sb, m_splits, out=buf).data_ptr() == buf.data_ptr() and torch.equal(buf, out)
+    # one group == the dense GEMM, bit for bit (same kernel body, same accumulation order)
+    one = m.fp8_grouped_matmul(qa[:256], sa[:256], qb[:1], sb[:1], [256])
+    assert torch.equal(one, m.fp8_matmul(qa[:256], sa[:256], qb[0], sb[0]))
+
+
+@pytest.mark.parametrize("M,N,seed", [(256, 512, 0), (130, 300, 1), (1000, 256, 2)])
+def test_per_token_cast_with_transpose_bit_exact(M, N, seed):
+    x = P.activations("outliers", M, N, seed)
+    for g_, r_ in zip(m.per_token_cast_to_fp8(x.to(DEV), True), O.per_token_cast_to_fp8(x, True)):
+        same(g_, r_)
+
+
+def test_group_per_token_cast_bit_exact():
+    m_splits = [256, 0, 512, 256]
+    x = P.activations("outliers", sum(m_splits), 768, 5)
+    y, s, yts, sts = m.group_per_token_cast_to_fp8(x.to(DEV), m_splits)
+    ry, rs, ryts, rsts = O.group_per_token_cast_to_fp8(x, m_splits)
+    same(y, ry); same(s, rs)
+    assert len(yts) == len(sts) == 4
+    for a_, b_ in zip(yts + sts, ryts + rsts):
+        same(a_, b_)
+    with pytest.raises(AssertionError):
+        m.group_per_token_cast_to_fp8(x.to(DEV), [100, 924])
+
+
+@pytest.mark.parametrize("normal,transpose", [(True, False), (True, True), (False, True)])
+def test_per_block_cast_bit_exact(normal, transpose):
+    g = torch.Generator().manual_seed(9)
+    ws = [(torch.randn(200, 300, generator=g) * 0.02).bfloat16() for _ in range(3)]
+    got = m.per_block_cast_to_fp8([w.to(DEV) for w in ws], normal, transpose)
+    ref = O.per_block_cast_to_fp8(ws, normal, transpose)
+    assert len(got) == len(ref) == 2 * (int(normal) + int(transpose))
+    for a_, b_ in zip(got, ref):
+        same(a_, b_)
+    single = m.per_block_cast_to_fp8(ws[0].to(DEV), normal, transpose)
+    for a_, b_ in zip(single, O.per_block_cast_to_fp8(ws[0], normal, transpose)):
+        same(a_, b_)
+
+
+def test_grouped_abi_rejects_bad_arguments():
+    import ctypes
+    L = _lib.load()
+    a = torch.zeros(256, 128, dtype=torch.uint8, device=DEV)
+    s = torch.ones(256, 1, device=DEV)
+    b = torch.zeros(2, 128, 128, dtype=torch.uint8, device=DEV)
+    bs = torch.ones(2, 1, 1, device=DEV)
+    c = torch.empty(256, 128, dtype=torch.bfloat16, device=DEV)
+    ok = (ctypes.c_int64 * 2)(128, 128)
+    neg = (ctypes.c_int64 * 2)(300, -44)
+    args = lambda sp, **kw: [a.data_ptr(), s.data_ptr(), 1, 1, b.data_ptr(), bs.data_ptr(), kw.get("c", c.data_ptr()), None,
+                             ctypes.cast(sp, ctypes.c_void_p) if sp is not None else None, 2, 128, 128, kw.get("dt", 0), None]
+    assert L.mdy_fp8_grouped_gemm_nt(*args(ok)) == 0
+    assert L.mdy_fp8_grouped_gemm_nt(*args(neg)) == -2
+    assert L.mdy_fp8_grouped_gemm_nt(*args(None)) == -1
+    assert L.mdy_fp8_grouped_gemm_nt(*args(ok, dt=5)) == -4
+    assert L.mdy_fp8_grouped_gemm_nt(*args(ok, c=c.data_ptr() + 1)) == -3
+    with pytest.raises(ValueError):
+        m.fp8_grouped_matmul(a.view(FP8), s, b.view(FP8), bs, [100, 100])

@@ -232,11 +232,12 @@ def test_quant_transpose_abi_rejects_bad_arguments():
     y = torch.empty(256, 256, dtype=torch.uint8, device=DEV)
     s = torch.empty(2, 256, dtype=torch.float32, device=DEV)
     args = lambda **kw: [kw.get("x", x.data_ptr()), kw.get("y", y.data_ptr()), s.data_ptr(), kw.get("y_t", y.data_ptr()),
-                         s.data_ptr(), 256, 256, 256, 1, kw.get("PM", 256), kw.get("PK", 256), kw.get("t_mode", 0), None]
+                         s.data_ptr(), 256, 256, 256, 1, kw.get("PM", 256), kw.get("PK", 256), kw.get("skb", 256), kw.get("t_mode", 0), None]
     assert L.mdy_quant_transpose(*args(t_mode=2)) == -4
     assert L.mdy_quant_transpose(*args(PM=200)) == -2
     assert L.mdy_quant_transpose(*args(PK=384 + 64)) == -2
     assert L.mdy_quant_transpose(*args(y_t=None)) == -1
+    assert L.mdy_quant_transpose(*args(skb=100)) == -2
     assert L.mdy_quant_transpose(*args(y=y.data_ptr() + 4)) == -3
 
 

@@ -328,3 +328,33 @@ def test_silu_matches_torch_functional_and_autograd():
     e = torch.tensor([[1.0, 1.0, 1.0, 0.0, 60.0, -60.0]]).bfloat16()
     got = O.silu_fwd(e).tolist()[0]
     assert got[:2] == [0.0, 60.0] and abs(got[2] / (-60.0 * np.exp(-60.0)) - 1) < 2.0 ** -8
+
+
+def test_grouped_oracle_functions_reduce_to_the_pinned_ones():
+    g = torch.Generator().manual_seed(15)
+    x = torch.randn(512, 256, generator=g).bfloat16()
+    # M % 256 == 0: per_token_cast_to_fp8(output_transpose) is quant_grad_output
+    for a_, b_ in zip(O.per_token_cast_to_fp8(x, True), O.quant_grad_output(x)):
+        assert a_.shape == b_.shape and a_.stride() == b_.stride()
+        assert np.array_equal(u8(a_), u8(b_)) if a_.dtype == FP8 else torch.equal(a_.contiguous(), b_.contiguous())
+    # rows pad to 128, not 256
+    y, s, y_t, s_t = O.per_token_cast_to_fp8(x[:130], True)
+    assert tuple(y.shape) == (256, 256) and tuple(y_t.shape) == (256, 256) and tuple(s_t.shape) == (256, 2)
+    y, s, y_t, s_t = O.per_token_cast_to_fp8(x[:100], True)
+    assert tuple(y.shape) == (128, 256) and tuple(s_t.shape) == (256, 1) and s.stride() == (1, 128)
+    # grouped quantizer = the row quantizer on all rows + the transposed quantizer per group
+    ya, sa, yts, sts = O.group_per_token_cast_to_fp8(x, [256, 256])
+    yr, sr, _, _ = O.quant_input(x, True)
+    assert np.array_equal(u8(ya), u8(yr)) and torch.equal(sa.contiguous(), sr.contiguous()) and sa.stride() == (1, 512)
+    assert np.array_equal(u8(yts[1]), u8(O.quant_grad_output(x[256:])[2]))
+    # block quantizer on a list = quant_weight per member
+    ws = [(torch.randn(200, 300, generator=g) * 0.02).bfloat16() for _ in range(2)]
+    yb, sb, ybt, sbt = O.per_block_cast_to_fp8(ws, True, True)
+    q = O.quant_weight(ws[1], False)
+    assert np.array_equal(u8(yb[1]), u8(q[0])) and torch.equal(sb[1], q[1]) and np.array_equal(u8(ybt[1]), u8(q[2])) and torch.equal(sbt[1], q[3])
+    # grouped GEMM: rows of group g see only weight g
+    qa, sa, _, _ = O.per_token_cast_to_fp8(x)
+    qb, sb2 = O.per_block_cast_to_fp8([w[:128, :256].contiguous() for w in ws])
+    out = O.fp8_grouped_matmul(qa, sa, qb, sb2, [300, 212])
+    assert torch.equal(out[:300], O.fp8_gemm(qa[:300], sa.contiguous()[:300], qb[0], sb2[0]))
+    assert torch.equal(out[300:], O.fp8_gemm(qa[300:], sa.contiguous()[300:], qb[1], sb2[1]))
