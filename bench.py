@@ -295,6 +295,21 @@ def table(torch, m, timer, dev):
     line("C4 silu_fwd + act_quant (2 passes) %dx%d" % (Ms, Ns), timer.run(unfused, 20)[0], 9.03125 * Ms * Ns, "GB/s", PEAK_HBM_GBS)
     line("C4 silu_fwd %dx%d" % (Ms, Ns), timer.run(lambda: m.silu_fwd(ug), 20)[0], 6.0 * Ms * Ns, "GB/s", PEAK_HBM_GBS)
     del ug
+    # grouped (MoE) GEMM: 32 routed experts of the up/gate projection (N = 2 x 2048, K = 7168)
+    G, Ng, Kg = 32, 4096, 7168
+    bq = torch.randint(0, 120, (G, Ng, Kg), dtype=torch.uint8, device=dev).view(FP8)
+    bsg = torch.rand(G, Ng // 128, Kg // 128, device=dev)
+    for mg in (512, 16):
+        Mt = G * mg
+        aq = torch.randint(0, 120, (Mt, Kg), dtype=torch.uint8, device=dev).view(FP8)
+        asg = torch.rand(Mt, Kg // 128, device=dev)
+        us = timer.run(lambda: m.fp8_grouped_matmul(aq, asg, bq, bsg, [mg] * G), 10)[0]
+        if mg >= 256:
+            line("grouped fp8_gemm %d experts x %d rows, N=%d K=%d" % (G, mg, Ng, Kg), us, 2.0 * Mt * Ng * Kg, "TFLOP/s", PEAK_FP8_TFLOPS)
+        else:
+            line("grouped fp8_gemm %d experts x %d rows, N=%d K=%d" % (G, mg, Ng, Kg), us,
+                 Mt * Kg + G * Ng * Kg + 2.0 * Mt * Ng + 4.0 * Mt * Kg / 128, "GB/s", PEAK_HBM_GBS)
+    del bq, bsg, aq, asg
     for M in (1, 16, 64):
         for (N, K) in ((7168, 2048), (2048, 7168)):
             a = torch.randint(0, 120, (M, K), dtype=torch.uint8, device=dev).view(FP8)
