@@ -89,13 +89,28 @@ __device__ __forceinline__ void dma4(const intx4& rsrc, int voff, int soff, uint
 
 // One BM x BN tile of C: WGM x WGN waves, each wave (BM/WGM) x (BN/WGN).
 //   rows m0 .. min(m0+BM, m_end) of a (m_end = end of the matrix, or of the expert group the tile belongs to),
-//   columns n0 .. of b / b_s / bias (already offset to the group's weight), K % 128 == 0.
+//   columns n0 .. of b / b_s / bias (already offset to the group's weight), K % 128 == 0, K <= 65536.
 // as_bytes = byte size of the addressed part of a_s (host computed, < 2^31); m_total = rows of a_s.
+// a_duty (0..7) / b_duty (0..3): which share of the A / B panel lines this workgroup pre-touches for the
+// workgroups that copy the same panels (those with the same tile row / tile column).
+//
+// Schedule of one K block (NT = TI*TJ MFMA slots, each followed DEPTH slots later by its 4 FMAs):
+//   slots 0..      the last copies of K block kb+1 (those that did not fit into the tail below), one per slot,
+//                  then one "duty touch" load for K block kb+3;
+//   slot TB        = first MFMA of the last streamed fragment: every LDS read of this K block has been
+//                  consumed, so the wave waits for its copies of kb+1 and meets the others at THE barrier
+//                  of the K block; behind it buffer `cur` is free and buffer `cur^1` is complete;
+//   slots TB..     while the last MFMAs and FMAs of kb still run: reload the held fragments, the first
+//                  streamed fragment and the scales from buffer cur^1, and issue the first copies of kb+2
+//                  into buffer cur, one per slot.
+// So the LDS latency after the barrier and the issue time of the copies sit in the shadow of the matrix
+// pipe instead of in front of the first MFMA of the next K block.
 template <int BM, int BN, int WGM, int WGN, typename OUT>
 __device__ __forceinline__ void fp8_gemm_tile(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
-    const uint16_t* __restrict__ bias, int m0, int m_end, int m_total, int n0, int N, int K, int ldc) {
+    const uint16_t* __restrict__ bias, int m0, int m_end, int m_total, int n0, int N, int K, int ldc, int a_duty,
+    int b_duty) {
     constexpr int WAVES = WGM * WGN;
     constexpr int WM = BM / WGM, WN = BN / WGN, TI = WM / 16, TJ = WN / 16;
     constexpr int PASS_ROWS = WAVES * 8;  // rows copied by one DMA instruction of every wave
@@ -103,13 +118,23 @@ __device__ __forceinline__ void fp8_gemm_tile(
     constexpr int S_WAVES = BM / 64;      // waves that also copy the activation scales
     constexpr int DEPTH = 4;              // MFMAs in flight before their results are folded
     static_assert(BM % PASS_ROWS == 0 && BN % PASS_ROWS == 0 && PASS_ROWS % 16 == 0, "tile/threads mismatch");
-    static_assert(WN <= 128 && 128 % WN == 0 && S_WAVES <= WAVES, "one weight-scale block per wave column");
+    static_assert(WN <= 128 && 128 % WN == 0 && S_WAVES <= WAVES && WAVES >= 2, "one weight-scale block per wave column");
     constexpr bool HOLD_A = TI <= TJ;
     constexpr int NH = HOLD_A ? TI : TJ, NS = HOLD_A ? TJ : TI;
+    constexpr int NT = TI * TJ;
+    constexpr int NDMA = 1 + A_PASSES + B_PASSES;       // copies per K block and wave: scales, A passes, B passes
+    constexpr int TB = NT - NH;                         // slot of the barrier
+    constexpr int TAIL = NT + DEPTH - 1 - TB;           // slots behind the barrier
+    constexpr int FIRST = TAIL < NDMA ? TAIL : NDMA;    // copies of K block kb+2 issued in the tail of kb
+    constexpr int TD = 3;                               // duty touches run this many K blocks ahead
+    static_assert(NS % 2 == 0 && NS >= 2, "the first streamed fragment of the next K block reuses queue slot 0");
+    static_assert(NDMA - FIRST + 1 <= TB, "not enough slots in front of the barrier");
 
     __shared__ __attribute__((aligned(1024))) uint8_t lds_a[2][BM * 128];
     __shared__ __attribute__((aligned(1024))) uint8_t lds_b[2][BN * 128];
     __shared__ __attribute__((aligned(256))) float lds_s[2][BM];
+    __shared__ __attribute__((aligned(256))) float lds_bs[BN / 128][512];   // weight scales of the tile, all K blocks
+    __shared__ __attribute__((aligned(256))) uint8_t lds_dummy[WAVES * 512];   // target of copies that must go nowhere
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -120,23 +145,35 @@ __device__ __forceinline__ void fp8_gemm_tile(
     // ---- DMA: descriptors limited to the rows of this tile, so that the M and N tails read 0
     const intx4 ra = make_rsrc(a + (size_t)m0 * K, (uint32_t)min(BM, M - m0) * (uint32_t)K);
     const intx4 rb = make_rsrc(b + (size_t)n0 * K, (uint32_t)min(BN, N - n0) * (uint32_t)K);
-    const intx4 rs = make_rsrc(a_s, as_bytes);
+    intx4 rs = make_rsrc(a_s, as_bytes);
+    if (wave >= S_WAVES) rs[2] = 0;                                   // these waves copy no scales: always out of range
     const int prow = wave * 8 + (lane >> 3);                          // row inside a pass
     const int voff = prow * K + (((lane & 7) ^ swz(prow)) << 4);      // permuted chunk of that row
-    const int s_voff = min(m0 + wave * 64 + lane, m_total - 1) * as_rs * 4;
+    const int s_voff = min(m0 + (wave % S_WAVES) * 64 + lane, m_total - 1) * as_rs * 4;
+    const uint32_t ld_base = lds_addr(&lds_dummy[0]) + wave * 512;
     const uint32_t la_base = lds_addr(&lds_a[0][0]) + wave * 1024;
     const uint32_t lb_base = lds_addr(&lds_b[0][0]) + wave * 1024;
-    const uint32_t ls_base = lds_addr(&lds_s[0][0]) + wave * 256;
+    const uint32_t ls_base = wave < S_WAVES ? lds_addr(&lds_s[0][0]) + wave * 256 : ld_base;
+    const uint32_t ls_buf = wave < S_WAVES ? BM * 4 : 0;
 
-    auto dma_tile = [&](int kb, int buf) {
-        if (wave < S_WAVES) dma4(rs, s_voff, kb * as_cs * 4, ls_base + buf * (BM * 4));
-#pragma unroll
-        for (int i = 0; i < A_PASSES; ++i)
-            dma16(ra, voff, i * PASS_ROWS * K + kb * 128, la_base + buf * (BM * 128) + i * PASS_ROWS * 128);
-#pragma unroll
-        for (int i = 0; i < B_PASSES; ++i)
-            dma16(rb, voff, i * PASS_ROWS * K + kb * 128, lb_base + buf * (BN * 128) + i * PASS_ROWS * 128);
+    // copy i (0: scales, then the A passes, then the B passes) of K block kb into buffer buf.  Past the last K
+    // block the offsets run beyond the descriptors: no memory access, zeros into a buffer nobody reads any more.
+    auto issue = [&](int i, int kb, int buf) {
+        const bool more = kb < KB;
+        if (i == 0)
+            dma4(rs, s_voff, more ? kb * as_cs * 4 : (int)as_bytes, ls_base + buf * ls_buf);
+        else if (i <= A_PASSES)
+            dma16(ra, voff, (i - 1) * PASS_ROWS * K + (more ? kb * 128 : ra[2]), la_base + buf * (BM * 128) + (i - 1) * PASS_ROWS * 128);
+        else
+            dma16(rb, voff, (i - 1 - A_PASSES) * PASS_ROWS * K + (more ? kb * 128 : rb[2]),
+                  lb_base + buf * (BN * 128) + (i - 1 - A_PASSES) * PASS_ROWS * 128);
     };
+    // duty touch: wave 0 loads one dword of every line of its share of the B panel, wave 1 of the A panel,
+    // TD K blocks ahead, into the dummy area: the lines are in L2 when this workgroup and its neighbours
+    // copy them.  The other waves run the same instruction on an empty descriptor.
+    intx4 rt = wave == 0 ? rb : ra;
+    if (wave >= 2) rt[2] = 0;
+    const int touch_off = wave == 0 ? (b_duty * (BN / 4) + lane % (BN / 4)) * K : (a_duty * (BM / 8) + lane % (BM / 8)) * K;
 
     // ---- fragment reads: lane -> row (lane%16) and the 32-byte K slice (lane/16) of a 16-row sub-tile
     const int frow = lane & 15, fk = lane >> 4;
@@ -144,8 +181,10 @@ __device__ __forceinline__ void fp8_gemm_tile(
     const int a_rd1 = (wm * WM + frow) * 128 + (((2 * fk + 1) ^ swz(frow)) << 4);
     const int b_rd0 = (wn * WN + frow) * 128 + (((2 * fk) ^ swz(frow)) << 4);
     const int b_rd1 = (wn * WN + frow) * 128 + (((2 * fk + 1) ^ swz(frow)) << 4);
+    const int h0 = HOLD_A ? a_rd0 : b_rd0, h1 = HOLD_A ? a_rd1 : b_rd1;   // held operand
+    const int x0 = HOLD_A ? b_rd0 : a_rd0, x1 = HOLD_A ? b_rd1 : a_rd1;   // streamed operand
     const int s_rd = wm * WM + frow;
-    const float* bs_row = b_s + (size_t)(min(n0 + wn * WN, N - 1) >> 7) * KB;
+    const float* my_bs = lds_bs[(wn * WN) >> 7];
 
     floatx4 acc[TI][TJ];
 #pragma unroll
@@ -159,31 +198,37 @@ __device__ __forceinline__ void fp8_gemm_tile(
         return intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     };
 
-    dma_tile(0, 0);
+    // ---- prologue: the tile's weight scales, K block 0, the registers of step 0, the first copies of K block 1
+    if (wave < BN / 128) {
+        const int nb = min((n0 >> 7) + wave, ((N + 127) >> 7) - 1);
+        const intx4 rbs = make_rsrc(b_s + (size_t)nb * KB, (uint32_t)KB * 4u);
+        for (int cc = 0; cc < KB; cc += 64) dma4(rbs, lane * 4, cc * 4, lds_addr(&lds_bs[wave][cc]));
+    }
+#pragma unroll
+    for (int i = 0; i < NDMA; ++i) issue(i, 0, 0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    intx8 fh[NH], fx[2];
+    float sc[TI];
+#pragma unroll
+    for (int h = 0; h < NH; ++h) fh[h] = read_frag(HOLD_A ? lds_a[0] : lds_b[0], h0, h1, h);
+    {
+        const float sb = my_bs[0];
+#pragma unroll
+        for (int i = 0; i < TI; ++i) sc[i] = lds_s[0][s_rd + i * 16] * sb;
+    }
+    fx[0] = read_frag(HOLD_A ? lds_b[0] : lds_a[0], x0, x1, 0);
+#pragma unroll
+    for (int i = 0; i < FIRST; ++i) issue(i, 1, 1);
 
     for (int kb = 0; kb < KB; ++kb) {
         const int cur = kb & 1;
-        if (kb + 1 < KB) dma_tile(kb + 1, cur ^ 1);
-        const uint8_t* la = lds_a[cur];
-        const uint8_t* lb = lds_b[cur];
-        const float* ls = lds_s[cur];
-        const uint8_t* lh = HOLD_A ? la : lb;    // held operand
-        const uint8_t* lx = HOLD_A ? lb : la;    // streamed operand
-        const int h0 = HOLD_A ? a_rd0 : b_rd0, h1 = HOLD_A ? a_rd1 : b_rd1;
-        const int x0 = HOLD_A ? b_rd0 : a_rd0, x1 = HOLD_A ? b_rd1 : a_rd1;
-        const float sb = bs_row[kb];
-        intx8 fh[NH];
-#pragma unroll
-        for (int h = 0; h < NH; ++h) fh[h] = read_frag(lh, h0, h1, h);
-        float sc[TI];
-#pragma unroll
-        for (int i = 0; i < TI; ++i) sc[i] = ls[s_rd + i * 16] * sb;
-        intx8 fx[2];
-        fx[0] = read_frag(lx, x0, x1, 0);
+        const uint8_t* lx = HOLD_A ? lds_b[cur] : lds_a[cur];            // streamed operand of this K block
+        const uint8_t* lh_n = HOLD_A ? lds_a[cur ^ 1] : lds_b[cur ^ 1];  // operands and scales of the next one
+        const uint8_t* lx_n = HOLD_A ? lds_b[cur ^ 1] : lds_a[cur ^ 1];
+        const float* ls_n = lds_s[cur ^ 1];
+        float sc_n[TI];
         floatx4 p[DEPTH + 1];
-        constexpr int NT = TI * TJ;
 #pragma unroll
         for (int t = 0; t < NT + DEPTH; ++t) {
             if (t < NT) {
@@ -194,6 +239,16 @@ __device__ __forceinline__ void fp8_gemm_tile(
                 const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
                 // rows of the MFMA = n (B panel), columns = m (A panel)
                 p[t % (DEPTH + 1)] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb_, fa_, zero, 0, 0, 0, 0, 0, 0);
+                if (t == TB) {
+                    // the only outstanding load that may stay in flight is this step's touch (the youngest)
+                    asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+                    __syncthreads();
+                    fx[0] = read_frag(lx_n, x0, x1, 0);      // queue slot 0 was last used by streamed fragment NS-2
+                    const float sb = my_bs[min(kb + 1, KB - 1)];
+#pragma unroll
+                    for (int i = 0; i < TI; ++i) sc_n[i] = ls_n[s_rd + i * 16] * sb;
+                }
+                if (t >= TB) fh[h] = read_frag(lh_n, h0, h1, h);   // fh[h] had its last use just above
             }
             if (t >= DEPTH) {
                 const int u = t - DEPTH, si = u / NH, h = u % NH;
@@ -204,11 +259,15 @@ __device__ __forceinline__ void fp8_gemm_tile(
                 acc[i][j][2] = __builtin_fmaf(q[2], sc[i], acc[i][j][2]);
                 acc[i][j][3] = __builtin_fmaf(q[3], sc[i], acc[i][j][3]);
             }
-            __builtin_amdgcn_sched_barrier(0);  // keep the MFMA / FMA / ds_read interleaving as written
+            if (t < NDMA - FIRST) issue(FIRST + t, kb + 1, cur ^ 1);
+            if (t == NDMA - FIRST) dma4(rt, touch_off, kb + TD < KB ? (kb + TD) * 128 : rt[2], ld_base + 256);
+            if (t > TB && t - TB - 1 < FIRST) issue(t - TB - 1, kb + 2, cur);
+            __builtin_amdgcn_sched_barrier(0);  // keep the MFMA / FMA / ds_read / copy interleaving as written
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the next K block has landed in LDS
-        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < TI; ++i) sc[i] = sc_n[i];
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing may still be writing LDS when the wave ends
 
     // ---- epilogue: lane holds c[m][n..n+3], m = .. + lane%16, n = .. + 4*(lane/16)
     const bool vec_ok = (ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
@@ -250,7 +309,8 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
     const uint16_t* __restrict__ bias, int M, int N, int K, int ldc, int tiles_m, int tiles_n) {
     int tm, tn;
     tile_of(xcd_contiguous(blockIdx.x, tiles_m * tiles_n), tiles_m, tiles_n, tm, tn);
-    fp8_gemm_tile<BM, BN, WGM, WGN, OUT>(a, a_s, as_rs, as_cs, as_bytes, b, b_s, c, bias, tm * BM, M, M, tn * BN, N, K, ldc);
+    fp8_gemm_tile<BM, BN, WGM, WGN, OUT>(a, a_s, as_rs, as_cs, as_bytes, b, b_s, c, bias, tm * BM, M, M, tn * BN, N, K, ldc, tn & 7,
+                                         tm & 3);
 }
 
 // ---------------------------------------------------------------------------
@@ -290,7 +350,8 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_grouped_gemm_kernel(
     fp8_gemm_tile<BM, BN, WGM, WGN, OUT>(a, a_s, as_rs, as_cs, as_bytes, b + (size_t)g * N * K,
                                          b_s + (size_t)g * NB * KB, c, bias ? bias + (size_t)g * N : nullptr,
                                          __builtin_amdgcn_readfirstlane(r0 + tm * BM), r1,
-                                         __builtin_amdgcn_readfirstlane(tbl.row_start[G]), __builtin_amdgcn_readfirstlane(tn * BN), N, K, N);
+                                         __builtin_amdgcn_readfirstlane(tbl.row_start[G]), __builtin_amdgcn_readfirstlane(tn * BN), N, K, N,
+                                         __builtin_amdgcn_readfirstlane(tn & 7), __builtin_amdgcn_readfirstlane(tm & 3));
 }
 
 // ---------------------------------------------------------------------------
@@ -474,7 +535,7 @@ static int dispatch(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t a
     const int64_t as_extent = ((int64_t)(M - 1) * as_rs + (int64_t)(KB - 1) * as_cs + 1) * 4;
     const bool mfma_ok = (K % 128 == 0) && ((reinterpret_cast<uintptr_t>(a) & 15) == 0) &&
                          ((reinterpret_cast<uintptr_t>(b) & 15) == 0);
-    const bool big_ok = mfma_ok && K <= (1 << 22) && as_rs >= 0 && as_cs >= 0 && as_extent < ((int64_t)1 << 31);
+    const bool big_ok = mfma_ok && K <= (1 << 16) && as_rs >= 0 && as_cs >= 0 && as_extent < ((int64_t)1 << 31);
     if (!mfma_ok || (M > 64 && !big_ok)) {
         dim3 grid((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16));
         hipLaunchKernelGGL((fp8_gemm_scalar_kernel<OUT>), grid, dim3(256), 0, stream, a, a_s, as_rs, as_cs, b, b_s, c,
@@ -552,7 +613,7 @@ static int dispatch_grouped(const uint8_t* a, const float* a_s, int64_t as_rs, i
     const int KB = (K + 127) / 128, NB = (N + 127) / 128;
     const int64_t as_extent = ((M - 1) * as_rs + (int64_t)(KB - 1) * as_cs + 1) * 4;
     const bool tiled_ok = (K % 128 == 0) && ((reinterpret_cast<uintptr_t>(a) & 15) == 0) &&
-                          ((reinterpret_cast<uintptr_t>(b) & 15) == 0) && K <= (1 << 22) && as_rs >= 0 && as_cs >= 0 &&
+                          ((reinterpret_cast<uintptr_t>(b) & 15) == 0) && K <= (1 << 16) && as_rs >= 0 && as_cs >= 0 &&
                           as_extent < ((int64_t)1 << 31) && G <= kMaxGroups;
     if (tiled_ok) {
         bool all256 = true;
