@@ -34,12 +34,12 @@ if ROOT not in sys.path:
 PEAK_FP8_TFLOPS = 5000.0   # MI355X dense FP8 MFMA, published
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E, published
 
-# HBM bytes per fp8_gemm launch at the C3 shape, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (KiB per dispatch, scaled by the same counters read on a plain copy kernel of known size);
-# the runs are summarised in profiles/bench_C3_hbm_traffic.txt: FETCH_SIZE 407 706 KiB x 1.9997 (copy-kernel
-# calibration) = 834.9 MB read, WRITE_SIZE 150 687 KiB x 1.0 = 154.3 MB written; algorithmic bytes are 313 MB
-# (the A and B panels are re-fetched by the eight XCD-local L2s).
-GEMM_C3_HBM_TRAFFIC_BYTES = 989.2e6
+# HBM bytes per fp8_gemm call at the C3 shape (both of its launches), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (KiB per dispatch, scaled by the same counters read on a plain copy kernel of known size); the runs are
+# summarised in profiles/bench_C3_hbm_traffic.txt: FETCH_SIZE (349 095 + 72 421) KiB x 1.9997 (copy-kernel
+# calibration) = 863.2 MB read, WRITE_SIZE (133 707 + 16 426) KiB x 1.0 = 153.7 MB written; algorithmic bytes are
+# 313 MB (the A and B panels are re-fetched by the eight XCD-local L2s).
+GEMM_C3_HBM_TRAFFIC_BYTES = 1016.9e6
 
 WORKLOADS = {
     # name: (activation kind, M, N, K, description)
@@ -230,7 +230,10 @@ def main():
         "data": "synthetic",
         "config": {"workload": "%s %s; step = act_quant + fp8_gemm (pre-quantized weight)" % (args.workload, desc),
                    "M": M, "N": N, "K": K},
-        "roofline": {"bound": "mfma", "kernel": "fp8_gemm", "achieved": round(achieved, 2), "peak": PEAK_FP8_TFLOPS,
+        "roofline": {"bound": "mfma",
+                     "kernel": "fp8_gemm (one call = fp8_gemm_mfma_kernel<256,256> on the first 16384 columns + <128,256> on the last 2048)"
+                     if args.workload == "C3" else "fp8_gemm",
+                     "achieved": round(achieved, 2), "peak": PEAK_FP8_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP8_TFLOPS, 4),
                      "launch_us": round(gemm_us, 2), "flops_per_launch": flops,
                      "traffic": GEMM_C3_HBM_TRAFFIC_BYTES if args.workload == "C3" else None},
