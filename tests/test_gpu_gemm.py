@@ -90,6 +90,19 @@ def test_gemm_split_launch_with_bias_bf16():
     assert close_biased(got[rows.to(DEV)], ref, bias)
 
 
+def test_gemm_is_deterministic_and_k_tail_blocks_are_not_touched():
+    """Copies and prefetch touches that run past the last K block must go nowhere: the same call repeated
+    gives identical bits, and a weight with a single K block works on every tile shape."""
+    a, a_s, wq, ws = quantized_problem("normal", 4096, 4352, 128, 5)
+    args = (a.to(DEV), a_s.to(DEV), wq.to(DEV), ws.to(DEV))
+    first = m.fp8_gemm(*args, out_dtype=torch.float32)
+    for _ in range(3):
+        assert torch.equal(m.fp8_gemm(*args, out_dtype=torch.float32), first)
+    ref = O.fp8_gemm(a[::97].contiguous(), a_s[::97].contiguous(), wq, ws, dtype=torch.float32)
+    assert torch.allclose(first[::97].cpu(), ref, rtol=2e-3, atol=1e-3)
+    test_gemm_exact_integer_cases_all_kernels(300, 520, 128)      # 128x128 tiles, one K block
+
+
 @pytest.mark.parametrize("M", [1, 5, 16, 17, 33, 64])
 def test_gemm_small_m_exact(M):
     test_gemm_exact_integer_cases_all_kernels(M, 272, 384)
