@@ -378,6 +378,7 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_kernel(const ui
     const int frow = lane & 15, fk = lane >> 4;
     const int n0 = blockIdx.x * 16;
     const int KB = K >> 7;
+    const int m_base = blockIdx.y * (MT * 16);     // grid.y splits the rows when there are few column groups
     const int nrow = min(n0 + frow, N - 1);
     const uint8_t* bp = b + (int64_t)nrow * K + fk * 32;
     const float* bsp = b_s + (int64_t)(n0 >> 7) * KB;
@@ -385,7 +386,7 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_kernel(const ui
     const float* asp[MT];
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
-        const int m = min(i * 16 + frow, M - 1);
+        const int m = min(m_base + i * 16 + frow, M - 1);
         ap[i] = a + (int64_t)m * K + fk * 32;
         asp[i] = a_s + (int64_t)m * as_rs;
     }
@@ -451,7 +452,7 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_kernel(const ui
             for (int w = 0; w < kSmWaves; ++w) t += red[w][i][lane][e];
             v[e] = t;
         }
-        const int m = i * 16 + frow, n = n0 + 4 * fk;
+        const int m = m_base + i * 16 + frow, n = n0 + 4 * fk;
         if (bias != nullptr) {
 #pragma unroll
             for (int e = 0; e < 4; ++e)
@@ -543,13 +544,19 @@ static int dispatch(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t a
         return (int)hipGetLastError();
     }
     if (M <= 64) {
-        dim3 grid((unsigned)((N + 15) / 16));
+        // one workgroup streams 16 weight columns against MT row sub-tiles; every workgroup re-reads its rows of
+        // a, so with few column groups (N small) the rows are split over grid.y as well: more workgroups, less
+        // traffic through each CU's L1
+        const int sub = (M + 15) / 16;
+        int mt = sub;
+        if ((N + 15) / 16 < 200 && sub >= 2) mt = (sub + 1) / 2;
+        dim3 grid((unsigned)((N + 15) / 16), (unsigned)((sub + mt - 1) / mt));
 #define MDY_SM(MT)                                                                                                 \
     hipLaunchKernelGGL((fp8_gemm_smallm_kernel<MT, OUT>), grid, dim3(kSmWaves * 64), 0, stream, a, a_s, as_rs, as_cs, b, b_s, \
                        c, bias, M, N, K)
-        if (M <= 16) MDY_SM(1);
-        else if (M <= 32) MDY_SM(2);
-        else if (M <= 48) MDY_SM(3);
+        if (mt == 1) MDY_SM(1);
+        else if (mt == 2) MDY_SM(2);
+        else if (mt == 3) MDY_SM(3);
         else MDY_SM(4);
 #undef MDY_SM
         return (int)hipGetLastError();
