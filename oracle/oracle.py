@@ -22,6 +22,19 @@ Pinning status (what fixes each function besides its own formula):
   fp8_gemm
       float64 matmul on small shapes; exactly-representable integer cases that
       must match bit for bit; one-hot rows; single-scale-block perturbation.
+  quant_grad_output / quant_input(only_forward=False) / per_token_cast_to_fp8 /
+  group_per_token_cast_to_fp8 / per_block_cast_to_fp8
+      reduce to the pinned forward quantizers: row-wise copy == quant_input, the
+      column-wise transposed copy == quant_input of the transposed matrix, the
+      block-scaled transposed copy == quant_weight's; padding, strides and single
+      tiles re-derived by brute force in numpy (tests/test_oracle.py).
+  silu_fwd / silu_bwd / silu_act_quant
+      floating point: compared with torch.nn.functional.silu and its autograd
+      gradient (library routines) and closed forms; the quantizer half is act_quant.
+  deep_linear_backward / fp8_grouped_matmul
+      compositions of the above (per group: fp8_gemm); checked against unquantized
+      fp32 gradients within the quantization error band and for operand roles
+      (swapping x and dy transposes wgrad).
   fp8_matmul (DeepLinear's GEMM)
       PARITY UNPINNED at the third-party boundary: the reference calls
       `deep_gemm.gemm_fp8_fp8_bf16_nt` (dpsk_fp8linear/fp8.py:310), an
