@@ -37,7 +37,8 @@ Pinning status (what fixes each function besides its own formula):
       (swapping x and dy transposes wgrad).
   fp8_matmul (DeepLinear's GEMM)
       PARITY UNPINNED at the third-party boundary: the reference calls
-      `deep_gemm.gemm_fp8_fp8_bf16_nt` (dpsk_fp8linear/fp8.py:310), an
+      `deep_gemm.gemm_fp8_fp8_bf16_nt` (dpsk_fp8linear/fp8.py:310; the grouped
+      call is megatron_patchs/fp8_matmul.py:412), an
       un-vendored, un-pinned package whose source is not in the reference and
       whose only recorded outputs are unseeded notebook prints.  The oracle
       follows the in-tree formula with the same contract
