@@ -66,6 +66,35 @@ __device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float 
     return (uint32_t)w;
 }
 
+// 4x4 byte transpose with v_perm_b32: r[i] holds bytes (i,0..3); on return c[j] holds bytes (0..3, j).
+__device__ __forceinline__ void transpose4x4_bytes(const uint32_t (&r)[4], uint32_t (&c)[4]) {
+    // __builtin_amdgcn_perm(s0, s1, sel): result byte k = byte sel[k] of {s1: 0..3, s0: 4..7}
+    const uint32_t t0 = __builtin_amdgcn_perm(r[1], r[0], 0x05010400u);   // r0.b0 r1.b0 r0.b1 r1.b1
+    const uint32_t t1 = __builtin_amdgcn_perm(r[1], r[0], 0x07030602u);   // r0.b2 r1.b2 r0.b3 r1.b3
+    const uint32_t t2 = __builtin_amdgcn_perm(r[3], r[2], 0x05010400u);
+    const uint32_t t3 = __builtin_amdgcn_perm(r[3], r[2], 0x07030602u);
+    c[0] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
+    c[1] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
+    c[2] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
+    c[3] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
+}
+// 8 rows x 8 columns of bytes: row i = (lo[i], hi[i]); column j comes back as tb[j][0] (rows 0..3), tb[j][1] (rows 4..7)
+__device__ __forceinline__ void transpose8x8_bytes(const uint32_t (&lo)[8], const uint32_t (&hi)[8], uint32_t (&tb)[8][2]) {
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        const uint32_t rl[4] = {lo[4 * half], lo[4 * half + 1], lo[4 * half + 2], lo[4 * half + 3]};
+        const uint32_t rh[4] = {hi[4 * half], hi[4 * half + 1], hi[4 * half + 2], hi[4 * half + 3]};
+        uint32_t cl[4], ch[4];
+        transpose4x4_bytes(rl, cl);
+        transpose4x4_bytes(rh, ch);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            tb[j][half] = cl[j];
+            tb[4 + j][half] = ch[j];
+        }
+    }
+}
+
 // Streaming (non-temporal) vector accesses: the quantizers and the dequantizer touch every
 // byte exactly once, so they bypass cache allocation; measured 1.25-1.5x over plain accesses.
 typedef unsigned uintx4_t __attribute__((ext_vector_type(4)));

@@ -145,9 +145,7 @@ __global__ __launch_bounds__(256) void quant_transpose_kernel(const uint16_t* __
         tr[j] = 1.0f / tsc[j];
         tfast = tfast && (tamax[j] <= 1e4f);
     }
-    uint32_t tb[8][2];   // [column j][rows 0..3 | 4..7] quantized bytes of the transposed copy
-#pragma unroll
-    for (int j = 0; j < 8; ++j) tb[j][0] = tb[j][1] = 0u;
+    uint32_t qlo[8], qhi[8];   // row i of the transposed copy's bytes: columns 0..3 | 4..7
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         float q[8];
@@ -158,11 +156,11 @@ __global__ __launch_bounds__(256) void quant_transpose_kernel(const uint16_t* __
 #pragma unroll
             for (int j = 0; j < 8; ++j) q[j] = qt_quot<false>(f[i][j], tsc[j], tr[j]);
         }
-        const uint32_t lo = pack4_e4m3(q[0], q[1], q[2], q[3]), hi = pack4_e4m3(q[4], q[5], q[6], q[7]);
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-            tb[j][i >> 2] |= (((j < 4 ? lo : hi) >> (8 * (j & 3))) & 0xFFu) << (8 * (i & 3));
+        qlo[i] = pack4_e4m3(q[0], q[1], q[2], q[3]);
+        qhi[i] = pack4_e4m3(q[4], q[5], q[6], q[7]);
     }
+    uint32_t tb[8][2];   // [column j][rows 0..3 | 4..7]
+    transpose8x8_bytes(qlo, qhi, tb);
 #pragma unroll
     for (int j = 0; j < 8; ++j) *reinterpret_cast<uint2*>(&tile[cl + j][rg * 8]) = make_uint2(tb[j][0], tb[j][1]);
     __syncthreads();

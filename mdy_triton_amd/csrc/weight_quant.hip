@@ -74,9 +74,7 @@ __global__ __launch_bounds__(256) void weight_quant_kernel(const uint16_t* __res
         s[(int64_t)bn * (PK >> 7) + bk] = sc;
         if (s_t) s_t[(int64_t)bk * (PN >> 7) + bn] = sc;
     }
-    uint32_t tb[8][2];   // [column j][rows 0..3 | 4..7] bytes of the transposed copy
-#pragma unroll
-    for (int j = 0; j < 8; ++j) tb[j][0] = tb[j][1] = 0u;
+    uint32_t qlo[8], qhi[8];   // row i of the quantized bytes: columns 0..3 | 4..7
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         float q[8];
@@ -98,11 +96,12 @@ __global__ __launch_bounds__(256) void weight_quant_kernel(const uint16_t* __res
         o.y = pack4_e4m3(q[4], q[5], q[6], q[7]);
         const int row = rbase + i;  // < PN because PN % 128 == 0
         store_nt8(y + (int64_t)row * PK + c0, o);
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-            tb[j][i >> 2] |= (((j < 4 ? o.x : o.y) >> (8 * (j & 3))) & 0xFFu) << (8 * (i & 3));
+        qlo[i] = o.x;
+        qhi[i] = o.y;
     }
     if (y_t) {
+        uint32_t tb[8][2];   // [column j][rows 0..3 | 4..7]
+        transpose8x8_bytes(qlo, qhi, tb);
 #pragma unroll
         for (int j = 0; j < 8; ++j)
             *reinterpret_cast<uint2*>(&tile[(t & 15) * 8 + j][(t >> 4) * 8]) = make_uint2(tb[j][0], tb[j][1]);
