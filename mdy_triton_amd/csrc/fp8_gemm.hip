@@ -463,6 +463,133 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_kernel(const ui
 }
 
 // ---------------------------------------------------------------------------
+// Strip kernel: few rows (<= 16*MT <= 64 per group) against a weight that is wide enough to give every CU
+// work without splitting K (many column strips: a vocabulary-sized N, or many experts).  One workgroup = 8
+// waves = 128 weight columns of one group, wave w streams rows n0+16w .. +15 of the weight straight from
+// global memory into MFMA fragments (each row is read once, 512 contiguous bytes per row and step), while
+// the activation rows of the step (<= 64 rows x 512 bytes) and their scales are copied into LDS ONCE per
+// workgroup and shared by the 8 waves - in the kernel above every 16 columns re-read them, which is what
+// bounds it as soon as there are 16 or more rows.  grid = (ceil(N/128), groups).
+// ---------------------------------------------------------------------------
+constexpr int kStripKC = 4;   // K blocks per step
+
+template <int MT, typename OUT>
+__global__ __launch_bounds__(512) void fp8_gemm_strip_kernel(
+    const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
+    const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
+    const uint16_t* __restrict__ bias, int N, int K, const GroupTable tbl) {
+    constexpr int ROWS = MT * 16, KC = kStripKC;
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a[2][KC][ROWS * 128];
+    __shared__ __attribute__((aligned(256))) float lds_sa[2][KC][64];
+    __shared__ __attribute__((aligned(256))) float lds_bs[512];
+    __shared__ __attribute__((aligned(256))) uint8_t lds_dummy[8 * 1024];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = blockIdx.y;
+    const int r0 = __builtin_amdgcn_readfirstlane(tbl.row_start[g]);
+    const int r1 = __builtin_amdgcn_readfirstlane(tbl.row_start[g + 1]);
+    const int m_total = __builtin_amdgcn_readfirstlane(tbl.row_start[tbl.n_groups]);
+    const int rows = r1 - r0;                  // <= ROWS
+    if (rows <= 0) return;
+    const int n0 = blockIdx.x * 128;
+    const int KB = K >> 7, NB = (N + 127) >> 7;
+    const int steps = (KB + KC - 1) / KC;
+    const uint8_t* bg = b + (size_t)g * N * K;
+
+    // ---- copies: activation rows (8 rows x 128 bytes per instruction) and their scales (one row per lane)
+    const intx4 ra = make_rsrc(a + (size_t)r0 * K, (uint32_t)rows * (uint32_t)K);
+    intx4 rs = make_rsrc(a_s, as_bytes);
+    if (wave >= KC) rs[2] = 0;
+    const int prow = lane >> 3;
+    // a wave's instructions all land on row groups of the same parity (j / KC = wave / 4 + 2t): one swizzle per wave
+    const int voff = prow * K + (((lane & 7) ^ swz(((wave >> 2) & 1) * 8 + prow)) << 4);
+    const int s_voff = min(r0 + min(lane, rows - 1), m_total - 1) * as_rs * 4;
+    const uint32_t la0 = lds_addr(&lds_a[0][0][0]);
+    const uint32_t ls0 = wave < KC ? lds_addr(&lds_sa[0][wave][0]) : lds_addr(&lds_dummy[0]) + wave * 1024;
+    const uint32_t ls_buf = wave < KC ? KC * 64 * 4 : 0;
+    auto copy_step = [&](int step, int buf) {
+        // instruction j of the step: K block j % KC, row group j / KC (8 rows); wave w takes j = w, w + 8, ...
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            const int j = wave + 8 * t, kc = j % KC, rg = j / KC;
+            dma16(ra, voff, rg * 8 * K + (step * KC + kc) * 128, la0 + (buf * KC + kc) * (ROWS * 128) + rg * 1024);
+        }
+        dma4(rs, s_voff, min(step * KC + wave, KB - 1) * as_cs * 4, ls0 + buf * ls_buf);
+    };
+
+    // ---- weight fragments straight from global memory: lane -> row lane%16, 32-byte K slice lane/16
+    const int frow = lane & 15, fk = lane >> 4;
+    const uint8_t* bp = bg + (size_t)min(n0 + wave * 16 + frow, N - 1) * K + fk * 32;
+    uint4 blo[KC], bhi[KC];
+    auto load_b = [&](int step) {
+#pragma unroll
+        for (int kc = 0; kc < KC; ++kc) {
+            const int kb = min(step * KC + kc, KB - 1);      // the clamped duplicates are never used
+            blo[kc] = load_nt16(bp + (size_t)kb * 128);
+            bhi[kc] = load_nt16(bp + (size_t)kb * 128 + 16);
+        }
+    };
+    const int a_rd0 = frow * 128 + (((2 * fk) ^ swz(frow)) << 4);
+    const int a_rd1 = frow * 128 + (((2 * fk + 1) ^ swz(frow)) << 4);
+
+    floatx4 acc[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    if (wave == 0) {
+        const intx4 rbs = make_rsrc(b_s + ((size_t)g * NB + min(n0 >> 7, NB - 1)) * KB, (uint32_t)KB * 4u);
+        for (int cc = 0; cc < KB; cc += 64) dma4(rbs, lane * 4, cc * 4, lds_addr(&lds_bs[cc]));
+    }
+    copy_step(0, 0);
+    for (int step = 0; step < steps; ++step) {
+        const int buf = step & 1;
+        load_b(step);                                   // this step's weight rows: the long-latency part
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();                                // the step's activation rows are in LDS; buffer buf^1 is free
+        if (step + 1 < steps) copy_step(step + 1, buf ^ 1);
+#pragma unroll
+        for (int kc = 0; kc < KC; ++kc) {
+            const int kb = step * KC + kc;
+            if (kb < KB) {
+                const float sb = lds_bs[kb];
+                const intx8 fb = intx8{(int)blo[kc].x, (int)blo[kc].y, (int)blo[kc].z, (int)blo[kc].w,
+                                       (int)bhi[kc].x, (int)bhi[kc].y, (int)bhi[kc].z, (int)bhi[kc].w};
+#pragma unroll
+                for (int i = 0; i < MT; ++i) {
+                    const uint8_t* la = &lds_a[buf][kc][i * 2048];
+                    const intx4 lo = *reinterpret_cast<const intx4*>(la + a_rd0);
+                    const intx4 hi = *reinterpret_cast<const intx4*>(la + a_rd1);
+                    const intx8 fa = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    const float sc = lds_sa[buf][kc][i * 16 + frow] * sb;
+                    const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+                    const floatx4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, zero, 0, 0, 0, 0, 0, 0);
+                    acc[i][0] = __builtin_fmaf(p[0], sc, acc[i][0]);
+                    acc[i][1] = __builtin_fmaf(p[1], sc, acc[i][1]);
+                    acc[i][2] = __builtin_fmaf(p[2], sc, acc[i][2]);
+                    acc[i][3] = __builtin_fmaf(p[3], sc, acc[i][3]);
+                }
+            }
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    const bool vec_ok = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
+    const uint16_t* gbias = bias ? bias + (size_t)g * N : nullptr;
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int m = r0 + i * 16 + frow, n = n0 + wave * 16 + 4 * fk;
+        float v[4] = {acc[i][0], acc[i][1], acc[i][2], acc[i][3]};
+        if (gbias != nullptr) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (n + e < N) v[e] += bf16_one(gbias[n + e]);
+        }
+        store4<OUT>(c, N, m, n, r1, N, v, vec_ok);
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Scalar kernel: any M, N, K, any alignment (K tail reads as zero, like the masked
 // loads at offical_kernel.py:82-83).  One thread per output element.
 // ---------------------------------------------------------------------------
@@ -529,6 +656,35 @@ static int main_tile_columns(int tiles_m, int tiles_n) {
 }
 
 template <typename OUT>
+static int launch_strip(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, uint32_t as_bytes,
+                        const uint8_t* b, const float* b_s, OUT* c, const uint16_t* bias, const int64_t* m_splits, int G,
+                        int max_rows, int N, int K, hipStream_t stream) {
+    GroupTable tbl;
+    tbl.n_groups = G;
+    int row = 0;
+    for (int g = 0; g < G; ++g) {
+        tbl.row_start[g] = row;
+        tbl.tile_start[g] = 0;
+        row += (int)m_splits[g];
+    }
+    for (int g = G; g <= kMaxGroups; ++g) { tbl.row_start[g] = row; tbl.tile_start[g] = 0; }
+    dim3 grid((unsigned)((N + 127) / 128), (unsigned)G), block(512);
+#define MDY_STRIP(MT)                                                                                              \
+    hipLaunchKernelGGL((fp8_gemm_strip_kernel<MT, OUT>), grid, block, 0, stream, a, a_s, (int)as_rs, (int)as_cs, as_bytes, b, \
+                       b_s, c, bias, N, K, tbl)
+    if (max_rows <= 16) MDY_STRIP(1);
+    else if (max_rows <= 32) MDY_STRIP(2);
+    else if (max_rows <= 48) MDY_STRIP(3);
+    else MDY_STRIP(4);
+#undef MDY_STRIP
+    return (int)hipGetLastError();
+}
+
+// few rows per group and enough 128-column strips to fill the CUs without splitting K (with a handful of rows the
+// 16-column kernel re-reads so little of a that it stays ahead)
+static bool strip_pays(int64_t max_rows, int64_t strips) { return max_rows > 4 && max_rows <= 64 && strips >= 200; }
+
+template <typename OUT>
 static int dispatch(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, const uint8_t* b,
                     const float* b_s, OUT* c, const uint16_t* bias, int M, int N, int K, hipStream_t stream) {
     const int KB = (K + 127) / 128;
@@ -542,6 +698,10 @@ static int dispatch(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t a
         hipLaunchKernelGGL((fp8_gemm_scalar_kernel<OUT>), grid, dim3(256), 0, stream, a, a_s, as_rs, as_cs, b, b_s, c,
                            bias, M, N, K);
         return (int)hipGetLastError();
+    }
+    if (M <= 64 && big_ok && strip_pays(M, (N + 127) / 128)) {
+        const int64_t one = M;
+        return launch_strip<OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, &one, 1, M, N, K, stream);
     }
     if (M <= 64) {
         // one workgroup streams 16 weight columns against MT row sub-tiles; every workgroup re-reads its rows of
@@ -624,7 +784,14 @@ static int dispatch_grouped(const uint8_t* a, const float* a_s, int64_t as_rs, i
                           as_extent < ((int64_t)1 << 31) && G <= kMaxGroups;
     if (tiled_ok) {
         bool all256 = true;
-        for (int g = 0; g < G; ++g) all256 = all256 && (m_splits[g] % 256 == 0);
+        int64_t max_rows = 0;
+        for (int g = 0; g < G; ++g) {
+            all256 = all256 && (m_splits[g] % 256 == 0);
+            max_rows = m_splits[g] > max_rows ? m_splits[g] : max_rows;
+        }
+        if (strip_pays(max_rows, (int64_t)G * ((N + 127) / 128)))
+            return launch_strip<OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, m_splits, G, (int)max_rows, N, K,
+                                     stream);
         if (all256)
             return launch_grouped<256, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, m_splits, G, N, K, stream);
         return launch_grouped<128, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, m_splits, G, N, K, stream);

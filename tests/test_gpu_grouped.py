@@ -70,6 +70,21 @@ def test_grouped_gemm_exact_integer(m_splits, N, K):
     exact_grouped_case(m_splits, N, K, sum(m_splits) + N + K, call_f32)
 
 
+@pytest.mark.parametrize("m_splits,N,K", [([1, 64, 0, 17, 33, 48, 16, 5], 3300, 896),    # ragged rows and columns, K tail step
+                                          ([16] * 40, 640, 128),                          # one K block
+                                          ([64] * 4, 6400, 1152)])
+def test_grouped_gemm_exact_integer_strip_kernel(m_splits, N, K):
+    """<= 64 rows per group and >= 200 strips of 128 columns: the weight-streaming strip kernel runs."""
+    assert max(m_splits) <= 64 and len(m_splits) * ((N + 127) // 128) >= 200
+    exact_grouped_case(m_splits, N, K, 3 * sum(m_splits) + N + K, call_f32)
+
+
+def test_dense_wide_weight_exact_integer_strip_kernel():
+    from tests.test_gpu_gemm import test_gemm_exact_integer_cases_all_kernels as dense_case
+    dense_case(40, 25640, 640)       # 201 strips, 5 K blocks (two steps, the second partly past K), ragged N
+    dense_case(5, 25600, 256)
+
+
 def test_grouped_gemm_exact_integer_per_group_fallback():
     # more groups than the single-launch table holds, and K not a multiple of 128 is rejected by the MFMA path
     exact_grouped_case([2] * 300, 48, 128, 7, call_f32)
@@ -93,6 +108,16 @@ def test_grouped_matmul_against_oracle_with_bias_and_column_major_scales():
     ref = O.fp8_grouped_matmul(ra[:M], rsa[:M], rb, rsb, m_splits)
     assert out.dtype == torch.bfloat16 and out.shape == (M, N)
     assert torch.allclose(out.float().cpu(), ref.float(), rtol=RTOL, atol=ATOL)
+    # decode-like split of the same rows (strip kernel): 8 experts would not fill it, 64 small ones do
+    small = [16] * 64
+    Ms = sum(small)
+    qb64, sb64 = qb.repeat(11, 1, 1)[:64].contiguous(), sb.repeat(11, 1, 1)[:64].contiguous()
+    outs = m.fp8_grouped_matmul(qa[:Ms], sa[:Ms], qb64, sb64, small, bias=bias.repeat(11, 1)[:64].contiguous().to(DEV))
+    refs = O.fp8_grouped_matmul(ra[:Ms], rsa[:Ms], rb.repeat(11, 1, 1)[:64], rsb.repeat(11, 1, 1)[:64], small,
+                                bias=bias.repeat(11, 1)[:64])
+    rows_s = torch.repeat_interleave(torch.arange(64), torch.tensor(small))
+    mag_s = torch.maximum(refs.float().abs(), (refs.float() - bias.repeat(11, 1)[:64].float()[rows_s]).abs())
+    assert bool(((outs.float().cpu() - refs.float()).abs() <= ATOL + RTOL * mag_s).all())
     outb = m.fp8_grouped_matmul(qa[:M], sa[:M], qb, sb, m_splits, bias=bias.to(DEV))
     refb = O.fp8_grouped_matmul(ra[:M], rsa[:M], rb, rsb, m_splits, bias=bias)
     rows = torch.repeat_interleave(torch.arange(G), torch.tensor(m_splits))
