@@ -1,0 +1,138 @@
+"""Operands beyond 2^31 elements / 2^32 bytes: every kernel must address them with 64-bit offsets.
+Inputs are generated on the device (they are too large to ship from the host); the oracle checks
+slabs of rows at the start, across the 2^31-element / 2^32-byte boundary and at the end, and a
+device-side restatement of the scale formula checks every scale."""
+import numpy as np
+import pytest
+import torch
+
+import mdy_triton_amd as m
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+FP8 = torch.float8_e4m3fn
+DEV = "cuda:0"
+M_BIG, K_BIG = 36864, 65536          # 2.4e9 elements; element 2^31 is the first of row 32768
+
+
+def u8(t):
+    return t.contiguous().view(torch.uint8).cpu().numpy()
+
+
+def big_bf16(rows, cols, seed):
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    x = torch.empty(rows, cols, dtype=torch.bfloat16, device=DEV)
+    for r in range(0, rows, 4096):
+        x[r:r + 4096].normal_(generator=g)
+        x[r:r + 4096] *= float(1 + (r // 4096) % 7)        # slabs differ in magnitude as well
+    return x
+
+
+H = 256                                # slab height (the training quantizers pad rows to 256)
+
+
+def slabs(rows, boundary_row):
+    """256-aligned slabs of H rows: first, the two around the boundary, last."""
+    b = boundary_row // H * H
+    return [0, b - H, b, rows - H]
+
+
+@pytest.fixture(scope="module")
+def x_big():
+    x = big_bf16(M_BIG, K_BIG, 11)
+    yield x
+    del x
+    torch.cuda.empty_cache()
+
+
+def test_act_quant_beyond_2g_elements(x_big):
+    y, s = m.act_quant(x_big)
+    assert y.shape == x_big.shape and s.shape == (M_BIG, K_BIG // 128)
+    # every scale: the group maximum comes from the device (exact), the IEEE division from the host
+    for r in range(0, M_BIG, 8192):
+        amax = x_big[r:r + 8192].view(-1, K_BIG // 128, 128).abs().amax(-1).float().cpu()
+        assert torch.equal(s[r:r + 8192].cpu(), amax / 448.0), r
+    for r in slabs(M_BIG, 32768):
+        yr, sr = O.act_quant(x_big[r:r + H].cpu())
+        assert np.array_equal(u8(y[r:r + H]), u8(yr)), r
+        assert torch.equal(s[r:r + H].cpu(), sr), r
+
+
+def test_training_quantizers_beyond_2g_elements(x_big):
+    for fn, ofn in ((m.quant_input, lambda t: O.quant_input(t, only_forward=False)),
+                    (m.quant_grad_output, O.quant_grad_output)):
+        got = fn(x_big, only_forward=False) if fn is m.quant_input else fn(x_big)
+        y, s, y_t, s_t = got
+        assert y.shape == (M_BIG, K_BIG) and y_t.shape == (K_BIG, M_BIG)
+        for r in slabs(M_BIG, 32768):
+            yr, sr, ytr, str_ = ofn(x_big[r:r + H].cpu())
+            assert np.array_equal(u8(y[r:r + H]), u8(yr)), r
+            assert torch.equal(s[r:r + H].cpu(), sr), r
+            assert np.array_equal(u8(y_t[:, r:r + H]), u8(ytr)), r
+            # [K, M/128] (one scale per column and 128 rows) or [K/128, M/128] (one per 128x128 block)
+            assert torch.equal(s_t[:, r // 128:(r + H) // 128].cpu(), str_), r
+        del got, y, s, y_t, s_t
+        torch.cuda.empty_cache()
+
+
+def test_weight_quant_and_dequant_beyond_2g_elements(x_big):
+    w = x_big                                              # any bf16 matrix with 128-aligned sides
+    y, s = m.weight_quant_block(w)
+    assert s.shape == (M_BIG // 128, K_BIG // 128)
+    for r in slabs(M_BIG, 32768):
+        yr, sr = O.weight_quant_block(w[r:r + H].cpu())
+        assert np.array_equal(u8(y[r:r + H]), u8(yr)), r
+        assert torch.equal(s[r // 128:(r + H) // 128].cpu(), sr), r
+    for dt in (torch.bfloat16, torch.float32):
+        d = m.weight_dequant(y, s, out_dtype=dt)
+        assert d.shape == w.shape and d.dtype == dt
+        for r in slabs(M_BIG, 32768):
+            dr = O.weight_dequant(y[r:r + H].cpu(), s[r // 128:(r + H) // 128].cpu(), dtype=dt)
+            assert torch.equal(d[r:r + H].cpu(), dr), r
+        # everything: the same fp32 product, rounded once to the output type, restated on the device
+        for r in range(0, M_BIG, 4096):
+            ref = (y[r:r + 4096].float().view(32, 128, K_BIG // 128, 128) *
+                   s[r // 128:r // 128 + 32][:, None, :, None]).view(4096, K_BIG).to(dt)
+            assert torch.equal(d[r:r + 4096], ref), r
+        del d
+        torch.cuda.empty_cache()
+
+
+def test_fp8_gemm_operand_beyond_4g_bytes():
+    """a is 66560 x 65536 bytes: byte 2^32 is the first of row 65536.  Small integers and power-of-two
+    scales keep every sum exact in fp32, so slabs are compared bit for bit with an integer computation."""
+    M, N, K = 66560, 256, 65536
+    KB = K // 128
+    g = torch.Generator(device=DEV).manual_seed(5)
+    a = torch.empty(M, K, dtype=FP8, device=DEV)
+    for r in range(0, M, 8192):
+        a[r:r + 8192] = torch.randint(-2, 3, (min(8192, M - r), K), device=DEV, generator=g, dtype=torch.int8).float().to(FP8)
+    b = torch.randint(-2, 3, (N, K), device=DEV, generator=g, dtype=torch.int8).float().to(FP8)
+    ae = torch.randint(-1, 2, (M, KB), device=DEV, generator=g)
+    be = torch.randint(-1, 2, (N // 128, KB), device=DEV, generator=g)
+    c = m.fp8_gemm(a, torch.exp2(ae.float()), b, torch.exp2(be.float()), out_dtype=torch.float32)
+    assert c.shape == (M, N)
+    bd = b.cpu().float().double().view(N, KB, 128)
+    for r in slabs(M, 65536):
+        ad = a[r:r + H].cpu().float().double().view(H, KB, 128)
+        part = torch.einsum("mkc,nkc->kmn", ad, bd)                          # [KB, H, N]
+        e = ae[r:r + H].cpu().t()[:, :, None] + be.cpu()[torch.arange(N) // 128].t()[:, None, :]
+        ref = (part * torch.exp2(e.double())).sum(0)
+        assert torch.equal(c[r:r + H].cpu().double(), ref), r
+
+
+def test_swiglu_beyond_4g_bytes(x_big):
+    """The kernels are deterministic, so a slab of the large run must equal the same kernel run on that
+    slab alone (the slab runs are what the small parity tests compare with the oracle)."""
+    y, s, act = m.silu_act_quant(x_big, "gate-up", return_act=True)
+    assert act.shape == (M_BIG, K_BIG // 2) and y.shape == act.shape and s.shape == (M_BIG, K_BIG // 256)
+    assert torch.equal(act, m.silu_fwd(x_big, "gate-up"))
+    dy = act                                               # any bf16 [M, N]
+    dx = m.silu_bwd(dy, x_big, "gate-up")
+    assert dx.shape == x_big.shape
+    for r in slabs(M_BIG, 32768):
+        xs = x_big[r:r + H].contiguous()
+        ys, ss, acts = m.silu_act_quant(xs, "gate-up", return_act=True)
+        assert torch.equal(act[r:r + H], acts), r
+        assert np.array_equal(u8(y[r:r + H]), u8(ys)) and torch.equal(s[r:r + H], ss), r
+        assert torch.equal(dx[r:r + H], m.silu_bwd(dy[r:r + H].contiguous(), xs, "gate-up")), r
