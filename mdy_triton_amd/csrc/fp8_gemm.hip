@@ -95,14 +95,14 @@ __device__ __forceinline__ void dma4(const intx4& rsrc, int voff, int soff, uint
 // workgroups that copy the same panels (those with the same tile row / tile column).
 //
 // Schedule of one K block (NT = TI*TJ MFMA slots, each followed DEPTH slots later by its 4 FMAs):
-//   slots 0..      the last copies of K block kb+1 (those that did not fit into the tail below), one per slot,
-//                  then one "duty touch" load for K block kb+3;
+//   slots 0..      the last copies of K block kb+1 (those that did not fit into the tail below), one per GAP
+//                  slots, then one "duty touch" load for K block kb+3;
 //   slot TB        = first MFMA of the last streamed fragment: every LDS read of this K block has been
 //                  consumed, so the wave waits for its copies of kb+1 and meets the others at THE barrier
 //                  of the K block; behind it buffer `cur` is free and buffer `cur^1` is complete;
 //   slots TB..     while the last MFMAs and FMAs of kb still run: reload the held fragments, the first
 //                  streamed fragment and the scales from buffer cur^1, and issue the first copies of kb+2
-//                  into buffer cur, one per slot.
+//                  into buffer cur, one per GAP slots.
 // So the LDS latency after the barrier and the issue time of the copies sit in the shadow of the matrix
 // pipe instead of in front of the first MFMA of the next K block.
 template <int BM, int BN, int WGM, int WGN, typename OUT>
@@ -124,11 +124,19 @@ __device__ __forceinline__ void fp8_gemm_tile(
     constexpr int NT = TI * TJ;
     constexpr int NDMA = 1 + A_PASSES + B_PASSES;       // copies per K block and wave: scales, A passes, B passes
     constexpr int TB = NT - NH;                         // slot of the barrier
-    constexpr int TAIL = NT + DEPTH - 1 - TB;           // slots behind the barrier
-    constexpr int FIRST = TAIL < NDMA ? TAIL : NDMA;    // copies of K block kb+2 issued in the tail of kb
+    constexpr int NSLOT = NT + DEPTH;                   // slots of a K block (the last DEPTH hold FMAs only)
+    // Copy j of a K block goes out in slot TB+1 + GAP*j, counted on from the barrier of the block two before it
+    // and running over into the first slots of the next block.  With 8 waves one copy per slot and wave is
+    // twice what the CU's address unit takes (64 lanes x 16 bytes = 16 clocks each, a slot is 64 clocks for
+    // the two waves of a SIMD): the waves then queue on the copy instruction and their MFMAs behind it wait.
+    // Measured: 256x256 tiles 1-5 % faster with every second slot, 128x256 tiles (half as many slots) not.
+    constexpr int GAP = (WAVES >= 8 && NT >= 32) ? 2 : 1;
+    constexpr int TAIL = (NSLOT - TB - 1 + GAP - 1) / GAP;   // copies that still fit behind the barrier
+    constexpr int FIRST = TAIL < NDMA ? TAIL : NDMA;         // copies of K block kb+2 issued in the tail of kb
+    constexpr int TOUCH = FIRST < NDMA ? TB + 1 + GAP * (NDMA - 1) - NSLOT + 1 : 0;   // slot after the last copy
     constexpr int TD = 3;                               // duty touches run this many K blocks ahead
     static_assert(NS % 2 == 0 && NS >= 2, "the first streamed fragment of the next K block reuses queue slot 0");
-    static_assert(NDMA - FIRST + 1 <= TB, "not enough slots in front of the barrier");
+    static_assert(TOUCH < TB, "not enough slots in front of the barrier");
 
     __shared__ __attribute__((aligned(1024))) uint8_t lds_a[2][BM * 128];
     __shared__ __attribute__((aligned(1024))) uint8_t lds_b[2][BN * 128];
@@ -259,9 +267,13 @@ __device__ __forceinline__ void fp8_gemm_tile(
                 acc[i][j][2] = __builtin_fmaf(q[2], sc[i], acc[i][j][2]);
                 acc[i][j][3] = __builtin_fmaf(q[3], sc[i], acc[i][j][3]);
             }
-            if (t < NDMA - FIRST) issue(FIRST + t, kb + 1, cur ^ 1);
-            if (t == NDMA - FIRST) dma4(rt, touch_off, kb + TD < KB ? (kb + TD) * 128 : rt[2], ld_base + 256);
-            if (t > TB && t - TB - 1 < FIRST) issue(t - TB - 1, kb + 2, cur);
+#pragma unroll
+            for (int j = 0; j < NDMA; ++j) {
+                const int v = TB + 1 + GAP * j;
+                if (v < NSLOT && v == t) issue(j, kb + 2, cur);                 // behind the barrier: buffer cur is free
+                if (v >= NSLOT && v - NSLOT == t) issue(j, kb + 1, cur ^ 1);    // the rest of the block started in kb-1
+            }
+            if (t == TOUCH) dma4(rt, touch_off, kb + TD < KB ? (kb + TD) * 128 : rt[2], ld_base + 256);
             __builtin_amdgcn_sched_barrier(0);  // keep the MFMA / FMA / ds_read / copy interleaving as written
         }
 #pragma unroll
