@@ -105,7 +105,7 @@ __device__ __forceinline__ void dma4(const intx4& rsrc, int voff, int soff, uint
 //                  into buffer cur, one per GAP slots.
 // So the LDS latency after the barrier and the issue time of the copies sit in the shadow of the matrix
 // pipe instead of in front of the first MFMA of the next K block.
-template <int BM, int BN, int WGM, int WGN, typename OUT>
+template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT>
 __device__ __forceinline__ void fp8_gemm_tile(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
@@ -134,14 +134,20 @@ __device__ __forceinline__ void fp8_gemm_tile(
     constexpr int TAIL = (NSLOT - TB - 1 + GAP - 1) / GAP;   // copies that still fit behind the barrier
     constexpr int FIRST = TAIL < NDMA ? TAIL : NDMA;         // copies of K block kb+2 issued in the tail of kb
     constexpr int TOUCH = FIRST < NDMA ? TB + 1 + GAP * (NDMA - 1) - NSLOT + 1 : 0;   // slot after the last copy
-    constexpr int TD = 3;                               // duty touches run this many K blocks ahead
+    constexpr int TD = STAGES + 1;                      // duty touches run this many K blocks ahead (in front of the copies)
+    // loads younger than the last copy of K block kb+1 when the wave waits for it in K block kb: the copies of
+    // blocks kb+2 .. kb+STAGES-1 and one touch per K block since (loads complete in order, so vmcnt(YOUNGER)
+    // means "block kb+1 has landed")
+    constexpr int YOUNGER = (STAGES - 2) * NDMA + STAGES - 1;
+    static_assert(STAGES >= 2 && YOUNGER <= 63, "vmcnt is a 6-bit counter");
     static_assert(NS % 2 == 0 && NS >= 2, "the first streamed fragment of the next K block reuses queue slot 0");
     static_assert(TOUCH < TB, "not enough slots in front of the barrier");
 
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_a[2][BM * 128];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_b[2][BN * 128];
-    __shared__ __attribute__((aligned(256))) float lds_s[2][BM];
-    __shared__ __attribute__((aligned(256))) float lds_bs[BN / 128][512];   // weight scales of the tile, all K blocks
+    constexpr int NBS = (BN + 127) / 128;
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a[STAGES][BM * 128];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_b[STAGES][BN * 128];
+    __shared__ __attribute__((aligned(256))) float lds_s[STAGES][BM];
+    __shared__ __attribute__((aligned(256))) float lds_bs[NBS][512];   // weight scales of the tile, all K blocks
     __shared__ __attribute__((aligned(256))) uint8_t lds_dummy[WAVES * 512];   // target of copies that must go nowhere
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -206,15 +212,25 @@ __device__ __forceinline__ void fp8_gemm_tile(
         return intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     };
 
-    // ---- prologue: the tile's weight scales, K block 0, the registers of step 0, the first copies of K block 1
-    if (wave < BN / 128) {
+    auto touch = [&](int kb) { dma4(rt, touch_off, kb < KB ? kb * 128 : rt[2], ld_base + 256); };
+
+    // ---- prologue: the tile's weight scales, then the copies in the order the K loop keeps up: for every K
+    // block its first FIRST copies, the rest, one touch; K blocks 0 .. STAGES-2 whole and the first copies of
+    // block STAGES-1.  Then wait for block 0 and load the registers of step 0.
+    if (wave < NBS) {
         const int nb = min((n0 >> 7) + wave, ((N + 127) >> 7) - 1);
         const intx4 rbs = make_rsrc(b_s + (size_t)nb * KB, (uint32_t)KB * 4u);
         for (int cc = 0; cc < KB; cc += 64) dma4(rbs, lane * 4, cc * 4, lds_addr(&lds_bs[wave][cc]));
     }
 #pragma unroll
-    for (int i = 0; i < NDMA; ++i) issue(i, 0, 0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    for (int blk = 0; blk < STAGES - 1; ++blk) {
+#pragma unroll
+        for (int i = 0; i < NDMA; ++i) issue(i, blk, blk);
+        touch(blk + 1 + TD - STAGES);
+    }
+#pragma unroll
+    for (int i = 0; i < FIRST; ++i) issue(i, STAGES - 1, STAGES - 1);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 2) * (NDMA + 1) + 1 + FIRST) : "memory");
     __syncthreads();
     intx8 fh[NH], fx[2];
     float sc[TI];
@@ -226,15 +242,15 @@ __device__ __forceinline__ void fp8_gemm_tile(
         for (int i = 0; i < TI; ++i) sc[i] = lds_s[0][s_rd + i * 16] * sb;
     }
     fx[0] = read_frag(HOLD_A ? lds_b[0] : lds_a[0], x0, x1, 0);
-#pragma unroll
-    for (int i = 0; i < FIRST; ++i) issue(i, 1, 1);
 
+    int cur = 0;                                             // buffer of K block kb: kb % STAGES
     for (int kb = 0; kb < KB; ++kb) {
-        const int cur = kb & 1;
+        const int nxt = cur + 1 == STAGES ? 0 : cur + 1;     // buffer of K block kb+1
+        const int last = cur == 0 ? STAGES - 1 : cur - 1;    // buffer of K block kb+STAGES-1
         const uint8_t* lx = HOLD_A ? lds_b[cur] : lds_a[cur];            // streamed operand of this K block
-        const uint8_t* lh_n = HOLD_A ? lds_a[cur ^ 1] : lds_b[cur ^ 1];  // operands and scales of the next one
-        const uint8_t* lx_n = HOLD_A ? lds_b[cur ^ 1] : lds_a[cur ^ 1];
-        const float* ls_n = lds_s[cur ^ 1];
+        const uint8_t* lh_n = HOLD_A ? lds_a[nxt] : lds_b[nxt];          // operands and scales of the next one
+        const uint8_t* lx_n = HOLD_A ? lds_b[nxt] : lds_a[nxt];
+        const float* ls_n = lds_s[nxt];
         float sc_n[TI];
         floatx4 p[DEPTH + 1];
 #pragma unroll
@@ -248,8 +264,8 @@ __device__ __forceinline__ void fp8_gemm_tile(
                 // rows of the MFMA = n (B panel), columns = m (A panel)
                 p[t % (DEPTH + 1)] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb_, fa_, zero, 0, 0, 0, 0, 0, 0);
                 if (t == TB) {
-                    // the only outstanding load that may stay in flight is this step's touch (the youngest)
-                    asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+                    // K block kb+1 has landed once only the younger loads are left in flight
+                    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(YOUNGER) : "memory");
                     __syncthreads();
                     fx[0] = read_frag(lx_n, x0, x1, 0);      // queue slot 0 was last used by streamed fragment NS-2
                     const float sb = my_bs[min(kb + 1, KB - 1)];
@@ -270,14 +286,15 @@ __device__ __forceinline__ void fp8_gemm_tile(
 #pragma unroll
             for (int j = 0; j < NDMA; ++j) {
                 const int v = TB + 1 + GAP * j;
-                if (v < NSLOT && v == t) issue(j, kb + 2, cur);                 // behind the barrier: buffer cur is free
-                if (v >= NSLOT && v - NSLOT == t) issue(j, kb + 1, cur ^ 1);    // the rest of the block started in kb-1
+                if (v < NSLOT && v == t) issue(j, kb + STAGES, cur);                    // behind the barrier: buffer cur is free
+                if (v >= NSLOT && v - NSLOT == t) issue(j, kb + STAGES - 1, last);      // the rest of the block started in kb-1
             }
-            if (t == TOUCH) dma4(rt, touch_off, kb + TD < KB ? (kb + TD) * 128 : rt[2], ld_base + 256);
+            if (t == TOUCH) touch(kb + TD);
             __builtin_amdgcn_sched_barrier(0);  // keep the MFMA / FMA / ds_read / copy interleaving as written
         }
 #pragma unroll
         for (int i = 0; i < TI; ++i) sc[i] = sc_n[i];
+        cur = nxt;
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing may still be writing LDS when the wave ends
 
@@ -314,14 +331,14 @@ __device__ __forceinline__ void tile_of(int local, int tiles_m, int tiles_n, int
     tn = (local % (GM * tiles_n)) / gsz;
 }
 
-template <int BM, int BN, int WGM, int WGN, typename OUT>
+template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT>
 __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
     const uint16_t* __restrict__ bias, int M, int N, int K, int ldc, int tiles_m, int tiles_n) {
     int tm, tn;
     tile_of(xcd_contiguous(blockIdx.x, tiles_m * tiles_n), tiles_m, tiles_n, tm, tn);
-    fp8_gemm_tile<BM, BN, WGM, WGN, OUT>(a, a_s, as_rs, as_cs, as_bytes, b, b_s, c, bias, tm * BM, M, M, tn * BN, N, K, ldc, tn & 7,
+    fp8_gemm_tile<BM, BN, WGM, WGN, STAGES, OUT>(a, a_s, as_rs, as_cs, as_bytes, b, b_s, c, bias, tm * BM, M, M, tn * BN, N, K, ldc, tn & 7,
                                          tm & 3);
 }
 
@@ -359,7 +376,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_grouped_gemm_kernel(
     tile_of(pid - tbl.tile_start[g] * tiles_n, tiles_m, tiles_n, tm, tn);
     const int KB = K >> 7, NB = (N + 127) >> 7;
     const int r0 = __builtin_amdgcn_readfirstlane(tbl.row_start[g]), r1 = __builtin_amdgcn_readfirstlane(tbl.row_start[g + 1]);
-    fp8_gemm_tile<BM, BN, WGM, WGN, OUT>(a, a_s, as_rs, as_cs, as_bytes, b + (size_t)g * N * K,
+    fp8_gemm_tile<BM, BN, WGM, WGN, 2, OUT>(a, a_s, as_rs, as_cs, as_bytes, b + (size_t)g * N * K,
                                          b_s + (size_t)g * NB * KB, c, bias ? bias + (size_t)g * N : nullptr,
                                          __builtin_amdgcn_readfirstlane(r0 + tm * BM), r1,
                                          __builtin_amdgcn_readfirstlane(tbl.row_start[G]), __builtin_amdgcn_readfirstlane(tn * BN), N, K, N,
@@ -636,13 +653,13 @@ __global__ __launch_bounds__(256) void fp8_gemm_scalar_kernel(const uint8_t* __r
         reinterpret_cast<float*>(c)[(int64_t)m * N + n] = acc;
 }
 
-template <int BM, int BN, int WGM, int WGN, typename OUT>
+template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT>
 static int launch_mfma(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, uint32_t as_bytes,
                        const uint8_t* b, const float* b_s, OUT* c, const uint16_t* bias, int M, int N, int K,
                        int ldc, hipStream_t stream) {
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     dim3 grid((unsigned)(tiles_m * tiles_n)), block(WGM * WGN * 64);
-    hipLaunchKernelGGL((fp8_gemm_mfma_kernel<BM, BN, WGM, WGN, OUT>), grid, block, 0, stream, a, a_s, (int)as_rs,
+    hipLaunchKernelGGL((fp8_gemm_mfma_kernel<BM, BN, WGM, WGN, STAGES, OUT>), grid, block, 0, stream, a, a_s, (int)as_rs,
                        (int)as_cs, as_bytes, b, b_s, c, bias, M, N, K, ldc, tiles_m, tiles_n);
     return (int)hipGetLastError();
 }
@@ -665,6 +682,20 @@ static int main_tile_columns(int tiles_m, int tiles_n) {
     const double cost_split = (double)rounds_main + 0.6 * (double)((rem_small + kCUs - 1) / kCUs);
     const double cost_plain = (double)((total + kCUs - 1) / kCUs);
     return cost_split < cost_plain - 0.05 ? cols_main : tiles_n;
+}
+
+// Tile and ring depth for shapes with fewer than 200 tiles of 256x256:
+//   0: 128x128, 2 K blocks in LDS (two workgroups share a CU)   1: 128x128, 4 K blocks (one workgroup per CU)
+//   2: 128x64, 6 K blocks                                       3: 64x64, 8 K blocks
+// Measured rule: the smallest tile that still gives every workgroup a CU of its own (the time of these
+// shapes goes with the bytes each CU has to pull, not with its MFMAs), and the ring as deep as LDS allows.
+static int few_tiles_config(int M, int N) {
+    const long rows128 = (M + 127) / 128, rows64 = (M + 63) / 64;
+    const long cols128 = (N + 127) / 128, cols64 = (N + 63) / 64;
+    if (rows64 * cols64 <= kCUs) return 3;
+    if (rows128 * cols64 <= kCUs) return 2;
+    if (rows128 * cols128 <= kCUs) return 1;
+    return 0;
 }
 
 template <typename OUT>
@@ -738,15 +769,27 @@ static int dispatch(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t a
         const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
         const int cols_main = main_tile_columns(tiles_m, tiles_n);
         const int n_main = cols_main < tiles_n ? cols_main * 256 : N;
-        int rc = launch_mfma<256, 256, 2, 4, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, n_main, K, N,
+        int rc = launch_mfma<256, 256, 2, 4, 2, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, n_main, K, N,
                                                   stream);
         if (rc != 0 || n_main == N) return rc;
-        // remaining columns as 128x256 tiles; n_main is a multiple of 256, so every pointer below keeps its alignment
-        return launch_mfma<128, 256, 2, 4, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b + (size_t)n_main * K,
+        // remaining columns as 128x256 tiles (LDS has room for a ring of 3 K blocks there: 1-2 % of the whole
+        // call); n_main is a multiple of 256, so every pointer below keeps its alignment
+        return launch_mfma<128, 256, 2, 4, 3, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b + (size_t)n_main * K,
                                                 b_s + (size_t)(n_main >> 7) * KB, c + n_main,
                                                 bias ? bias + n_main : nullptr, M, N - n_main, K, N, stream);
     }
-    return launch_mfma<128, 128, 2, 2, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
+    // Fewer tiles than that: the workgroups no longer fill the CUs, every K block's copy latency shows, and
+    // the time goes with K.  Use the LDS that the missing co-resident workgroups leave free for a deeper ring of
+    // K blocks in flight, and smaller tiles when even 128x128 tiles leave most CUs idle.
+#define MDY_FEW(BM_, BN_, ST_)                                                                                       \
+    return launch_mfma<BM_, BN_, 2, 2, ST_, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream)
+    switch (few_tiles_config(M, N)) {
+        case 1: MDY_FEW(128, 128, 4);
+        case 2: MDY_FEW(128, 64, 6);
+        case 3: MDY_FEW(64, 64, 8);
+        default: MDY_FEW(128, 128, 2);
+    }
+#undef MDY_FEW
 }
 
 int launch_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,
