@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define MDY_FP8_ABI_VERSION 1
+#define MDY_FP8_ABI_VERSION 2
 
 /* error codes (negative = argument rejected before any launch) */
 #define MDY_OK 0
@@ -154,6 +154,22 @@ int mdy_weight_dequant(const void* x, const float* s, void* y, int64_t N, int64_
 int mdy_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
                     const void* b, const float* b_s, void* c, const void* bias, int64_t M, int64_t N,
                     int64_t K, int out_dtype, void* stream);
+
+/* The same GEMM with a caller-provided scratch buffer.  Shapes whose output tiles do not fill the GPU
+ * (roughly 16 < M <= 1024 against a long K: small-batch prefill, large-batch decode) are cut along K as
+ * well; the fp32 partial sums of the K slices go through `workspace` and are added in a fixed order, so the
+ * result is deterministic, but it may differ in the last bit from mdy_fp8_gemm_nt (another summation order).
+ * No counterpart in the reference (its Triton kernel / DeepGEMM never split K); the Python wrappers fp8_gemm
+ * and fp8_matmul call it with a torch-allocated buffer.
+ *
+ *   mdy_fp8_gemm_workspace_bytes(M, N, K)  bytes of workspace with which this shape runs split (0: it never does)
+ *   workspace        device memory, 16-byte aligned, workspace_bytes long; may be NULL / too small: the call
+ *                    then is mdy_fp8_gemm_nt.  Calls that overlap in time need separate workspaces.
+ */
+int64_t mdy_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int mdy_fp8_gemm_nt_ws(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
+                       const void* b, const float* b_s, void* c, const void* bias, int64_t M, int64_t N,
+                       int64_t K, int out_dtype, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Grouped (mixture-of-experts) block-scaled FP8 GEMM, NT layout: the rows of a are split into G
  * consecutive groups of m_splits[g] rows and group g is multiplied with its own weight,

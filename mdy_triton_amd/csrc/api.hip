@@ -174,6 +174,30 @@ int mdy_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int6
                     "fp8_gemm_nt");
 }
 
+int64_t mdy_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K < 1 || M > kMaxDim || N > kMaxDim || K > kMaxDim) return 0;
+    return mdy::fp8_gemm_workspace_bytes(M, N, K);
+}
+
+int mdy_fp8_gemm_nt_ws(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,
+                       const float* b_s, void* c, const void* bias, int64_t M, int64_t N, int64_t K, int out_dtype,
+                       void* workspace, int64_t workspace_bytes, void* stream) {
+    if (out_dtype != MDY_DT_BF16 && out_dtype != MDY_DT_F32) return fail(MDY_E_DTYPE, "fp8_gemm_nt_ws: unknown out_dtype %d", out_dtype);
+    if (M < 0 || N < 0 || K < 1 || M > kMaxDim || N > kMaxDim || K > kMaxDim)
+        return fail(MDY_E_SHAPE, "fp8_gemm_nt_ws: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+    if ((M + 15) / 16 > 65535) return fail(MDY_E_SHAPE, "fp8_gemm_nt_ws: M too large");
+    if (workspace_bytes < 0) return fail(MDY_E_SHAPE, "fp8_gemm_nt_ws: workspace_bytes < 0");
+    if (M == 0 || N == 0) return 0;
+    if (!a || !a_s || !b || !b_s || !c) return fail(MDY_E_NULL, "fp8_gemm_nt_ws: null pointer");
+    if (!aligned(c, out_dtype == MDY_DT_BF16 ? 2 : 4) || !aligned(a_s, 4) || !aligned(b_s, 4) || (bias && !aligned(bias, 2)))
+        return fail(MDY_E_ALIGN, "fp8_gemm_nt_ws: misaligned pointer");
+    if (workspace && !aligned(workspace, 16)) return fail(MDY_E_ALIGN, "fp8_gemm_nt_ws: workspace must be 16-byte aligned");
+    if (int e = check_device()) return e;
+    return launched(mdy::launch_fp8_gemm_nt_ws(a, a_s, as_row_stride, as_col_stride, b, b_s, c, bias, M, N, K, out_dtype,
+                                               workspace, workspace_bytes, static_cast<hipStream_t>(stream)),
+                    "fp8_gemm_nt_ws");
+}
+
 int mdy_fp8_grouped_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,
                             const float* b_s, void* c, const void* bias, const int64_t* m_splits, int64_t G, int64_t N,
                             int64_t K, int out_dtype, void* stream) {

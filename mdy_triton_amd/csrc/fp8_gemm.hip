@@ -89,7 +89,8 @@ __device__ __forceinline__ void dma4(const intx4& rsrc, int voff, int soff, uint
 
 // One BM x BN tile of C: WGM x WGN waves, each wave (BM/WGM) x (BN/WGN).
 //   rows m0 .. min(m0+BM, m_end) of a (m_end = end of the matrix, or of the expert group the tile belongs to),
-//   columns n0 .. of b / b_s / bias (already offset to the group's weight), K % 128 == 0, K <= 65536.
+//   columns n0 .. of b / b_s / bias (already offset to the group's weight), K % 128 == 0, K <= 65536,
+//   K blocks kb0 .. kb1-1 of them (all of them except in the split-K kernel).
 // as_bytes = byte size of the addressed part of a_s (host computed, < 2^31); m_total = rows of a_s.
 // a_duty (0..7) / b_duty (0..3): which share of the A / B panel lines this workgroup pre-touches for the
 // workgroups that copy the same panels (those with the same tile row / tile column).
@@ -110,7 +111,7 @@ __device__ __forceinline__ void fp8_gemm_tile(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
     const uint16_t* __restrict__ bias, int m0, int m_end, int m_total, int n0, int N, int K, int ldc, int a_duty,
-    int b_duty) {
+    int b_duty, int kb0, int kb1) {
     constexpr int WAVES = WGM * WGN;
     constexpr int WM = BM / WGM, WN = BN / WGN, TI = WM / 16, TJ = WN / 16;
     constexpr int PASS_ROWS = WAVES * 8;  // rows copied by one DMA instruction of every wave
@@ -173,7 +174,7 @@ __device__ __forceinline__ void fp8_gemm_tile(
     // copy i (0: scales, then the A passes, then the B passes) of K block kb into buffer buf.  Past the last K
     // block the offsets run beyond the descriptors: no memory access, zeros into a buffer nobody reads any more.
     auto issue = [&](int i, int kb, int buf) {
-        const bool more = kb < KB;
+        const bool more = kb < kb1;
         if (i == 0)
             dma4(rs, s_voff, more ? kb * as_cs * 4 : (int)as_bytes, ls_base + buf * ls_buf);
         else if (i <= A_PASSES)
@@ -212,7 +213,7 @@ __device__ __forceinline__ void fp8_gemm_tile(
         return intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     };
 
-    auto touch = [&](int kb) { dma4(rt, touch_off, kb < KB ? kb * 128 : rt[2], ld_base + 256); };
+    auto touch = [&](int kb) { dma4(rt, touch_off, kb < kb1 ? kb * 128 : rt[2], ld_base + 256); };
 
     // ---- prologue: the tile's weight scales, then the copies in the order the K loop keeps up: for every K
     // block its first FIRST copies, the rest, one touch; K blocks 0 .. STAGES-2 whole and the first copies of
@@ -225,11 +226,11 @@ __device__ __forceinline__ void fp8_gemm_tile(
 #pragma unroll
     for (int blk = 0; blk < STAGES - 1; ++blk) {
 #pragma unroll
-        for (int i = 0; i < NDMA; ++i) issue(i, blk, blk);
-        touch(blk + 1 + TD - STAGES);
+        for (int i = 0; i < NDMA; ++i) issue(i, kb0 + blk, blk);
+        touch(kb0 + blk + 1 + TD - STAGES);
     }
 #pragma unroll
-    for (int i = 0; i < FIRST; ++i) issue(i, STAGES - 1, STAGES - 1);
+    for (int i = 0; i < FIRST; ++i) issue(i, kb0 + STAGES - 1, STAGES - 1);
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 2) * (NDMA + 1) + 1 + FIRST) : "memory");
     __syncthreads();
     intx8 fh[NH], fx[2];
@@ -237,14 +238,14 @@ __device__ __forceinline__ void fp8_gemm_tile(
 #pragma unroll
     for (int h = 0; h < NH; ++h) fh[h] = read_frag(HOLD_A ? lds_a[0] : lds_b[0], h0, h1, h);
     {
-        const float sb = my_bs[0];
+        const float sb = my_bs[kb0];
 #pragma unroll
         for (int i = 0; i < TI; ++i) sc[i] = lds_s[0][s_rd + i * 16] * sb;
     }
     fx[0] = read_frag(HOLD_A ? lds_b[0] : lds_a[0], x0, x1, 0);
 
     int cur = 0;                                             // buffer of K block kb: kb % STAGES
-    for (int kb = 0; kb < KB; ++kb) {
+    for (int kb = kb0; kb < kb1; ++kb) {
         const int nxt = cur + 1 == STAGES ? 0 : cur + 1;     // buffer of K block kb+1
         const int last = cur == 0 ? STAGES - 1 : cur - 1;    // buffer of K block kb+STAGES-1
         const uint8_t* lx = HOLD_A ? lds_b[cur] : lds_a[cur];            // streamed operand of this K block
@@ -339,7 +340,60 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
     int tm, tn;
     tile_of(xcd_contiguous(blockIdx.x, tiles_m * tiles_n), tiles_m, tiles_n, tm, tn);
     fp8_gemm_tile<BM, BN, WGM, WGN, STAGES, OUT>(a, a_s, as_rs, as_cs, as_bytes, b, b_s, c, bias, tm * BM, M, M, tn * BN, N, K, ldc, tn & 7,
-                                         tm & 3);
+                                                 tm & 3, 0, K >> 7);
+}
+
+// ---------------------------------------------------------------------------
+// Split-K: shapes whose tiles do not fill the CUs (few rows against a long K) are cut along K as well.
+// Workgroup (ks, tile) accumulates K blocks ks*kb_per .. of its tile and stores the fp32 partial sums
+// into slab ks of a caller-provided workspace [ksplit][M][N]; splitk_reduce_kernel then adds the slabs in
+// slab order (so the result does not depend on scheduling), adds the bias and converts.
+// ---------------------------------------------------------------------------
+template <int BM, int BN, int WGM, int WGN, int STAGES>
+__global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_splitk_kernel(
+    const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
+    const uint8_t* __restrict__ b, const float* __restrict__ b_s, float* __restrict__ ws, int M, int N, int K,
+    int tiles_m, int tiles_n, int ksplit, int kb_per) {
+    const int ntiles = tiles_m * tiles_n;
+    // slab-major order: the workgroups that share an XCD work on the same K range, so they share its A rows
+    const int pid = xcd_contiguous(blockIdx.x, ntiles * ksplit);
+    const int ks = __builtin_amdgcn_readfirstlane(pid / ntiles);
+    int tm, tn;
+    tile_of(pid - ks * ntiles, tiles_m, tiles_n, tm, tn);
+    const int kb0 = ks * kb_per, kb1 = min(K >> 7, kb0 + kb_per);
+    fp8_gemm_tile<BM, BN, WGM, WGN, STAGES, float>(a, a_s, as_rs, as_cs, as_bytes, b, b_s, ws + (size_t)ks * M * N, nullptr,
+                                                   tm * BM, M, M, tn * BN, N, K, N, tn & 7, tm & 3, kb0, kb1);
+}
+
+template <typename OUT, bool VEC>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, OUT* __restrict__ c,
+                                                            const uint16_t* __restrict__ bias, int64_t MN, int N,
+                                                            int ksplit) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * (VEC ? 4 : 1);
+    if (i >= MN) return;
+    if (VEC) {   // N % 4 == 0: the 4 elements lie in one row
+        float4 s = *reinterpret_cast<const float4*>(ws + i);
+        for (int k = 1; k < ksplit; ++k) {
+            const float4 v = *reinterpret_cast<const float4*>(ws + (int64_t)k * MN + i);
+            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+        }
+        if (bias != nullptr) {
+            const int n = (int)(i % N);
+            s.x += bf16_one(bias[n]); s.y += bf16_one(bias[n + 1]); s.z += bf16_one(bias[n + 2]); s.w += bf16_one(bias[n + 3]);
+        }
+        if (sizeof(OUT) == 2)
+            *reinterpret_cast<uint2*>(c + i) = make_uint2(pack2_bf16(s.x, s.y), pack2_bf16(s.z, s.w));
+        else
+            *reinterpret_cast<float4*>(c + i) = s;
+    } else {
+        float s = ws[i];
+        for (int k = 1; k < ksplit; ++k) s += ws[(int64_t)k * MN + i];
+        if (bias != nullptr) s += bf16_one(bias[i % N]);
+        if (sizeof(OUT) == 2)
+            reinterpret_cast<uint16_t*>(c)[i] = (uint16_t)(pack2_bf16(s, 0.0f) & 0xFFFFu);
+        else
+            reinterpret_cast<float*>(c)[i] = s;
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -380,7 +434,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_grouped_gemm_kernel(
                                          b_s + (size_t)g * NB * KB, c, bias ? bias + (size_t)g * N : nullptr,
                                          __builtin_amdgcn_readfirstlane(r0 + tm * BM), r1,
                                          __builtin_amdgcn_readfirstlane(tbl.row_start[G]), __builtin_amdgcn_readfirstlane(tn * BN), N, K, N,
-                                         __builtin_amdgcn_readfirstlane(tn & 7), __builtin_amdgcn_readfirstlane(tm & 3));
+                                         __builtin_amdgcn_readfirstlane(tn & 7), __builtin_amdgcn_readfirstlane(tm & 3), 0, K >> 7);
 }
 
 // ---------------------------------------------------------------------------
@@ -790,6 +844,102 @@ static int dispatch(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t a
         default: MDY_FEW(128, 128, 2);
     }
 #undef MDY_FEW
+}
+
+// ---- split-K plan: which tile, how many K slices; ksplit == 1 means "do not split"
+struct SplitPlan {
+    int config;     // 1: 128x128 tiles (ring of 4)   2: 128x64 (ring of 6)   3: 64x64 (ring of 8)
+    int ksplit;     // slabs of the workspace
+    int kb_per;     // K blocks per slab
+};
+
+static SplitPlan plan_split(int64_t M, int64_t N, int64_t K) {
+    SplitPlan p{0, 1, 0};
+    // up to 32 rows the weight-streaming kernel is as fast; below 32 K blocks the second pass costs more than
+    // the split gains
+    if (M <= 32 || K % 128 != 0 || K > (1 << 16) || M > (1 << 20)) return p;
+    const int KB = (int)(K / 128);
+    const long t256 = ((M + 255) / 256) * ((N + 255) / 256);
+    if (t256 >= 200 || KB < 32) return p;
+    if (M <= 64 && strip_pays(M, (N + 127) / 128)) return p;
+    // the largest tile that, cut into slabs of at least 8 K blocks, still yields a workgroup for most CUs
+    const long rows128 = (M + 127) / 128, rows64 = (M + 63) / 64;
+    const long cols128 = (N + 127) / 128, cols64 = (N + 63) / 64;
+    const long tiles[4] = {0, rows128 * cols128, rows128 * cols64, rows64 * cols64};
+    for (int cfg = 1; cfg <= 3; ++cfg) {
+        if (cfg != 3 && M <= 64) continue;                       // 128-row tiles would be half empty
+        long ks = kCUs / tiles[cfg];
+        if (ks > KB / 8) ks = KB / 8;
+        if (ks < 2) continue;
+        if (tiles[cfg] * ks < kCUs * 3 / 4 && cfg != 3) continue;  // a smaller tile fills the machine better
+        p.config = cfg;
+        p.kb_per = (int)((KB + ks - 1) / ks);
+        p.ksplit = (KB + p.kb_per - 1) / p.kb_per;
+        if (p.ksplit < 2) p = SplitPlan{0, 1, 0};
+        return p;
+    }
+    return p;
+}
+
+int64_t fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    const SplitPlan p = plan_split(M, N, K);
+    return p.ksplit > 1 ? (int64_t)p.ksplit * M * N * 4 : 0;
+}
+
+// returns -1 when the shape / pointers do not qualify (the caller then runs the plain path)
+template <typename OUT>
+static int launch_splitk(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, const uint8_t* b,
+                         const float* b_s, OUT* c, const uint16_t* bias, int M, int N, int K, float* ws,
+                         int64_t ws_bytes, hipStream_t stream) {
+    const SplitPlan p = plan_split(M, N, K);
+    if (p.ksplit < 2 || ws == nullptr || ws_bytes < (int64_t)p.ksplit * M * N * 4) return -1;
+    const int KB = K / 128;
+    const int64_t as_extent = ((int64_t)(M - 1) * as_rs + (int64_t)(KB - 1) * as_cs + 1) * 4;
+    const bool ok = ((reinterpret_cast<uintptr_t>(a) & 15) == 0) && ((reinterpret_cast<uintptr_t>(b) & 15) == 0) &&
+                    ((reinterpret_cast<uintptr_t>(ws) & 15) == 0) && as_rs >= 0 && as_cs >= 0 &&
+                    as_extent < ((int64_t)1 << 31);
+    if (!ok) return -1;
+#define MDY_SPLIT(BM_, BN_, ST_)                                                                                      \
+    {                                                                                                                 \
+        const int tiles_m = (M + BM_ - 1) / BM_, tiles_n = (N + BN_ - 1) / BN_;                                       \
+        hipLaunchKernelGGL((fp8_gemm_splitk_kernel<BM_, BN_, 2, 2, ST_>), dim3((unsigned)(tiles_m * tiles_n * p.ksplit)), \
+                           dim3(256), 0, stream, a, a_s, (int)as_rs, (int)as_cs, (uint32_t)as_extent, b, b_s, ws, M, N, K, \
+                           tiles_m, tiles_n, p.ksplit, p.kb_per);                                                     \
+    }
+    if (p.config == 1) MDY_SPLIT(128, 128, 4)
+    else if (p.config == 2) MDY_SPLIT(128, 64, 6)
+    else MDY_SPLIT(64, 64, 8)
+#undef MDY_SPLIT
+    int rc = (int)hipGetLastError();
+    if (rc != 0) return rc;
+    const int64_t MN = (int64_t)M * N;
+    const bool vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
+    if (vec)
+        hipLaunchKernelGGL((splitk_reduce_kernel<OUT, true>), dim3((unsigned)((MN / 4 + 255) / 256)), dim3(256), 0, stream,
+                           ws, c, bias, MN, N, p.ksplit);
+    else
+        hipLaunchKernelGGL((splitk_reduce_kernel<OUT, false>), dim3((unsigned)((MN + 255) / 256)), dim3(256), 0, stream, ws,
+                           c, bias, MN, N, p.ksplit);
+    return (int)hipGetLastError();
+}
+
+int launch_fp8_gemm_nt_ws(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,
+                          const float* b_s, void* c, const void* bias, int64_t M, int64_t N, int64_t K, int out_dtype,
+                          void* workspace, int64_t workspace_bytes, hipStream_t stream) {
+    if (M == 0 || N == 0) return 0;
+    int rc = -1;
+    if (out_dtype == 0)
+        rc = launch_splitk<uint16_t>(static_cast<const uint8_t*>(a), a_s, as_row_stride, as_col_stride,
+                                     static_cast<const uint8_t*>(b), b_s, static_cast<uint16_t*>(c),
+                                     static_cast<const uint16_t*>(bias), (int)M, (int)N, (int)K,
+                                     static_cast<float*>(workspace), workspace_bytes, stream);
+    else
+        rc = launch_splitk<float>(static_cast<const uint8_t*>(a), a_s, as_row_stride, as_col_stride,
+                                  static_cast<const uint8_t*>(b), b_s, static_cast<float*>(c),
+                                  static_cast<const uint16_t*>(bias), (int)M, (int)N, (int)K,
+                                  static_cast<float*>(workspace), workspace_bytes, stream);
+    if (rc >= 0) return rc;
+    return launch_fp8_gemm_nt(a, a_s, as_row_stride, as_col_stride, b, b_s, c, bias, M, N, K, out_dtype, stream);
 }
 
 int launch_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,

@@ -10,7 +10,7 @@ from typing import Optional, Tuple
 
 import torch
 
-from ._torch_glue import FP8, check, lib, on_device, ptr, require_gpu, stream_ptr
+from ._torch_glue import FP8, check, gemm_workspace, lib, on_device, ptr, require_gpu, stream_ptr
 
 
 def _cdiv(a: int, b: int) -> int:
@@ -151,8 +151,10 @@ def fp8_matmul(qa: torch.Tensor, sa: torch.Tensor, qb: torch.Tensor, sb: torch.T
     if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != N or not bias.is_contiguous()):
         raise ValueError("bias must be a contiguous bfloat16 [N] tensor")
     with on_device(dev):
-        check(lib().mdy_fp8_gemm_nt(ptr(qa), ptr(sa), sa.stride(0), sa.stride(1), ptr(qb), ptr(sb), ptr(out),
-                                    ptr(bias), M, N, K, 0, stream_ptr(dev)), "fp8_matmul")
+        ws = gemm_workspace(dev, M, N, K)      # scratch for shapes that are split along K, else None
+        check(lib().mdy_fp8_gemm_nt_ws(ptr(qa), ptr(sa), sa.stride(0), sa.stride(1), ptr(qb), ptr(sb), ptr(out),
+                                       ptr(bias), M, N, K, 0, ptr(ws), ws.numel() if ws is not None else 0,
+                                       stream_ptr(dev)), "fp8_matmul")
     return out
 
 

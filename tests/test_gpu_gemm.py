@@ -9,6 +9,7 @@ import pytest
 import torch
 
 import mdy_triton_amd as m
+from mdy_triton_amd import _lib
 from oracle import oracle as O
 from tests import problems as P
 
@@ -80,6 +81,76 @@ def test_gemm_exact_integer_few_tiles_configs(M, N, K):
     """Shapes with fewer than 200 tiles of 256x256 pick tile size and LDS ring depth by tile count; K runs
     from one K block (shorter than every ring) to more K blocks than the deepest ring, M and N ragged."""
     test_gemm_exact_integer_cases_all_kernels(M, N, K)
+
+
+SPLIT_SHAPES = [(128, 1536, 4096), (100, 777, 4224), (64, 2048, 4352), (40, 300, 8192), (256, 4096, 4096),
+                (130, 1100, 5120), (33, 130, 4096)]
+
+
+@pytest.mark.parametrize("M,N,K", SPLIT_SHAPES)
+def test_gemm_exact_integer_split_k(M, N, K):
+    """Few rows against a long K: fp8_gemm hands the library a workspace and the shape runs split along K
+    (64x64, 128x64 and 128x128 tiles; N % 4 != 0 takes the scalar reduction).  Exact operands stay exact."""
+    assert _lib.load().mdy_fp8_gemm_workspace_bytes(M, N, K) >= 2 * M * N * 4
+    test_gemm_exact_integer_cases_all_kernels(M, N, K)
+
+
+def _raw_gemm(a, a_s, b, b_s, bias, dtype, ws, ws_bytes=None):
+    M, K = a.shape
+    N = b.shape[0]
+    c = torch.full((M, N), float("nan"), device=DEV, dtype=dtype)
+    code = 0 if dtype == torch.bfloat16 else 1
+    lib = _lib.load()
+    if ws == "plain":
+        rc = lib.mdy_fp8_gemm_nt(a.data_ptr(), a_s.data_ptr(), K // 128, 1, b.data_ptr(), b_s.data_ptr(), c.data_ptr(),
+                                 bias.data_ptr() if bias is not None else None, M, N, K, code, None)
+    else:
+        rc = lib.mdy_fp8_gemm_nt_ws(a.data_ptr(), a_s.data_ptr(), K // 128, 1, b.data_ptr(), b_s.data_ptr(), c.data_ptr(),
+                                    bias.data_ptr() if bias is not None else None, M, N, K, code,
+                                    ws.data_ptr() if ws is not None else None,
+                                    (ws.numel() if ws is not None else 0) if ws_bytes is None else ws_bytes, None)
+    torch.cuda.synchronize()
+    return rc, c
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("M,N,K", [(128, 1536, 7168), (100, 777, 4224), (64, 2048, 7168)])
+def test_gemm_split_k_against_oracle_and_plain_path(M, N, K, dtype):
+    """Through the C ABI: with a workspace the result is within the GEMM tolerance of the oracle and of the
+    single-pass kernel (another summation order), deterministic, and the bias is added once; without one, or
+    with one that is too small, the call is the single-pass kernel bit for bit."""
+    a, a_s, b, b_s = quantized_problem("outliers", M, N, K, seed=K + M)
+    bias = (torch.randn(N, generator=torch.Generator().manual_seed(3)) * 0.5).bfloat16()
+    ref = O.fp8_gemm(a, a_s, b, b_s, dtype=torch.float32) + bias.float()
+    ad, asd, bd, bsd, biasd = a.to(DEV), a_s.to(DEV), b.to(DEV), b_s.to(DEV), bias.to(DEV)
+    need = _lib.load().mdy_fp8_gemm_workspace_bytes(M, N, K)
+    assert need > 0
+    ws = torch.empty(need, device=DEV, dtype=torch.uint8)
+    rc, plain = _raw_gemm(ad, asd, bd, bsd, biasd, dtype, "plain")
+    assert rc == 0
+    ws.fill_(0xFF)                                         # stale contents must not matter
+    rc, split = _raw_gemm(ad, asd, bd, bsd, biasd, dtype, ws)
+    assert rc == 0
+    assert close_biased(split, ref, bias) and close_biased(plain, ref, bias)
+    assert torch.allclose(split.float(), plain.float(), rtol=RTOL, atol=ATOL)
+    rc, again = _raw_gemm(ad, asd, bd, bsd, biasd, dtype, ws)
+    assert rc == 0 and torch.equal(again, split)
+    for small in (None, ws[:need - 16]):
+        rc, fb = _raw_gemm(ad, asd, bd, bsd, biasd, dtype, small)
+        assert rc == 0 and torch.equal(fb, plain)
+    rc, _ = _raw_gemm(ad, asd, bd, bsd, biasd, dtype, ws[4:], need - 4)     # misaligned workspace
+    assert rc == -3                                        # MDY_E_ALIGN
+
+
+def test_gemm_workspace_query():
+    lib = _lib.load()
+    assert lib.mdy_fp8_gemm_workspace_bytes(4096, 18432, 7168) == 0      # fills the GPU: never split
+    assert lib.mdy_fp8_gemm_workspace_bytes(32, 7168, 16384) == 0        # weight-streaming kernel
+    assert lib.mdy_fp8_gemm_workspace_bytes(128, 7168, 2048) == 0        # K too short to cut
+    assert lib.mdy_fp8_gemm_workspace_bytes(128, 7168, 5000) == 0        # ragged K: scalar kernel
+    assert lib.mdy_fp8_gemm_workspace_bytes(0, 7168, 16384) == 0 and lib.mdy_fp8_gemm_workspace_bytes(-1, 1, 1) == 0
+    n = lib.mdy_fp8_gemm_workspace_bytes(128, 7168, 16384)
+    assert n > 0 and n % (128 * 7168 * 4) == 0
 
 
 @pytest.mark.parametrize("M,N,K", [(4000, 4328, 256), (3590, 4608, 384), (4096, 4352, 128)])
