@@ -326,6 +326,16 @@ def table(torch, m, timer, dev):
                     m.fp8_gemm(a, a_s, b, b_s, out_dtype=torch.bfloat16)
             us = timer.run(many, 10, cold=False)[0] / 20
             line("C5 fp8_gemm M=%d N=%d K=%d (warm, back-to-back)" % (M, N, K), us, byts, "GB/s", PEAK_HBM_GBS)
+    # few rows against a long K (small-batch prefill / large-batch decode): tiles do not fill the GPU, the
+    # wrapper hands the library a workspace and the shape is split along K; weight bytes bound these
+    for (M, N, K) in ((128, 7168, 16384), (128, 2112, 7168), (256, 7168, 18432), (512, 4096, 7168)):
+        a = torch.randint(0, 120, (M, K), dtype=torch.uint8, device=dev).view(FP8)
+        b = torch.randint(0, 120, (N, K), dtype=torch.uint8, device=dev).view(FP8)
+        a_s = torch.rand(M, K // 128, device=dev)
+        b_s = torch.rand((N + 127) // 128, K // 128, device=dev)
+        byts = M * K + N * K + 4 * M * K / 128 + 4 * ((N + 127) // 128) * (K // 128) + 2 * M * N
+        us = timer.run(lambda: m.fp8_gemm(a, a_s, b, b_s, out_dtype=torch.bfloat16), 10)[0]
+        line("fp8_gemm M=%d N=%d K=%d (split along K)" % (M, N, K), us, byts, "GB/s", PEAK_HBM_GBS)
 
 
 if __name__ == "__main__":
