@@ -85,12 +85,18 @@ class ColdTimer:
         self.flush = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
 
     def run(self, fn, reps, cold=True):
+        """cold=True: flush by rewriting 512 MiB, which leaves the caches full of dirty lines (every miss of
+        the timed kernel then also pays a write-back: the conservative protocol, used for every headline
+        figure); cold="read": flush by reading 512 MiB (clean lines, what a kernel sees when other weights
+        were streamed before it); cold=False: back to back."""
         torch = self.torch
         fn()
         torch.cuda.synchronize()
         ts = []
         for _ in range(reps):
-            if cold:
+            if cold == "read":
+                self.flush.view(torch.int64).sum()
+            elif cold:
                 self.flush.add_(1)
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
@@ -312,6 +318,9 @@ def table(torch, m, timer, dev):
         else:
             line("grouped fp8_gemm %d experts x %d rows, N=%d K=%d" % (G, mg, Ng, Kg), us,
                  Mt * Kg + G * Ng * Kg + 2.0 * Mt * Ng + 4.0 * Mt * Kg / 128, "GB/s", PEAK_HBM_GBS)
+            us = timer.run(lambda: m.fp8_grouped_matmul(aq, asg, bq, bsg, [mg] * G), 10, cold="read")[0]
+            line("   the same after a read-only cache flush", us,
+                 Mt * Kg + G * Ng * Kg + 2.0 * Mt * Ng + 4.0 * Mt * Kg / 128, "GB/s", PEAK_HBM_GBS)
     del bq, bsg, aq, asg
     for M in (1, 16, 64):
         for (N, K) in ((7168, 2048), (2048, 7168)):
@@ -336,6 +345,8 @@ def table(torch, m, timer, dev):
         byts = M * K + N * K + 4 * M * K / 128 + 4 * ((N + 127) // 128) * (K // 128) + 2 * M * N
         us = timer.run(lambda: m.fp8_gemm(a, a_s, b, b_s, out_dtype=torch.bfloat16), 10)[0]
         line("fp8_gemm M=%d N=%d K=%d (split along K)" % (M, N, K), us, byts, "GB/s", PEAK_HBM_GBS)
+        us = timer.run(lambda: m.fp8_gemm(a, a_s, b, b_s, out_dtype=torch.bfloat16), 10, cold="read")[0]
+        line("   the same after a read-only cache flush", us, byts, "GB/s", PEAK_HBM_GBS)
 
 
 if __name__ == "__main__":
