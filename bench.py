@@ -36,10 +36,10 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E, published
 
 # HBM bytes per fp8_gemm call at the C3 shape (both of its launches), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (KiB per dispatch, scaled by the same counters read on a plain copy kernel of known size); the runs are
-# summarised in profiles/bench_C3_hbm_traffic.txt: FETCH_SIZE (349 095 + 72 421) KiB x 1.9997 (copy-kernel
-# calibration) = 863.2 MB read, WRITE_SIZE (133 707 + 16 426) KiB x 1.0 = 153.7 MB written; algorithmic bytes are
+# summarised in profiles/bench_C3_hbm_traffic.txt: FETCH_SIZE (349 081 + 72 423) KiB x 1.9997 (copy-kernel
+# calibration) = 863.1 MB read, WRITE_SIZE (134 165 + 16 409) KiB x 1.0 = 154.2 MB written; algorithmic bytes are
 # 313 MB (the A and B panels are re-fetched by the eight XCD-local L2s).
-GEMM_C3_HBM_TRAFFIC_BYTES = 1016.9e6
+GEMM_C3_HBM_TRAFFIC_BYTES = 1017.3e6
 
 WORKLOADS = {
     # name: (activation kind, M, N, K, description)
