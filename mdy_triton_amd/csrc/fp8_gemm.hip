@@ -738,7 +738,15 @@ static int main_tile_columns(int tiles_m, int tiles_n) {
     return cost_split < cost_plain - 0.05 ? cols_main : tiles_n;
 }
 
-// Tile and ring depth for shapes with fewer than 200 tiles of 256x256:
+// 256x256 tiles (one workgroup per CU) when they fill most of the CUs, or when 128x128 tiles (two workgroups
+// per CU) would need a second round: 144..199 tiles of 256x256 measured 20-26 % faster than 577..796 of 128x128.
+static bool big_tiles_pay(int64_t M, int64_t N) {
+    const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
+    const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128);
+    return t256 >= 200 || t128 > 2 * kCUs;
+}
+
+// Tile and ring depth for the shapes that do not take 256x256 tiles:
 //   0: 128x128, 2 K blocks in LDS (two workgroups share a CU)   1: 128x128, 4 K blocks (one workgroup per CU)
 //   2: 128x64, 6 K blocks                                       3: 64x64, 8 K blocks
 // Measured rule: the smallest tile that still gives every workgroup a CU of its own (the time of these
@@ -818,8 +826,7 @@ static int dispatch(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t a
 #undef MDY_SM
         return (int)hipGetLastError();
     }
-    const long tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-    if (tiles256 >= 200) {
+    if (big_tiles_pay(M, N)) {
         const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
         const int cols_main = main_tile_columns(tiles_m, tiles_n);
         const int n_main = cols_main < tiles_n ? cols_main * 256 : N;
@@ -859,8 +866,7 @@ static SplitPlan plan_split(int64_t M, int64_t N, int64_t K) {
     // the split gains
     if (M <= 32 || K % 128 != 0 || K > (1 << 16) || M > (1 << 20)) return p;
     const int KB = (int)(K / 128);
-    const long t256 = ((M + 255) / 256) * ((N + 255) / 256);
-    if (t256 >= 200 || KB < 32) return p;
+    if (big_tiles_pay(M, N) || KB < 32) return p;
     if (M <= 64 && strip_pays(M, (N + 127) / 128)) return p;
     // the largest tile that, cut into slabs of at least 8 K blocks, still yields a workgroup for most CUs
     const long rows128 = (M + 127) / 128, rows64 = (M + 63) / 64;

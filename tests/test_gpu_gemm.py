@@ -153,11 +153,12 @@ def test_gemm_workspace_query():
     assert n > 0 and n % (128 * 7168 * 4) == 0
 
 
-@pytest.mark.parametrize("M,N,K", [(4000, 4328, 256), (3590, 4608, 384), (4096, 4352, 128)])
+@pytest.mark.parametrize("M,N,K", [(4000, 4328, 256), (3590, 4608, 384), (4096, 4352, 128), (4000, 2400, 256)])
 def test_gemm_exact_integer_big_tiles_and_split_launch(M, N, K):
     """>= 200 tiles of 256x256: the big-tile kernel runs, and because the tile count is not a multiple
     of the CU count the last tile columns go to a second launch with 128x256 tiles (ragged M and N edges
-    in both)."""
+    in both).  The last shape has 160 tiles of 256x256 (more 128x128 tiles than fit in one round): one
+    partly filled round of the big tile."""
     test_gemm_exact_integer_cases_all_kernels(M, N, K)
 
 
