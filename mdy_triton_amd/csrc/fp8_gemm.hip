@@ -87,13 +87,19 @@ __device__ __forceinline__ void dma4(const intx4& rsrc, int voff, int soff, uint
                  :: "v"(voff), "s"(rsrc), "s"(soff), "s"(lds) : "memory");
 }
 
+// Shares of the panel pre-touches: the A panel of a tile row is cut into 2^a_sh shares among the tiles of
+// that row that run side by side, the B panel of a tile column into 2^b_sh shares among its tile rows.
+struct Duty {
+    int a_duty, a_sh, b_duty, b_sh;
+};
+
 // One BM x BN tile of C: WGM x WGN waves, each wave (BM/WGM) x (BN/WGN).
 //   rows m0 .. min(m0+BM, m_end) of a (m_end = end of the matrix, or of the expert group the tile belongs to),
 //   columns n0 .. of b / b_s / bias (already offset to the group's weight), K % 128 == 0, K <= 65536,
 //   K blocks kb0 .. kb1-1 of them (all of them except in the split-K kernel).
 // as_bytes = byte size of the addressed part of a_s (host computed, < 2^31); m_total = rows of a_s.
-// a_duty (0..7) / b_duty (0..3): which share of the A / B panel lines this workgroup pre-touches for the
-// workgroups that copy the same panels (those with the same tile row / tile column).
+// duty: which share of the A / B panel lines this workgroup pre-touches for the workgroups that copy the same
+// panels (those with the same tile row / tile column), and into how many shares the panels are cut.
 //
 // Schedule of one K block (NT = TI*TJ MFMA slots, each followed DEPTH slots later by its 4 FMAs):
 //   slots 0..      the last copies of K block kb+1 (those that did not fit into the tail below), one per GAP
@@ -110,8 +116,8 @@ template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT>
 __device__ __forceinline__ void fp8_gemm_tile(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
-    const uint16_t* __restrict__ bias, int m0, int m_end, int m_total, int n0, int N, int K, int ldc, int a_duty,
-    int b_duty, int kb0, int kb1) {
+    const uint16_t* __restrict__ bias, int m0, int m_end, int m_total, int n0, int N, int K, int ldc, const Duty duty,
+    int kb0, int kb1) {
     constexpr int WAVES = WGM * WGN;
     constexpr int WM = BM / WGM, WN = BN / WGN, TI = WM / 16, TJ = WN / 16;
     constexpr int PASS_ROWS = WAVES * 8;  // rows copied by one DMA instruction of every wave
@@ -183,12 +189,17 @@ __device__ __forceinline__ void fp8_gemm_tile(
             dma16(rb, voff, (i - 1 - A_PASSES) * PASS_ROWS * K + (more ? kb * 128 : rb[2]),
                   lb_base + buf * (BN * 128) + (i - 1 - A_PASSES) * PASS_ROWS * 128);
     };
-    // duty touch: wave 0 loads one dword of every line of its share of the B panel, wave 1 of the A panel,
-    // TD K blocks ahead, into the dummy area: the lines are in L2 when this workgroup and its neighbours
-    // copy them.  The other waves run the same instruction on an empty descriptor.
-    intx4 rt = wave == 0 ? rb : ra;
-    if (wave >= 2) rt[2] = 0;
-    const int touch_off = wave == 0 ? (b_duty * (BN / 4) + lane % (BN / 4)) * K : (a_duty * (BM / 8) + lane % (BM / 8)) * K;
+    // duty touch: the even waves load one dword of every line of this workgroup's share of the B panel (64
+    // rows per wave), the odd waves of the A panel, TD K blocks ahead, into the dummy area: the lines are in L2
+    // when this workgroup and its neighbours copy them.  Waves beyond the share run the same instruction on an
+    // empty descriptor.
+    const bool touch_b = (wave & 1) == 0;
+    const int share = touch_b ? (BN >> duty.b_sh) : (BM >> duty.a_sh);      // rows of the share, a power of two
+    const int t_idx = (wave >> 1) * 64 + lane;
+    intx4 rt = touch_b ? rb : ra;
+    // nobody to share with: touching one's own lines ahead of the copy only adds requests (measured)
+    if ((wave >> 1) * 64 >= share || (touch_b ? duty.b_sh : duty.a_sh) == 0) rt[2] = 0;
+    const int touch_off = ((touch_b ? duty.b_duty : duty.a_duty) * share + (t_idx & (share - 1))) * K;
 
     // ---- fragment reads: lane -> row (lane%16) and the 32-byte K slice (lane/16) of a 16-row sub-tile
     const int frow = lane & 15, fk = lane >> 4;
@@ -323,13 +334,21 @@ __device__ __forceinline__ void fp8_gemm_tile(
 __device__ __forceinline__ int xcd_contiguous(int pid, int ntiles) {
     return (ntiles % 8 == 0) ? (pid & 7) * (ntiles >> 3) + (pid >> 3) : pid;
 }
-__device__ __forceinline__ void tile_of(int local, int tiles_m, int tiles_n, int& tm, int& tn) {
+__device__ __forceinline__ Duty tile_of(int local, int tiles_m, int tiles_n, int& tm, int& tn) {
     constexpr int GM = 4;
     const int group = local / (GM * tiles_n);
     const int first_m = group * GM;
     const int gsz = min(tiles_m - first_m, GM);
-    tm = first_m + (local % (GM * tiles_n)) % gsz;
+    const int in_group = (local % (GM * tiles_n)) % gsz;
+    tm = first_m + in_group;
     tn = (local % (GM * tiles_n)) / gsz;
+    // the workgroups of an XCD run a gsz x (up to 8) block of tiles at a time
+    Duty d;
+    d.b_sh = gsz >= 4 ? 2 : gsz >= 2 ? 1 : 0;
+    d.a_sh = tiles_n >= 8 ? 3 : tiles_n >= 4 ? 2 : tiles_n >= 2 ? 1 : 0;
+    d.b_duty = in_group & ((1 << d.b_sh) - 1);
+    d.a_duty = tn & ((1 << d.a_sh) - 1);
+    return d;
 }
 
 template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT>
@@ -338,9 +357,9 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
     const uint16_t* __restrict__ bias, int M, int N, int K, int ldc, int tiles_m, int tiles_n) {
     int tm, tn;
-    tile_of(xcd_contiguous(blockIdx.x, tiles_m * tiles_n), tiles_m, tiles_n, tm, tn);
-    fp8_gemm_tile<BM, BN, WGM, WGN, STAGES, OUT>(a, a_s, as_rs, as_cs, as_bytes, b, b_s, c, bias, tm * BM, M, M, tn * BN, N, K, ldc, tn & 7,
-                                                 tm & 3, 0, K >> 7);
+    const Duty duty = tile_of(xcd_contiguous(blockIdx.x, tiles_m * tiles_n), tiles_m, tiles_n, tm, tn);
+    fp8_gemm_tile<BM, BN, WGM, WGN, STAGES, OUT>(a, a_s, as_rs, as_cs, as_bytes, b, b_s, c, bias, tm * BM, M, M, tn * BN, N, K, ldc, duty,
+                                                 0, K >> 7);
 }
 
 // ---------------------------------------------------------------------------
@@ -359,10 +378,10 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_splitk_kernel(
     const int pid = xcd_contiguous(blockIdx.x, ntiles * ksplit);
     const int ks = __builtin_amdgcn_readfirstlane(pid / ntiles);
     int tm, tn;
-    tile_of(pid - ks * ntiles, tiles_m, tiles_n, tm, tn);
+    const Duty duty = tile_of(pid - ks * ntiles, tiles_m, tiles_n, tm, tn);
     const int kb0 = ks * kb_per, kb1 = min(K >> 7, kb0 + kb_per);
     fp8_gemm_tile<BM, BN, WGM, WGN, STAGES, float>(a, a_s, as_rs, as_cs, as_bytes, b, b_s, ws + (size_t)ks * M * N, nullptr,
-                                                   tm * BM, M, M, tn * BN, N, K, N, tn & 7, tm & 3, kb0, kb1);
+                                                   tm * BM, M, M, tn * BN, N, K, N, duty, kb0, kb1);
 }
 
 template <typename OUT, bool VEC>
@@ -427,14 +446,18 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_grouped_gemm_kernel(
     const int g = __builtin_amdgcn_readfirstlane(lo);
     const int tiles_m = __builtin_amdgcn_readfirstlane(tbl.tile_start[g + 1] - tbl.tile_start[g]);
     int tm, tn;
-    tile_of(pid - tbl.tile_start[g] * tiles_n, tiles_m, tiles_n, tm, tn);
+    Duty duty = tile_of(pid - tbl.tile_start[g] * tiles_n, tiles_m, tiles_n, tm, tn);
+    duty.a_duty = __builtin_amdgcn_readfirstlane(duty.a_duty);
+    duty.b_duty = __builtin_amdgcn_readfirstlane(duty.b_duty);
+    duty.a_sh = __builtin_amdgcn_readfirstlane(duty.a_sh);
+    duty.b_sh = __builtin_amdgcn_readfirstlane(duty.b_sh);
     const int KB = K >> 7, NB = (N + 127) >> 7;
     const int r0 = __builtin_amdgcn_readfirstlane(tbl.row_start[g]), r1 = __builtin_amdgcn_readfirstlane(tbl.row_start[g + 1]);
     fp8_gemm_tile<BM, BN, WGM, WGN, 2, OUT>(a, a_s, as_rs, as_cs, as_bytes, b + (size_t)g * N * K,
                                          b_s + (size_t)g * NB * KB, c, bias ? bias + (size_t)g * N : nullptr,
                                          __builtin_amdgcn_readfirstlane(r0 + tm * BM), r1,
                                          __builtin_amdgcn_readfirstlane(tbl.row_start[G]), __builtin_amdgcn_readfirstlane(tn * BN), N, K, N,
-                                         __builtin_amdgcn_readfirstlane(tn & 7), __builtin_amdgcn_readfirstlane(tm & 3), 0, K >> 7);
+                                         duty, 0, K >> 7);
 }
 
 // ---------------------------------------------------------------------------
