@@ -8,9 +8,9 @@
 // Main kernel (K % 128 == 0):
 //   * one workgroup owns a BM x BN tile of C; per 128-wide K block the A and B
 //     panels (BM x 128 and BN x 128 bytes) and the BM activation scales are
-//     copied global -> LDS by `buffer_load ... lds` (no registers involved),
-//     double buffered, one barrier per K block.  The buffer descriptors cover
-//     exactly the rows of the tile, so rows past M or N read as zero;
+//     copied global -> LDS by `buffer_load ... lds` (no registers involved) into
+//     a ring of 2..8 K blocks, one barrier per K block.  The buffer descriptors
+//     cover exactly the rows of the tile, so rows past M or N read as zero;
 //   * LDS rows are 128 bytes; the eight 16-byte chunks of a row are XOR-swizzled
 //     with (row & 7) ^ (row>>3 & 1): each DMA lane fetches the permuted chunk,
 //     the ds_read_b128 fragment reads are bank-conflict free;
@@ -27,8 +27,11 @@
 //     whole K block, the other one is streamed through a two-deep register queue;
 //   * workgroup ids are remapped so that the 32 workgroups that share an XCD's L2
 //     cover a compact 4 x 8 block of tiles.
+// Tile sizes from 64x64 to 256x256 share that body; the host picks by tile count, and with a
+// workspace also splits K (fp8_gemm_splitk_kernel + splitk_reduce_kernel).
 // Small-M kernel (M <= 64): weight streaming, one workgroup of 8 waves per 16 columns,
-// waves split K (next block prefetched) and reduce through LDS.  Scalar kernel: any other shape/alignment.
+// waves split K (next block prefetched) and reduce through LDS.  Strip kernel: 5..64 rows against
+// many 128-column strips.  Scalar kernel: any other shape/alignment.
 #include "common.h"
 
 namespace mdy {
@@ -76,7 +79,7 @@ __device__ __forceinline__ uint32_t lds_addr(const void* p) {
 }
 // 64 lanes x 16 bytes, global (descriptor base + voff + soff) -> LDS (lds + lane*16).
 // Issued as inline asm so that the copy stays asynchronous: the kernel waits for it
-// with an explicit vmcnt(0) + barrier at the end of the K block, nowhere else.
+// with an explicit s_waitcnt vmcnt + barrier once per K block, nowhere else.
 // rsrc, soff and lds must be wave-uniform.
 __device__ __forceinline__ void dma16(const intx4& rsrc, int voff, int soff, uint32_t lds) {
     asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
