@@ -834,6 +834,13 @@ static int dispatch(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t a
         const int64_t one = M;
         return launch_strip<OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, &one, 1, M, N, K, stream);
     }
+    // 32..64 rows against a wide weight: the kernel below re-reads the activation rows in every one of its
+    // N/16 workgroups, and from 32 rows on that traffic costs more than the empty rows of an MFMA tile.
+    // Measured (M=64): N=18432, K=7168 121 -> 64 us with 128x128 tiles; N=7168, K=16384 110 -> 80 us with 64x64.
+    if (M >= 32 && M <= 64 && big_ok && (N + 127) / 128 >= 128)
+        return launch_mfma<128, 128, 2, 2, 4, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
+    if (M >= 32 && M <= 64 && big_ok && (N + 63) / 64 >= 100)
+        return launch_mfma<64, 64, 2, 2, 8, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
     if (M <= 64) {
         // one workgroup streams 16 weight columns against MT row sub-tiles; every workgroup re-reads its rows of
         // a, so with few column groups (N small) the rows are split over grid.y as well: more workgroups, less

@@ -76,7 +76,8 @@ def test_gemm_exact_integer_cases_all_kernels(M, N, K):
 @pytest.mark.parametrize("M,N,K", [(2000, 2304, 256), (2048, 2200, 1152),      # 128x128 tiles, 2 K blocks in LDS
                                    (1536, 2048, 128), (1500, 2000, 1280),      # 128x128 tiles, ring of 4 K blocks
                                    (1024, 1100, 128), (1000, 1090, 1664),      # 128x64 tiles, ring of 6
-                                   (200, 300, 128), (130, 70, 2304), (520, 776, 1024)])   # 64x64 tiles, ring of 8
+                                   (200, 300, 128), (130, 70, 2304), (520, 776, 1024),    # 64x64 tiles, ring of 8
+                                   (40, 16400, 256), (64, 6500, 384), (33, 7168, 1280)])  # 32..64 rows, wide weight
 def test_gemm_exact_integer_few_tiles_configs(M, N, K):
     """Shapes with fewer than 200 tiles of 256x256 pick tile size and LDS ring depth by tile count; K runs
     from one K block (shorter than every ring) to more K blocks than the deepest ring, M and N ragged."""
