@@ -143,6 +143,34 @@ def test_gemm_split_k_against_oracle_and_plain_path(M, N, K, dtype):
     assert rc == -3                                        # MDY_E_ALIGN
 
 
+def test_gemm_exact_integer_random_shapes():
+    """60 seeded random shapes through every dispatch path (streaming, strip, 64..256-wide tiles, rings, split K,
+    scalar): exact operands, so any wrong index, stale LDS buffer or misplaced scale shows as a bit difference."""
+    g = torch.Generator().manual_seed(2024)
+    shapes = []
+    for _ in range(60):
+        M = int(torch.randint(1, 700, (1,), generator=g)) if torch.rand(1, generator=g) < 0.8 else int(torch.randint(700, 3000, (1,), generator=g))
+        N = int(torch.randint(1, 3000, (1,), generator=g))
+        K = 128 * int(torch.randint(1, 40, (1,), generator=g))
+        if torch.rand(1, generator=g) < 0.1:
+            K += int(torch.randint(1, 128, (1,), generator=g))          # ragged K: scalar kernel
+        shapes.append((M, N, K))
+    shapes += [(48, 26000, 256), (64, 16500, 512), (33, 6400, 4096), (5, 25700, 384)]   # strip / wide-weight rules
+    for M, N, K in shapes:
+        gi = torch.Generator().manual_seed(M * 7 + N * 3 + K)
+        ai = torch.randint(-2, 3, (M, K), generator=gi)
+        bi = torch.randint(-2, 3, (N, K), generator=gi)
+        KB, NB = (K + 127) // 128, (N + 127) // 128
+        ae = torch.randint(-1, 2, (M, KB), generator=gi)
+        be = torch.randint(-1, 2, (NB, KB), generator=gi)
+        got = m.fp8_gemm(ai.float().to(FP8).to(DEV), torch.exp2(ae.float()).to(DEV), bi.float().to(FP8).to(DEV),
+                         torch.exp2(be.float()).to(DEV), out_dtype=torch.float32).cpu().double()
+        sa = torch.exp2(ae.double()).repeat_interleave(128, 1)[:, :K]
+        sb = torch.exp2(be.double()).repeat_interleave(128, 0)[:N].repeat_interleave(128, 1)[:, :K]
+        ref = (ai.double() * sa) @ (bi.double() * sb).t()
+        assert torch.equal(got, ref), (M, N, K)
+
+
 def test_gemm_workspace_query():
     lib = _lib.load()
     assert lib.mdy_fp8_gemm_workspace_bytes(4096, 18432, 7168) == 0      # fills the GPU: never split
