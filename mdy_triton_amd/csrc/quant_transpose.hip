@@ -38,32 +38,34 @@ __device__ __forceinline__ float qt_quot(float x, float s, float r) {
     return sat_for_mode<1>(x / s);
 }
 
-template <int TMODE, bool VEC>
-__global__ __launch_bounds__(256) void quant_transpose_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ y,
+template <int TMODE, bool VEC, int RPT>
+__global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ y,
                                                                float* __restrict__ s, uint8_t* __restrict__ y_t,
                                                                float* __restrict__ s_t, int M, int K,
                                                                int64_t x_row_stride, int64_t x_col_stride, int PM,
                                                                int PK, int64_t s_kb_stride) {
-    __shared__ float col_part[16][128];   // per row group (t/16) partial column maxima
+    constexpr int NRG = 128 / RPT;        // row groups of RPT consecutive rows; 16 threads (8 columns each) per group
+    constexpr int WAVES = NRG / 4;
+    __shared__ float col_part[NRG][128];  // per row group partial column maxima
     __shared__ float col_amax[128];
-    __shared__ float blk_part[4];
+    __shared__ float blk_part[WAVES];
     __shared__ __attribute__((aligned(16))) uint8_t tile[128][128 + 8];   // [k][m], transposed
 
     const int t = threadIdx.x;
     const int lane = t & 63, wave = t >> 6;
     const int bm = blockIdx.y, bk = blockIdx.x;
     const int cl = (t & 15) * 8;          // first local column of this thread
-    const int rg = t >> 4;                // row group 0..15
+    const int rg = t >> 4;                // row group 0..NRG-1
     const int c0 = bk * 128 + cl;
 
-    float f[8][8];
-    float rmax[8];
+    float f[RPT][8];
+    float rmax[RPT];
     float cmax[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) cmax[j] = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int row = bm * 128 + rg * 8 + i;
+    for (int i = 0; i < RPT; ++i) {
+        const int row = bm * 128 + rg * RPT + i;
         uint32_t wd[4] = {0u, 0u, 0u, 0u};
         if (row < M && c0 < K) {
             if (VEC) {
@@ -91,8 +93,8 @@ __global__ __launch_bounds__(256) void quant_transpose_kernel(const uint16_t* __
 
     // ---- (1) row-wise quantization straight from registers
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int row = bm * 128 + rg * 8 + i;      // < PM
+    for (int i = 0; i < RPT; ++i) {
+        const int row = bm * 128 + rg * RPT + i;    // < PM
         const float sc = group_scale<1>(rmax[i]);
         const float r = 1.0f / sc;
         float q[8];
@@ -116,7 +118,7 @@ __global__ __launch_bounds__(256) void quant_transpose_kernel(const uint16_t* __
         if (t < 128) {
             float m = 0.0f;
 #pragma unroll
-            for (int g = 0; g < 16; ++g) m = fmaxf(m, col_part[g][t]);
+            for (int g = 0; g < NRG; ++g) m = fmaxf(m, col_part[g][t]);
             col_amax[t] = m;
             // logical s_t[k, a]: stored [A][PK]
             s_t[(int64_t)bm * PK + bk * 128 + t] = group_scale<1>(m);
@@ -127,12 +129,14 @@ __global__ __launch_bounds__(256) void quant_transpose_kernel(const uint16_t* __
     } else {
         float m = 0.0f;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) m = fmaxf(m, rmax[i]);
+        for (int i = 0; i < RPT; ++i) m = fmaxf(m, rmax[i]);
 #pragma unroll
         for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
         if (lane == 0) blk_part[wave] = m;
         __syncthreads();
-        const float bmax = fmaxf(fmaxf(blk_part[0], blk_part[1]), fmaxf(blk_part[2], blk_part[3]));
+        float bmax = blk_part[0];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) bmax = fmaxf(bmax, blk_part[w]);
         if (t == 0) s_t[(int64_t)bk * (PM >> 7) + bm] = group_scale<1>(bmax);
 #pragma unroll
         for (int j = 0; j < 8; ++j) tamax[j] = bmax;
@@ -145,9 +149,9 @@ __global__ __launch_bounds__(256) void quant_transpose_kernel(const uint16_t* __
         tr[j] = 1.0f / tsc[j];
         tfast = tfast && (tamax[j] <= 1e4f);
     }
-    uint32_t qlo[8], qhi[8];   // row i of the transposed copy's bytes: columns 0..3 | 4..7
+    uint32_t qlo[RPT], qhi[RPT];   // row i of the transposed copy's bytes: columns 0..3 | 4..7
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < RPT; ++i) {
         float q[8];
         if (tfast) {
 #pragma unroll
@@ -159,15 +163,32 @@ __global__ __launch_bounds__(256) void quant_transpose_kernel(const uint16_t* __
         qlo[i] = pack4_e4m3(q[0], q[1], q[2], q[3]);
         qhi[i] = pack4_e4m3(q[4], q[5], q[6], q[7]);
     }
-    uint32_t tb[8][2];   // [column j][rows 0..3 | 4..7]
-    transpose8x8_bytes(qlo, qhi, tb);
+    // column j of the thread's RPT x 8 bytes = RPT consecutive bytes of row cl+j of the transposed tile
+    if (RPT == 8) {
+        uint32_t tb[8][2];   // [column j][rows 0..3 | 4..7]
+        uint32_t lo8[8], hi8[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) *reinterpret_cast<uint2*>(&tile[cl + j][rg * 8]) = make_uint2(tb[j][0], tb[j][1]);
+        for (int i = 0; i < 8; ++i) { lo8[i] = qlo[i % RPT]; hi8[i] = qhi[i % RPT]; }
+        transpose8x8_bytes(lo8, hi8, tb);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) *reinterpret_cast<uint2*>(&tile[cl + j][rg * 8]) = make_uint2(tb[j][0], tb[j][1]);
+    } else {
+        const uint32_t rl[4] = {qlo[0], qlo[1 % RPT], qlo[2 % RPT], qlo[3 % RPT]};
+        const uint32_t rh[4] = {qhi[0], qhi[1 % RPT], qhi[2 % RPT], qhi[3 % RPT]};
+        uint32_t c_lo[4], c_hi[4];
+        transpose4x4_bytes(rl, c_lo);
+        transpose4x4_bytes(rh, c_hi);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            *reinterpret_cast<uint32_t*>(&tile[cl + j][rg * 4]) = c_lo[j];
+            *reinterpret_cast<uint32_t*>(&tile[cl + 4 + j][rg * 4]) = c_hi[j];
+        }
+    }
     __syncthreads();
-    // y_t[k][m]: thread owns output columns (t%16)*8..+7 (m) of output rows t/16 + 16*i (k)
+    // y_t[k][m]: thread owns output columns (t%16)*8..+7 (m) of output rows t/16 + NRG*i (k)
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int kk = rg + 16 * i;
+    for (int i = 0; i < RPT; ++i) {
+        const int kk = rg + NRG * i;
         const uint2 v = *reinterpret_cast<const uint2*>(&tile[kk][cl]);
         store_nt8(y_t + (int64_t)(bk * 128 + kk) * PM + bm * 128 + cl, v);
     }
@@ -178,15 +199,23 @@ int launch_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s
                            int t_mode, hipStream_t stream) {
     if (PM == 0 || PK == 0) return 0;
     dim3 grid((unsigned)(PK / 128), (unsigned)(PM / 128));
-    dim3 block(256);
+    // 512 threads (4 rows each) when there are few tiles per CU: more waves to hide the load and store latency
+    const bool wide = grid.x * (long)grid.y < 256 * 24;
+    dim3 block(wide ? 512 : 256);
     const bool vec = (x_col_stride == 1) && (K % 8 == 0) && (x_row_stride % 8 == 0) &&
                      ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     uint8_t* yp = static_cast<uint8_t*>(y);
     uint8_t* ytp = static_cast<uint8_t*>(y_t);
-#define MDY_QT(TM, VEC)                                                                                          \
-    hipLaunchKernelGGL((quant_transpose_kernel<TM, VEC>), grid, block, 0, stream, xp, yp, s, ytp, s_t, (int)M, \
-                       (int)K, x_row_stride, x_col_stride, (int)PM, (int)PK, s_kb_stride)
+#define MDY_QT(TM, VEC)                                                                                                 \
+    do {                                                                                                                \
+        if (wide)                                                                                                       \
+            hipLaunchKernelGGL((quant_transpose_kernel<TM, VEC, 4>), grid, block, 0, stream, xp, yp, s, ytp, s_t, (int)M, \
+                               (int)K, x_row_stride, x_col_stride, (int)PM, (int)PK, s_kb_stride);                      \
+        else                                                                                                            \
+            hipLaunchKernelGGL((quant_transpose_kernel<TM, VEC, 8>), grid, block, 0, stream, xp, yp, s, ytp, s_t, (int)M, \
+                               (int)K, x_row_stride, x_col_stride, (int)PM, (int)PK, s_kb_stride);                      \
+    } while (0)
     if (t_mode == 0) {
         if (vec) MDY_QT(0, true); else MDY_QT(0, false);
     } else {
