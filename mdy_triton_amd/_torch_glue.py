@@ -58,11 +58,19 @@ lib = _lib.load
 check = _lib.check
 
 
+_WS_BYTES = {}
+
+
 def gemm_workspace(device, M, N, K):
     """Scratch tensor for mdy_fp8_gemm_nt_ws, or None when the shape is never split along K.  It comes
     from torch's caching allocator on the current stream, so it may be dropped as soon as the launch
     has been enqueued: the allocator hands the memory out again in stream order only."""
-    nbytes = _lib.load().mdy_fp8_gemm_workspace_bytes(M, N, K)
+    key = (M, N, K)
+    nbytes = _WS_BYTES.get(key)
+    if nbytes is None:                      # one library call per shape, not per GEMM
+        if len(_WS_BYTES) > 4096:
+            _WS_BYTES.clear()
+        nbytes = _WS_BYTES[key] = _lib.load().mdy_fp8_gemm_workspace_bytes(M, N, K)
     if nbytes <= 0:
         return None
     return torch.empty(nbytes, device=device, dtype=torch.uint8)
