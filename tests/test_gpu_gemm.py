@@ -171,6 +171,29 @@ def test_gemm_exact_integer_random_shapes():
         assert torch.equal(got, ref), (M, N, K)
 
 
+def test_ops_follow_torchs_current_stream():
+    """The launches go to torch's current stream of the tensors' device: a chain issued under a side stream, after
+    work that is still running on that stream, gives the same bits as on the default stream (the reference
+    notebooks run under torch.cuda.set_stream)."""
+    x = P.activations("normal", 256, 4096, 9).to(DEV)
+    _, wq, ws = P.weights(1024, 4096, 10)
+    wq, ws = wq.to(DEV), ws.to(DEV)
+    xq0, xs0 = m.act_quant(x)
+    c0 = m.fp8_gemm(xq0, xs0, wq, ws, out_dtype=torch.bfloat16)        # this shape is split along K: workspace too
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    big = torch.randn(8192, 8192, device=DEV)
+    with torch.cuda.stream(side):
+        x2 = x.clone()
+        for _ in range(4):
+            big = big @ big * 1e-4                                       # keeps the side stream busy
+        x2 = x2 + 0                                                     # produced on the side stream, behind the matmuls
+        xq1, xs1 = m.act_quant(x2)
+        c1 = m.fp8_gemm(xq1, xs1, wq, ws, out_dtype=torch.bfloat16)
+    side.synchronize()
+    assert torch.equal(xq1.view(torch.uint8), xq0.view(torch.uint8)) and torch.equal(xs1, xs0) and torch.equal(c1, c0)
+
+
 def test_gemm_workspace_query():
     lib = _lib.load()
     assert lib.mdy_fp8_gemm_workspace_bytes(4096, 18432, 7168) == 0      # fills the GPU: never split
