@@ -473,7 +473,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_grouped_gemm_kernel(
 // ---------------------------------------------------------------------------
 constexpr int kSmWaves = 8;
 
-template <int MT, typename OUT>
+template <int MT, int NC, typename OUT>
 __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_kernel(const uint8_t* __restrict__ a,
                                                                           const float* __restrict__ a_s, int64_t as_rs,
                                                                           int64_t as_cs, const uint8_t* __restrict__ b,
@@ -481,16 +481,24 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_kernel(const ui
                                                                           OUT* __restrict__ c,
                                                                           const uint16_t* __restrict__ bias, int M,
                                                                           int N, int K) {
-    __shared__ float red[kSmWaves][MT][64][4];
+    // NC groups of 16 weight columns per workgroup: the activation fragments of a K block are loaded once per wave
+    // and used for all of them (with NC = 2 half as many workgroups re-read the activation rows)
+    static_assert(NC * MT <= kSmWaves, "one wave reduces one (column group, row sub-tile) pair");
+    __shared__ float red[kSmWaves][NC * MT][64][4];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int frow = lane & 15, fk = lane >> 4;
-    const int n0 = blockIdx.x * 16;
-    const int KB = K >> 7;
+    const int n0 = blockIdx.x * (16 * NC);
+    const int KB = K >> 7, NB = (N + 127) >> 7;
     const int m_base = blockIdx.y * (MT * 16);     // grid.y splits the rows when there are few column groups
-    const int nrow = min(n0 + frow, N - 1);
-    const uint8_t* bp = b + (int64_t)nrow * K + fk * 32;
-    const float* bsp = b_s + (int64_t)(n0 >> 7) * KB;
+    const uint8_t* bp[NC];
+    const float* bsp[NC];
+#pragma unroll
+    for (int j = 0; j < NC; ++j) {
+        const int nrow = min(n0 + 16 * j + frow, N - 1);
+        bp[j] = b + (int64_t)nrow * K + fk * 32;
+        bsp[j] = b_s + (int64_t)min((n0 + 16 * j) >> 7, NB - 1) * KB;
+    }
     const uint8_t* ap[MT];
     const float* asp[MT];
 #pragma unroll
@@ -500,27 +508,32 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_kernel(const ui
         asp[i] = a_s + (int64_t)m * as_rs;
     }
 
-    floatx4 acc[MT];
+    floatx4 acc[NC][MT];
 #pragma unroll
-    for (int i = 0; i < MT; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < NC; ++j)
+#pragma unroll
+        for (int i = 0; i < MT; ++i) acc[j][i] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    // everything one K block needs: B fragment, MT A fragments, MT activation scales, the weight scale
+    // everything one K block needs: NC B fragments, MT A fragments, MT activation scales, NC weight scales
     struct Operands {
-        uint4 blo, bhi;
+        uint4 blo[NC], bhi[NC];
         intx4 alo[MT], ahi[MT];
         float sa[MT];
-        float sb;
+        float sb[NC];
     };
     auto load_block = [&](int kb, Operands& o) {
-        o.blo = load_nt16(bp + (int64_t)kb * 128);
-        o.bhi = load_nt16(bp + (int64_t)kb * 128 + 16);
+#pragma unroll
+        for (int j = 0; j < NC; ++j) {
+            o.blo[j] = load_nt16(bp[j] + (int64_t)kb * 128);
+            o.bhi[j] = load_nt16(bp[j] + (int64_t)kb * 128 + 16);
+            o.sb[j] = bsp[j][kb];
+        }
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
             o.alo[i] = *reinterpret_cast<const intx4*>(ap[i] + (int64_t)kb * 128);
             o.ahi[i] = *reinterpret_cast<const intx4*>(ap[i] + (int64_t)kb * 128 + 16);
             o.sa[i] = asp[i][(int64_t)kb * as_cs];
         }
-        o.sb = bsp[kb];
     };
     Operands cur, nxt;
     int kb = wave;
@@ -528,40 +541,45 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_kernel(const ui
     for (; kb < KB; kb += kSmWaves) {
         const bool more = kb + kSmWaves < KB;
         if (more) load_block(kb + kSmWaves, nxt);   // in flight while this block's MFMAs run
-        const intx8 fb = intx8{(int)cur.blo.x, (int)cur.blo.y, (int)cur.blo.z, (int)cur.blo.w,
-                               (int)cur.bhi.x, (int)cur.bhi.y, (int)cur.bhi.z, (int)cur.bhi.w};
 #pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            const intx8 fa = intx8{cur.alo[i][0], cur.alo[i][1], cur.alo[i][2], cur.alo[i][3],
-                                   cur.ahi[i][0], cur.ahi[i][1], cur.ahi[i][2], cur.ahi[i][3]};
-            const float sc = cur.sa[i] * cur.sb;
-            const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
-            const floatx4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, zero, 0, 0, 0, 0, 0, 0);
-            acc[i][0] = __builtin_fmaf(p[0], sc, acc[i][0]);
-            acc[i][1] = __builtin_fmaf(p[1], sc, acc[i][1]);
-            acc[i][2] = __builtin_fmaf(p[2], sc, acc[i][2]);
-            acc[i][3] = __builtin_fmaf(p[3], sc, acc[i][3]);
+        for (int j = 0; j < NC; ++j) {
+            const intx8 fb = intx8{(int)cur.blo[j].x, (int)cur.blo[j].y, (int)cur.blo[j].z, (int)cur.blo[j].w,
+                                   (int)cur.bhi[j].x, (int)cur.bhi[j].y, (int)cur.bhi[j].z, (int)cur.bhi[j].w};
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                const intx8 fa = intx8{cur.alo[i][0], cur.alo[i][1], cur.alo[i][2], cur.alo[i][3],
+                                       cur.ahi[i][0], cur.ahi[i][1], cur.ahi[i][2], cur.ahi[i][3]};
+                const float sc = cur.sa[i] * cur.sb[j];
+                const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+                const floatx4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, zero, 0, 0, 0, 0, 0, 0);
+                acc[j][i][0] = __builtin_fmaf(p[0], sc, acc[j][i][0]);
+                acc[j][i][1] = __builtin_fmaf(p[1], sc, acc[j][i][1]);
+                acc[j][i][2] = __builtin_fmaf(p[2], sc, acc[j][i][2]);
+                acc[j][i][3] = __builtin_fmaf(p[3], sc, acc[j][i][3]);
+            }
         }
         if (more) cur = nxt;
     }
 #pragma unroll
-    for (int i = 0; i < MT; ++i)
+    for (int j = 0; j < NC; ++j)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) red[wave][i][lane][e] = acc[i][e];
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) red[wave][j * MT + i][lane][e] = acc[j][i][e];
     __syncthreads();
-    if (wave < MT) {
-        // wave i reduces row sub-tile i (fixed order, so results do not depend on timing)
-        const int i = wave;
+    if (wave < NC * MT) {
+        // wave (j, i) reduces column group j, row sub-tile i (fixed order, so results do not depend on timing)
+        const int j = wave / MT, i = wave % MT;
         const bool vec_ok = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
         float v[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             float t = 0.0f;
 #pragma unroll
-            for (int w = 0; w < kSmWaves; ++w) t += red[w][i][lane][e];
+            for (int w = 0; w < kSmWaves; ++w) t += red[w][wave][lane][e];
             v[e] = t;
         }
-        const int m = m_base + i * 16 + frow, n = n0 + 4 * fk;
+        const int m = m_base + i * 16 + frow, n = n0 + 16 * j + 4 * fk;
         if (bias != nullptr) {
 #pragma unroll
             for (int e = 0; e < 4; ++e)
@@ -848,14 +866,21 @@ static int dispatch(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t a
         const int sub = (M + 15) / 16;
         int mt = sub;
         if ((N + 15) / 16 < 200 && sub >= 2) mt = (sub + 1) / 2;
-        dim3 grid((unsigned)((N + 15) / 16), (unsigned)((sub + mt - 1) / mt));
-#define MDY_SM(MT)                                                                                                 \
-    hipLaunchKernelGGL((fp8_gemm_smallm_kernel<MT, OUT>), grid, dim3(kSmWaves * 64), 0, stream, a, a_s, as_rs, as_cs, b, b_s, \
-                       c, bias, M, N, K)
-        if (mt == 1) MDY_SM(1);
-        else if (mt == 2) MDY_SM(2);
-        else if (mt == 3) MDY_SM(3);
-        else MDY_SM(4);
+        // two column groups per workgroup when that still leaves enough workgroups: the activation rows are
+        // fetched by half as many of them (measured: pays from 17 rows on with 288 workgroups, from 5 rows on with
+        // 512; M=31, N=18432, K=7168: 70 -> 59 us)
+        const long wgs32 = (N + 31) / 32;
+        const bool two = mt <= 2 && ((M > 16 && wgs32 >= 288) || (M > 4 && wgs32 >= 512));
+        dim3 grid((unsigned)(two ? (N + 31) / 32 : (N + 15) / 16), (unsigned)((sub + mt - 1) / mt));
+#define MDY_SM(MT, NC)                                                                                             \
+    hipLaunchKernelGGL((fp8_gemm_smallm_kernel<MT, NC, OUT>), grid, dim3(kSmWaves * 64), 0, stream, a, a_s, as_rs, as_cs, b, \
+                       b_s, c, bias, M, N, K)
+        if (two && mt == 1) MDY_SM(1, 2);
+        else if (two) MDY_SM(2, 2);
+        else if (mt == 1) MDY_SM(1, 1);
+        else if (mt == 2) MDY_SM(2, 1);
+        else if (mt == 3) MDY_SM(3, 1);
+        else MDY_SM(4, 1);
 #undef MDY_SM
         return (int)hipGetLastError();
     }

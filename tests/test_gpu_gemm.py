@@ -155,7 +155,8 @@ def test_gemm_exact_integer_random_shapes():
         if torch.rand(1, generator=g) < 0.1:
             K += int(torch.randint(1, 128, (1,), generator=g))          # ragged K: scalar kernel
         shapes.append((M, N, K))
-    shapes += [(48, 26000, 256), (64, 16500, 512), (33, 6400, 4096), (5, 25700, 384)]   # strip / wide-weight rules
+    shapes += [(48, 26000, 256), (64, 16500, 512), (33, 6400, 4096), (5, 25700, 384),   # strip / wide-weight rules
+               (20, 9300, 384), (31, 18433, 256), (8, 16390, 512), (16, 24576, 128)]    # two column groups per workgroup
     for M, N, K in shapes:
         gi = torch.Generator().manual_seed(M * 7 + N * 3 + K)
         ai = torch.randint(-2, 3, (M, K), generator=gi)
