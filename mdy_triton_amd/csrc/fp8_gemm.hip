@@ -359,10 +359,18 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
     const uint16_t* __restrict__ bias, int M, int N, int K, int ldc, int tiles_m, int tiles_n) {
-    int tm, tn;
-    const Duty duty = tile_of(xcd_contiguous(blockIdx.x, tiles_m * tiles_n), tiles_m, tiles_n, tm, tn);
-    fp8_gemm_tile<BM, BN, WGM, WGN, STAGES, OUT>(a, a_s, as_rs, as_cs, as_bytes, b, b_s, c, bias, tm * BM, M, M, tn * BN, N, K, ldc, duty,
-                                                 0, K >> 7);
+    // The grid may be smaller than the number of tiles (one workgroup per CU for the 256x256 tile): a workgroup
+    // then walks tiles blockIdx.x, blockIdx.x + gridDim.x, ... itself, which saves the ~4.5 us that pass between
+    // the end of a workgroup and the start of its successor on the same CU.  Workgroup ids keep their XCD
+    // (id % 8) from tile to tile when gridDim.x is a multiple of 8.
+    const int ntiles = tiles_m * tiles_n;
+    for (int pid = blockIdx.x; pid < ntiles; pid += gridDim.x) {
+        int tm, tn;
+        const Duty duty = tile_of(xcd_contiguous(pid, ntiles), tiles_m, tiles_n, tm, tn);
+        fp8_gemm_tile<BM, BN, WGM, WGN, STAGES, OUT>(a, a_s, as_rs, as_cs, as_bytes, b, b_s, c, bias, tm * BM, M, M, tn * BN, N, K, ldc,
+                                                     duty, 0, K >> 7);
+        __syncthreads();   // every wave has left the tile's LDS buffers before the next tile's copies land in them
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -751,18 +759,21 @@ __global__ __launch_bounds__(256) void fp8_gemm_scalar_kernel(const uint8_t* __r
         reinterpret_cast<float*>(c)[(int64_t)m * N + n] = acc;
 }
 
+constexpr int kCUs = 256;   // workgroups of the big tile that run at once (one per CU)
+
 template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT>
 static int launch_mfma(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, uint32_t as_bytes,
                        const uint8_t* b, const float* b_s, OUT* c, const uint16_t* bias, int M, int N, int K,
                        int ldc, hipStream_t stream) {
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-    dim3 grid((unsigned)(tiles_m * tiles_n)), block(WGM * WGN * 64);
+    // the 256x256 tile fills a CU's LDS: one workgroup per CU that walks its tiles itself
+    const int wgs = (BM * BN >= 256 * 256 && tiles_m * tiles_n > kCUs) ? kCUs : tiles_m * tiles_n;
+    dim3 grid((unsigned)wgs), block(WGM * WGN * 64);
     hipLaunchKernelGGL((fp8_gemm_mfma_kernel<BM, BN, WGM, WGN, STAGES, OUT>), grid, block, 0, stream, a, a_s, (int)as_rs,
                        (int)as_cs, as_bytes, b, b_s, c, bias, M, N, K, ldc, tiles_m, tiles_n);
     return (int)hipGetLastError();
 }
 
-constexpr int kCUs = 256;   // workgroups of the big tile that run at once (one per CU)
 
 // How many 256-wide tile columns the 256x256 kernel should take when the tile count is not a
 // multiple of the CU count: if the last, partly filled round holds at most half a round of
