@@ -156,13 +156,15 @@ int mdy_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int6
                     int64_t K, int out_dtype, void* stream);
 
 /* The same GEMM with a caller-provided scratch buffer.  Shapes whose output tiles do not fill the GPU
- * (roughly 16 < M <= 1024 against a long K: small-batch prefill, large-batch decode) are cut along K as
+ * (roughly 32 < M <= 1024 against a long K: small-batch prefill, large-batch decode) are cut along K as
  * well; the fp32 partial sums of the K slices go through `workspace` and are added in a fixed order, so the
  * result is deterministic, but it may differ in the last bit from mdy_fp8_gemm_nt (another summation order).
+ * Large shapes with row-major activation scales (as_col_stride == 1) use the buffer for a [K/128, M] copy of
+ * the scales, which the tile kernels fetch with 32x fewer cache-line requests (about 3 % faster; same bits).
  * No counterpart in the reference (its Triton kernel / DeepGEMM never split K); the Python wrappers fp8_gemm
  * and fp8_matmul call it with a torch-allocated buffer.
  *
- *   mdy_fp8_gemm_workspace_bytes(M, N, K)  bytes of workspace with which this shape runs split (0: it never does)
+ *   mdy_fp8_gemm_workspace_bytes(M, N, K)  bytes of workspace this shape can use (0: none)
  *   workspace        device memory, 16-byte aligned, workspace_bytes long; may be NULL / too small: the call
  *                    then is mdy_fp8_gemm_nt.  Calls that overlap in time need separate workspaces.
  */

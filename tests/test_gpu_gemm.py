@@ -195,9 +195,31 @@ def test_ops_follow_torchs_current_stream():
     assert torch.equal(xq1.view(torch.uint8), xq0.view(torch.uint8)) and torch.equal(xs1, xs0) and torch.equal(c1, c0)
 
 
+def test_gemm_transposed_scale_scratch_is_bit_identical():
+    """Big shapes with row-major activation scales and a workspace run the same tile kernels on a transposed copy of
+    the scales: only addresses change, so the result equals the single-call path bit for bit (ragged M, bias)."""
+    M, N, K = 4000, 7200, 7168
+    g = torch.Generator().manual_seed(77)
+    a = torch.randint(0, 120, (M, K), generator=g, dtype=torch.uint8).view(FP8).to(DEV)
+    b = torch.randint(0, 120, (N, K), generator=g, dtype=torch.uint8).view(FP8).to(DEV)
+    a_s = (torch.rand(M, K // 128, generator=g) * 1e-3 + 1e-3).to(DEV)
+    b_s = (torch.rand((N + 127) // 128, K // 128, generator=g) * 1e-3 + 1e-3).to(DEV)
+    bias = torch.randn(N, generator=g).bfloat16().to(DEV)
+    need = _lib.load().mdy_fp8_gemm_workspace_bytes(M, N, K)
+    assert 0 < need < 2 * M * (K // 128) * 4
+    ws = torch.full((need,), 0xFF, device=DEV, dtype=torch.uint8)
+    for dtype in (torch.bfloat16, torch.float32):
+        rc0, plain = _raw_gemm(a, a_s, b, b_s, bias, dtype, "plain")
+        rc1, with_ws = _raw_gemm(a, a_s, b, b_s, bias, dtype, ws)
+        assert rc0 == 0 and rc1 == 0 and torch.equal(plain, with_ws)
+        assert not torch.isnan(with_ws.float()).any()
+
+
 def test_gemm_workspace_query():
     lib = _lib.load()
-    assert lib.mdy_fp8_gemm_workspace_bytes(4096, 18432, 7168) == 0      # fills the GPU: never split
+    big = lib.mdy_fp8_gemm_workspace_bytes(4096, 18432, 7168)            # fills the GPU: never split, but room for
+    assert 4096 * 56 * 4 <= big < 4096 * 56 * 4 + 256                    # the transposed activation scales
+    assert lib.mdy_fp8_gemm_workspace_bytes(4096, 1536, 7168) == 0       # too short a GEMM for that to pay
     assert lib.mdy_fp8_gemm_workspace_bytes(32, 7168, 16384) == 0        # weight-streaming kernel
     assert lib.mdy_fp8_gemm_workspace_bytes(128, 7168, 2048) == 0        # K too short to cut
     assert lib.mdy_fp8_gemm_workspace_bytes(128, 7168, 5000) == 0        # ragged K: scalar kernel
