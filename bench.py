@@ -346,7 +346,8 @@ def table(torch, m, timer, dev):
     for mg in (512, 16):
         Mt = G * mg
         aq = torch.randint(0, 120, (Mt, Kg), dtype=torch.uint8, device=dev).view(FP8)
-        asg = torch.rand(Mt, Kg // 128, device=dev)
+        asg = torch.rand(Kg // 128, Mt, device=dev).t()     # logical [Mt, K/128], strides (1, Mt): what
+        #                                                       group_per_token_cast_to_fp8 returns
         us = timer.run(lambda: m.fp8_grouped_matmul(aq, asg, bq, bsg, [mg] * G), 10)[0]
         if mg >= 256:
             line("grouped fp8_gemm %d experts x %d rows, N=%d K=%d" % (G, mg, Ng, Kg), us, 2.0 * Mt * Ng * Kg, "TFLOP/s", PEAK_FP8_TFLOPS)
