@@ -36,10 +36,10 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E, published
 
 # HBM bytes per fp8_gemm call at the C3 shape (both of its launches), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (KiB per dispatch, scaled by the same counters read on a plain copy kernel of known size); the runs are
-# summarised in profiles/bench_C3_hbm_traffic.txt: FETCH_SIZE (349 081 + 72 423) KiB x 1.9997 (copy-kernel
-# calibration) = 863.1 MB read, WRITE_SIZE (134 165 + 16 409) KiB x 1.0 = 154.2 MB written; algorithmic bytes are
+# summarised in profiles/bench_C3_hbm_traffic.txt: FETCH_SIZE (347 857 + 72 233) KiB x 1.9997 (copy-kernel
+# calibration) = 860.2 MB read, WRITE_SIZE (134 131 + 16 418) KiB x 1.0 = 154.2 MB written; algorithmic bytes are
 # 313 MB (the A and B panels are re-fetched by the eight XCD-local L2s).
-GEMM_C3_HBM_TRAFFIC_BYTES = 1017.3e6
+GEMM_C3_HBM_TRAFFIC_BYTES = 1014.4e6
 
 WORKLOADS = {
     # name: (activation kind, M, N, K, description)
@@ -266,7 +266,7 @@ def main():
         "config": {"workload": "%s %s; step = act_quant + fp8_gemm (pre-quantized weight)" % (args.workload, desc),
                    "M": M, "N": N, "K": K},
         "roofline": {"bound": "mfma",
-                     "kernel": "fp8_gemm (one call = fp8_gemm_mfma_kernel<256,256> on the first 16384 columns + <128,256> on the last 2048)"
+                     "kernel": "fp8_gemm (one call = transpose_scales_kernel + fp8_gemm_mfma_kernel<256,256> on the first 16384 columns + <128,256> on the last 2048)"
                      if args.workload == "C3" else "fp8_gemm",
                      "achieved": round(achieved, 2), "peak": PEAK_FP8_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP8_TFLOPS, 4),
