@@ -11,12 +11,15 @@ X[4096, 7168] bf16 ~ N(0,1), W[18432, 7168] e4m3fn with 128x128 fp32 block scale
 
 Prints ONE JSON line on stdout:
   value        whole-step throughput in TFLOP/s (2*M*N*K / step time, quantizer included)
-  roofline     the dominant kernel (fp8_gemm): algorithmic FLOPs per launch / its
-               average launch duration, measured with HIP events on the launch stream
-               inside the timed region, against the dense FP8 MFMA peak
+  roofline     the dominant kernel (fp8_gemm): algorithmic FLOPs per call / its average
+               duration, measured with HIP events on the launch stream inside the timed
+               region, against the dense FP8 MFMA peak (a call is fp8_gemm() as a user
+               makes it: the wrapper passes a scratch buffer, so at this shape the library
+               runs a 4 us scale-transposition kernel and two tile launches)
   kernels      the same for act_quant and weight_dequant against the HBM peak
                (algorithmic bytes: 3.03125*M*K and 3*N*K + 4*ceil(N/128)*ceil(K/128)),
-               each timed alone, cold cache (a 512 MiB buffer is rewritten before every launch)
+               each timed alone, cold cache (a 512 MiB buffer is rewritten before every launch),
+               and per launch of several back-to-back launches on uncached buffers (us_streamed)
   cpu_baseline the CPU oracle (dequantize + fp32 matmul, torch CPU ops) on a bounded
                sample of the same workload, on the host cores of this box
 With --table a per-kernel table for every benchmark configuration goes to stderr.
