@@ -96,6 +96,19 @@ struct Duty {
     int a_duty, a_sh, b_duty, b_sh;
 };
 
+// LDS of one tile workgroup, carved out of a pool that the kernel declares: the ring of A and B panels, the ring of activation scales, the tile's weight
+// scales for all K blocks, and a dummy area for copies that must go nowhere.
+template <int BM, int BN, int WAVES, int STAGES>
+struct TileLds {
+    static constexpr int NBS = (BN + 127) / 128;
+    static constexpr int a_off = 0;
+    static constexpr int b_off = a_off + STAGES * BM * 128;
+    static constexpr int s_off = b_off + STAGES * BN * 128;
+    static constexpr int bs_off = s_off + (STAGES * BM * 4 + 255) / 256 * 256;
+    static constexpr int dummy_off = bs_off + NBS * 512 * 4;
+    static constexpr int bytes = dummy_off + WAVES * 512;
+};
+
 // One BM x BN tile of C: WGM x WGN waves, each wave (BM/WGM) x (BN/WGN).
 //   rows m0 .. min(m0+BM, m_end) of a (m_end = end of the matrix, or of the expert group the tile belongs to),
 //   columns n0 .. of b / b_s / bias (already offset to the group's weight), K % 128 == 0, K <= 65536,
@@ -120,7 +133,7 @@ __device__ __forceinline__ void fp8_gemm_tile(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
     const uint16_t* __restrict__ bias, int m0, int m_end, int m_total, int n0, int N, int K, int ldc, const Duty duty,
-    int kb0, int kb1) {
+    int kb0, int kb1, uint8_t* __restrict__ pool) {
     constexpr int WAVES = WGM * WGN;
     constexpr int WM = BM / WGM, WN = BN / WGN, TI = WM / 16, TJ = WN / 16;
     constexpr int PASS_ROWS = WAVES * 8;  // rows copied by one DMA instruction of every wave
@@ -153,12 +166,13 @@ __device__ __forceinline__ void fp8_gemm_tile(
     static_assert(NS % 2 == 0 && NS >= 2, "the first streamed fragment of the next K block reuses queue slot 0");
     static_assert(TOUCH < TB, "not enough slots in front of the barrier");
 
-    constexpr int NBS = (BN + 127) / 128;
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_a[STAGES][BM * 128];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_b[STAGES][BN * 128];
-    __shared__ __attribute__((aligned(256))) float lds_s[STAGES][BM];
-    __shared__ __attribute__((aligned(256))) float lds_bs[NBS][512];   // weight scales of the tile, all K blocks
-    __shared__ __attribute__((aligned(256))) uint8_t lds_dummy[WAVES * 512];   // target of copies that must go nowhere
+    using L = TileLds<BM, BN, WAVES, STAGES>;
+    constexpr int NBS = L::NBS;
+    uint8_t(*lds_a)[BM * 128] = reinterpret_cast<uint8_t(*)[BM * 128]>(pool + L::a_off);     // [STAGES]
+    uint8_t(*lds_b)[BN * 128] = reinterpret_cast<uint8_t(*)[BN * 128]>(pool + L::b_off);     // [STAGES]
+    float(*lds_s)[BM] = reinterpret_cast<float(*)[BM]>(pool + L::s_off);                      // [STAGES]
+    float(*lds_bs)[512] = reinterpret_cast<float(*)[512]>(pool + L::bs_off);                  // [NBS] weight scales, all K blocks
+    uint8_t* lds_dummy = pool + L::dummy_off;                                                 // target of copies that must go nowhere
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -363,12 +377,13 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
     // then walks tiles blockIdx.x, blockIdx.x + gridDim.x, ... itself, which saves the ~4.5 us that pass between
     // the end of a workgroup and the start of its successor on the same CU.  Workgroup ids keep their XCD
     // (id % 8) from tile to tile when gridDim.x is a multiple of 8.
+    __shared__ __attribute__((aligned(1024))) uint8_t pool[TileLds<BM, BN, WGM * WGN, STAGES>::bytes];
     const int ntiles = tiles_m * tiles_n;
     for (int pid = blockIdx.x; pid < ntiles; pid += gridDim.x) {
         int tm, tn;
         const Duty duty = tile_of(xcd_contiguous(pid, ntiles), tiles_m, tiles_n, tm, tn);
         fp8_gemm_tile<BM, BN, WGM, WGN, STAGES, OUT>(a, a_s, as_rs, as_cs, as_bytes, b, b_s, c, bias, tm * BM, M, M, tn * BN, N, K, ldc,
-                                                     duty, 0, K >> 7);
+                                                     duty, 0, K >> 7, pool);
         __syncthreads();   // every wave has left the tile's LDS buffers before the next tile's copies land in them
     }
 }
@@ -384,6 +399,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_splitk_kernel(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, float* __restrict__ ws, int M, int N, int K,
     int tiles_m, int tiles_n, int ksplit, int kb_per) {
+    __shared__ __attribute__((aligned(1024))) uint8_t pool[TileLds<BM, BN, WGM * WGN, STAGES>::bytes];
     const int ntiles = tiles_m * tiles_n;
     // slab-major order: the workgroups that share an XCD work on the same K range, so they share its A rows
     const int pid = xcd_contiguous(blockIdx.x, ntiles * ksplit);
@@ -392,7 +408,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_splitk_kernel(
     const Duty duty = tile_of(pid - ks * ntiles, tiles_m, tiles_n, tm, tn);
     const int kb0 = ks * kb_per, kb1 = min(K >> 7, kb0 + kb_per);
     fp8_gemm_tile<BM, BN, WGM, WGN, STAGES, float>(a, a_s, as_rs, as_cs, as_bytes, b, b_s, ws + (size_t)ks * M * N, nullptr,
-                                                   tm * BM, M, M, tn * BN, N, K, N, duty, kb0, kb1);
+                                                   tm * BM, M, M, tn * BN, N, K, N, duty, kb0, kb1, pool);
 }
 
 template <typename OUT, bool VEC>
@@ -445,6 +461,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_grouped_gemm_kernel(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
     const uint16_t* __restrict__ bias, int N, int K, int tiles_n, const GroupTable tbl) {
+    __shared__ __attribute__((aligned(1024))) uint8_t pool[TileLds<BM, BN, WGM * WGN, 2>::bytes];
     const int G = tbl.n_groups;
     const int pid = xcd_contiguous(blockIdx.x, tbl.tile_start[G] * tiles_n);
     const int trow = pid / tiles_n;               // position in units of whole tile rows
@@ -468,7 +485,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_grouped_gemm_kernel(
                                          b_s + (size_t)g * NB * KB, c, bias ? bias + (size_t)g * N : nullptr,
                                          __builtin_amdgcn_readfirstlane(r0 + tm * BM), r1,
                                          __builtin_amdgcn_readfirstlane(tbl.row_start[G]), __builtin_amdgcn_readfirstlane(tn * BN), N, K, N,
-                                         duty, 0, K >> 7);
+                                         duty, 0, K >> 7, pool);
 }
 
 // ---------------------------------------------------------------------------
