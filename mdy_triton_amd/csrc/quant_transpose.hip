@@ -48,6 +48,7 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
     constexpr int WAVES = NRG / 4;
     __shared__ float col_part[NRG][128];  // per row group partial column maxima
     __shared__ float col_amax[128];
+    __shared__ float row_sc[128];         // the tile's 128 row scales, written out as one contiguous run
     __shared__ float blk_part[WAVES];
     __shared__ __attribute__((aligned(16))) uint8_t tile[128][128 + 8];   // [k][m], transposed
 
@@ -106,7 +107,7 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
             for (int j = 0; j < 8; ++j) q[j] = qt_quot<false>(f[i][j], sc, r);
         }
         store_nt8(y + (int64_t)row * PK + c0, make_uint2(pack4_e4m3(q[0], q[1], q[2], q[3]), pack4_e4m3(q[4], q[5], q[6], q[7])));
-        if ((t & 15) == 0) s[(int64_t)bk * s_kb_stride + row] = sc;
+        if ((t & 15) == 0) row_sc[rg * RPT + i] = sc;
     }
 
     // ---- (2) scales of the transposed copy
@@ -122,6 +123,7 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
             col_amax[t] = m;
             // logical s_t[k, a]: stored [A][PK]
             s_t[(int64_t)bm * PK + bk * 128 + t] = group_scale<1>(m);
+            s[(int64_t)bk * s_kb_stride + bm * 128 + t] = row_sc[t];
         }
         __syncthreads();
 #pragma unroll
@@ -138,6 +140,7 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
 #pragma unroll
         for (int w = 1; w < WAVES; ++w) bmax = fmaxf(bmax, blk_part[w]);
         if (t == 0) s_t[(int64_t)bk * (PM >> 7) + bm] = group_scale<1>(bmax);
+        if (t < 128) s[(int64_t)bk * s_kb_stride + bm * 128 + t] = row_sc[t];
 #pragma unroll
         for (int j = 0; j < 8; ++j) tamax[j] = bmax;
     }
