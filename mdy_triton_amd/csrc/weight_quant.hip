@@ -111,7 +111,9 @@ __global__ __launch_bounds__(256) void weight_quant_kernel(const uint16_t* __res
         for (int i = 0; i < 8; ++i) {
             const int kk = (t >> 4) + 16 * i;
             const int nn = (t & 15) * 8;
-            store_nt8(y_t + (int64_t)(bk * 128 + kk) * PN + bn * 128 + nn, *reinterpret_cast<const uint2*>(&tile[kk][nn]));
+            // cached store: neighbouring tiles complete the rows of y_t in L2 (1-7 % faster than non-temporal here)
+            *reinterpret_cast<uint2*>(y_t + (int64_t)(bk * 128 + kk) * PN + bn * 128 + nn) =
+                *reinterpret_cast<const uint2*>(&tile[kk][nn]);
         }
     }
 }
