@@ -46,7 +46,7 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
                                                                int PK, int64_t s_kb_stride) {
     constexpr int NRG = 128 / RPT;        // row groups of RPT consecutive rows; 16 threads (8 columns each) per group
     constexpr int WAVES = NRG / 4;
-    __shared__ float col_part[NRG][128];  // per row group partial column maxima
+    __shared__ float col_part[WAVES][128];  // per wave (4 row groups) partial column maxima
     __shared__ float col_amax[128];
     __shared__ float row_sc[128];         // the tile's 128 row scales, written out as one contiguous run
     __shared__ float blk_part[WAVES];
@@ -114,12 +114,17 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
     float tamax[8];   // amax that scales this thread's 8 columns in the transposed copy
     if (TMODE == 0) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) col_part[rg][cl + j] = cmax[j];
+        for (int j = 0; j < 8; ++j) {
+            // the 4 row groups of a wave hold the same columns in lanes 16 apart: fold them before going to LDS
+            float m = fmaxf(cmax[j], __shfl_xor(cmax[j], 16, 64));
+            m = fmaxf(m, __shfl_xor(m, 32, 64));
+            if (lane < 16) col_part[wave][cl + j] = m;
+        }
         __syncthreads();
         if (t < 128) {
             float m = 0.0f;
 #pragma unroll
-            for (int g = 0; g < NRG; ++g) m = fmaxf(m, col_part[g][t]);
+            for (int g = 0; g < WAVES; ++g) m = fmaxf(m, col_part[g][t]);
             col_amax[t] = m;
             // logical s_t[k, a]: stored [A][PK]
             s_t[(int64_t)bm * PK + bk * 128 + t] = group_scale<1>(m);
