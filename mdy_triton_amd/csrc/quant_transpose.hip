@@ -47,7 +47,9 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
     constexpr int NRG = 128 / RPT;        // row groups of RPT consecutive rows; 16 threads (8 columns each) per group
     constexpr int WAVES = NRG / 4;
     __shared__ float col_part[WAVES][128];  // per wave (4 row groups) partial column maxima
-    __shared__ float col_amax[128];
+    __shared__ __attribute__((aligned(16))) float col_amax[128];
+    __shared__ __attribute__((aligned(16))) float col_sc[128];   // per column: scale of the transposed copy ...
+    __shared__ __attribute__((aligned(16))) float col_rc[128];   // ... and its reciprocal, computed once per column
     __shared__ float row_sc[128];         // the tile's 128 row scales, written out as one contiguous run
     __shared__ float blk_part[WAVES];
     __shared__ __attribute__((aligned(16))) uint8_t tile[128][128 + 8];   // [k][m], transposed
@@ -112,6 +114,7 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
 
     // ---- (2) scales of the transposed copy
     float tamax[8];   // amax that scales this thread's 8 columns in the transposed copy
+    float tsc[8], tr[8];
     if (TMODE == 0) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
@@ -125,14 +128,21 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
             float m = 0.0f;
 #pragma unroll
             for (int g = 0; g < WAVES; ++g) m = fmaxf(m, col_part[g][t]);
+            const float sc = group_scale<1>(m);
             col_amax[t] = m;
+            col_sc[t] = sc;
+            col_rc[t] = 1.0f / sc;
             // logical s_t[k, a]: stored [A][PK]
-            s_t[(int64_t)bm * PK + bk * 128 + t] = group_scale<1>(m);
+            s_t[(int64_t)bm * PK + bk * 128 + t] = sc;
             s[(int64_t)bk * s_kb_stride + bm * 128 + t] = row_sc[t];
         }
         __syncthreads();
 #pragma unroll
-        for (int j = 0; j < 8; ++j) tamax[j] = col_amax[cl + j];
+        for (int j = 0; j < 8; ++j) {
+            tamax[j] = col_amax[cl + j];
+            tsc[j] = col_sc[cl + j];
+            tr[j] = col_rc[cl + j];
+        }
     } else {
         float m = 0.0f;
 #pragma unroll
@@ -146,17 +156,17 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
         for (int w = 1; w < WAVES; ++w) bmax = fmaxf(bmax, blk_part[w]);
         if (t == 0) s_t[(int64_t)bk * (PM >> 7) + bm] = group_scale<1>(bmax);
         if (t < 128) s[(int64_t)bk * s_kb_stride + bm * 128 + t] = row_sc[t];
+        const float bsc = group_scale<1>(bmax), brc = 1.0f / bsc;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) tamax[j] = bmax;
+        for (int j = 0; j < 8; ++j) {
+            tamax[j] = bmax;
+            tsc[j] = bsc;
+            tr[j] = brc;
+        }
     }
-    float tsc[8], tr[8];
     bool tfast = true;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        tsc[j] = group_scale<1>(tamax[j]);
-        tr[j] = 1.0f / tsc[j];
-        tfast = tfast && (tamax[j] <= 1e4f);
-    }
+    for (int j = 0; j < 8; ++j) tfast = tfast && (tamax[j] <= 1e4f);
     uint32_t qlo[RPT], qhi[RPT];   // row i of the transposed copy's bytes: columns 0..3 | 4..7
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
