@@ -19,12 +19,14 @@
 
 namespace mdy {
 
-template <int MODE, bool VEC>
-__global__ __launch_bounds__(256) void weight_quant_kernel(const uint16_t* __restrict__ w, uint8_t* __restrict__ y,
+template <int MODE, bool VEC, int RPT>
+__global__ __launch_bounds__(2048 / RPT) void weight_quant_kernel(const uint16_t* __restrict__ w, uint8_t* __restrict__ y,
                                                             float* __restrict__ s, uint8_t* __restrict__ y_t,
                                                             float* __restrict__ s_t, int N, int K, int64_t w_row_stride,
                                                             int64_t w_col_stride, int PN, int PK) {
-    __shared__ float wave_max[4];
+    constexpr int NRG = 128 / RPT;     // row groups of RPT consecutive rows, 16 threads (8 columns each) per group
+    constexpr int WAVES = NRG / 4;
+    __shared__ float wave_max[WAVES];
     __shared__ __attribute__((aligned(16))) uint8_t tile[128][128 + 8];   // [k][n], transposed
 
     const int t = threadIdx.x;
@@ -33,12 +35,12 @@ __global__ __launch_bounds__(256) void weight_quant_kernel(const uint16_t* __res
     const int bn = blockIdx.y;  // block row (along N)
     const int bk = blockIdx.x;  // block column (along K)
     const int c0 = bk * 128 + (t & 15) * 8;
-    const int rbase = bn * 128 + (t >> 4) * 8;
+    const int rbase = bn * 128 + (t >> 4) * RPT;
 
-    float f[8][8];
+    float f[RPT][8];
     float m = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < RPT; ++i) {
         const int row = rbase + i;
         uint32_t wd[4] = {0u, 0u, 0u, 0u};
         if (row < N && c0 < K) {
@@ -60,12 +62,14 @@ __global__ __launch_bounds__(256) void weight_quant_kernel(const uint16_t* __res
             m = fmaxf(fmaxf(fabsf(f[i][2 * j]), fabsf(f[i][2 * j + 1])), m);
         }
     }
-    // wave-wide max, then across the 4 waves
+    // wave-wide max, then across the waves
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
     if (lane == 0) wave_max[wave] = m;
     __syncthreads();
-    const float amax = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+    float amax = wave_max[0];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) amax = fmaxf(amax, wave_max[w]);
 
     const float sc = group_scale<MODE>(amax);
     const bool fast = MODE == 0 ? fast_quotient_ok<0>(amax) : (amax <= 1e4f);
@@ -74,9 +78,9 @@ __global__ __launch_bounds__(256) void weight_quant_kernel(const uint16_t* __res
         s[(int64_t)bn * (PK >> 7) + bk] = sc;
         if (s_t) s_t[(int64_t)bk * (PN >> 7) + bn] = sc;
     }
-    uint32_t qlo[8], qhi[8];   // row i of the quantized bytes: columns 0..3 | 4..7
+    uint32_t qlo[RPT], qhi[RPT];   // row i of the quantized bytes: columns 0..3 | 4..7
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < RPT; ++i) {
         float q[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
@@ -100,20 +104,36 @@ __global__ __launch_bounds__(256) void weight_quant_kernel(const uint16_t* __res
         qhi[i] = o.y;
     }
     if (y_t) {
-        uint32_t tb[8][2];   // [column j][rows 0..3 | 4..7]
-        transpose8x8_bytes(qlo, qhi, tb);
+        // column j of the thread's RPT x 8 bytes = RPT consecutive bytes of row (t%16)*8 + j of the transposed tile
+        const int cl = (t & 15) * 8, rg = t >> 4;
+        if (RPT == 8) {
+            uint32_t tb[8][2];   // [column j][rows 0..3 | 4..7]
+            uint32_t lo8[8], hi8[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-            *reinterpret_cast<uint2*>(&tile[(t & 15) * 8 + j][(t >> 4) * 8]) = make_uint2(tb[j][0], tb[j][1]);
+            for (int i = 0; i < 8; ++i) { lo8[i] = qlo[i % RPT]; hi8[i] = qhi[i % RPT]; }
+            transpose8x8_bytes(lo8, hi8, tb);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) *reinterpret_cast<uint2*>(&tile[cl + j][rg * 8]) = make_uint2(tb[j][0], tb[j][1]);
+        } else {
+            const uint32_t rl[4] = {qlo[0], qlo[1 % RPT], qlo[2 % RPT], qlo[3 % RPT]};
+            const uint32_t rh[4] = {qhi[0], qhi[1 % RPT], qhi[2 % RPT], qhi[3 % RPT]};
+            uint32_t c_lo[4], c_hi[4];
+            transpose4x4_bytes(rl, c_lo);
+            transpose4x4_bytes(rh, c_hi);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                *reinterpret_cast<uint32_t*>(&tile[cl + j][rg * 4]) = c_lo[j];
+                *reinterpret_cast<uint32_t*>(&tile[cl + 4 + j][rg * 4]) = c_hi[j];
+            }
+        }
         __syncthreads();
-        // y_t[k][n]: thread owns output columns (t%16)*8..+7 (n) of output rows t/16 + 16*i (k)
+        // y_t[k][n]: thread owns output columns (t%16)*8..+7 (n) of output rows t/16 + NRG*i (k)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int kk = (t >> 4) + 16 * i;
-            const int nn = (t & 15) * 8;
+        for (int i = 0; i < RPT; ++i) {
+            const int kk = rg + NRG * i;
             // cached store: neighbouring tiles complete the rows of y_t in L2 (1-7 % faster than non-temporal here)
-            *reinterpret_cast<uint2*>(y_t + (int64_t)(bk * 128 + kk) * PN + bn * 128 + nn) =
-                *reinterpret_cast<const uint2*>(&tile[kk][nn]);
+            *reinterpret_cast<uint2*>(y_t + (int64_t)(bk * 128 + kk) * PN + bn * 128 + cl) =
+                *reinterpret_cast<const uint2*>(&tile[kk][cl]);
         }
     }
 }
@@ -123,14 +143,16 @@ int launch_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t,
                         hipStream_t stream) {
     if (PN == 0 || PK == 0) return 0;
     dim3 grid((unsigned)(PK / 128), (unsigned)(PN / 128));
-    dim3 block(256);
+    // 512 threads per tile: 4 rows per thread, 56 VGPRs, 8 waves per SIMD (256 threads with 8 rows each need 89
+    // VGPRs and measured 1-5 % slower at every size tried)
+    dim3 block(512);
     const bool vec = (w_col_stride == 1) && (K % 8 == 0) && (w_row_stride % 8 == 0) &&
                      ((reinterpret_cast<uintptr_t>(w) & 15) == 0);
     const uint16_t* wp = static_cast<const uint16_t*>(w);
     uint8_t* yp = static_cast<uint8_t*>(y);
     uint8_t* ytp = static_cast<uint8_t*>(y_t);
-#define MDY_WQ(MODE, VEC)                                                                                      \
-    hipLaunchKernelGGL((weight_quant_kernel<MODE, VEC>), grid, block, 0, stream, wp, yp, s, ytp, s_t, (int)N, \
+#define MDY_WQ(MODE, VEC)                                                                                          \
+    hipLaunchKernelGGL((weight_quant_kernel<MODE, VEC, 4>), grid, block, 0, stream, wp, yp, s, ytp, s_t, (int)N, \
                        (int)K, w_row_stride, w_col_stride, (int)PN, (int)PK)
     if (mode == 0) {
         if (vec) MDY_WQ(0, true); else MDY_WQ(0, false);
