@@ -6,13 +6,13 @@
 // and _weight_quant_block_kernel
 // (/root/reference/triton_kernels/deepseekv3/fp8_kernel.py:88-122; plain amax/448).
 //
-// One 256-thread block per 128x128 tile.  Thread t owns columns (t%16)*8..+7 of
-// rows (t/16)*8 + i, i = 0..7: eight 16-byte loads kept in registers (the tile is
-// read from HBM exactly once), absmax by DPP inside 16-lane rows, ds_swizzle-free
-// cross-row reduction with __shfl_xor, four wave results combined through LDS.
+// One 512-thread block per 128x128 tile.  Thread t owns columns (t%16)*8..+7 of
+// rows (t/16)*4 + i, i = 0..3: four 16-byte loads kept in registers (the tile is
+// read from HBM exactly once), absmax reduced inside the wave with __shfl_xor,
+// the eight wave results combined through LDS.
 // The quotient is the same reciprocal + 2-FMA form as the activation quantizer.
-// The transposed copy goes through a padded LDS tile: a thread's 8 consecutive rows of one column are 8
-// consecutive bytes of a transposed row (8-byte LDS writes and reads).
+// The transposed copy goes through a padded LDS tile: a thread's 4 consecutive rows of one column are 4
+// consecutive bytes of a transposed row (4-byte LDS writes, 8-byte reads).
 //
 // HBM traffic per element: 2 B in + 1 B out (+ 1 B for the transposed copy).
 #include "common.h"
