@@ -66,7 +66,7 @@ __device__ __forceinline__ uint2 quantize8(const float (&f)[8], float amax, floa
     return out;
 }
 
-// grid.x = ceil(PK / 512), grid.y = ceil(PM / 8), block = 256
+// ceil(PK / 512) x ceil(PM / 8) blocks (grid_rows), block = 256
 template <int MODE, bool VEC>
 __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ y,
                                                          float* __restrict__ s, int M, int K, int64_t x_row_stride,
@@ -74,7 +74,7 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restri
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int col = blockIdx.x * 512 + lane * 8;  // first of this lane's 8 columns
-    const int row0 = blockIdx.y * kAqRowsPerBlock + wave * kAqRowsPerWave;
+    const int row0 = block_row() * kAqRowsPerBlock + wave * kAqRowsPerWave;   // rows >= PM are dropped below
     const bool col_in_out = col < PK;  // PK % 128 == 0, so whole 16-lane rows agree
 
     uint4 raw[kAqRowsPerWave];
@@ -122,8 +122,8 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restri
 int launch_act_quant(const void* x, void* y, float* s, int64_t M, int64_t K, int64_t x_row_stride, int64_t PM,
                      int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode, hipStream_t stream) {
     if (PM == 0 || PK == 0) return 0;
-    dim3 grid((unsigned)((PK + 511) / 512), (unsigned)((PM + kAqRowsPerBlock - 1) / kAqRowsPerBlock));
-    dim3 block(256);
+    dim3 grid, block(256);
+    if (!grid_rows((PK + 511) / 512, (PM + kAqRowsPerBlock - 1) / kAqRowsPerBlock, grid)) return kErrTooManyBlocks;
     const bool vec = (K % 8 == 0) && (x_row_stride % 8 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     uint8_t* yp = static_cast<uint8_t*>(y);

@@ -78,7 +78,6 @@ int mdy_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t, in
     if (N < 0 || K < 0 || PN < N || PK < K || PN > kMaxDim || PK > kMaxDim)
         return fail(MDY_E_SHAPE, "weight_quant: need 0 <= N <= PN, 0 <= K <= PK");
     if (PN % 128 != 0 || PK % 128 != 0) return fail(MDY_E_SHAPE, "weight_quant: PN=%lld, PK=%lld must be multiples of 128", (long long)PN, (long long)PK);
-    if (PN / 128 > 65535) return fail(MDY_E_SHAPE, "weight_quant: PN too large");
     if ((y_t == nullptr) != (s_t == nullptr)) return fail(MDY_E_NULL, "weight_quant: y_t and s_t must be given together");
     if (PN == 0 || PK == 0) return 0;
     if (!y || !s || (!w && N > 0 && K > 0)) return fail(MDY_E_NULL, "weight_quant: null pointer");
@@ -96,7 +95,6 @@ int mdy_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t,
     if (M < 0 || K < 0 || PM < M || PK < K || PM > kMaxDim || PK > kMaxDim)
         return fail(MDY_E_SHAPE, "quant_transpose: need 0 <= M <= PM, 0 <= K <= PK");
     if (PM % 128 != 0 || PK % 128 != 0) return fail(MDY_E_SHAPE, "quant_transpose: PM=%lld, PK=%lld must be multiples of 128", (long long)PM, (long long)PK);
-    if (PM / 128 > 65535) return fail(MDY_E_SHAPE, "quant_transpose: PM too large");
     if (s_kb_stride < PM) return fail(MDY_E_SHAPE, "quant_transpose: s_kb_stride=%lld < PM=%lld", (long long)s_kb_stride, (long long)PM);
     if (PM == 0 || PK == 0) return 0;
     if (!y || !s || !y_t || !s_t || (!x && M > 0 && K > 0)) return fail(MDY_E_NULL, "quant_transpose: null pointer");
@@ -119,10 +117,8 @@ int mdy_swiglu(const void* x, void* act, void* y, float* s, int64_t M, int64_t N
         if (PM == 0 || PN == 0) return 0;
         if (!s) return fail(MDY_E_NULL, "swiglu: y given without s");
         if (!aligned(y, 8) || !aligned(s, 4)) return fail(MDY_E_ALIGN, "swiglu: y must be 8-byte, s 4-byte aligned");
-        if ((PM + 7) / 8 > 65535) return fail(MDY_E_SHAPE, "swiglu: PM too large");
     } else {
         if (M == 0 || N == 0) return 0;
-        if ((M + 7) / 8 > 65535) return fail(MDY_E_SHAPE, "swiglu: M too large");
     }
     if (!x && M > 0 && N > 0) return fail(MDY_E_NULL, "swiglu: null x");
     if (M > 0 && x_row_stride < 2 * N) return fail(MDY_E_SHAPE, "swiglu: x_row_stride=%lld < 2N=%lld", (long long)x_row_stride, (long long)(2 * N));
@@ -136,7 +132,6 @@ int mdy_swiglu(const void* x, void* act, void* y, float* s, int64_t M, int64_t N
 int mdy_swiglu_bwd(const void* x, const void* dy, void* dx, int64_t M, int64_t N, int64_t x_row_stride, int gate_first,
                    void* stream) {
     if (M < 0 || N < 0 || M > kMaxDim || 2 * N > kMaxDim) return fail(MDY_E_SHAPE, "swiglu_bwd: bad shape");
-    if ((M + 7) / 8 > 65535) return fail(MDY_E_SHAPE, "swiglu_bwd: M too large");
     if (M == 0 || N == 0) return 0;
     if (!x || !dy || !dx) return fail(MDY_E_NULL, "swiglu_bwd: null pointer");
     if (x_row_stride < 2 * N) return fail(MDY_E_SHAPE, "swiglu_bwd: x_row_stride < 2N");
@@ -149,7 +144,6 @@ int mdy_swiglu_bwd(const void* x, const void* dy, void* dx, int64_t M, int64_t N
 int mdy_weight_dequant(const void* x, const float* s, void* y, int64_t N, int64_t K, int out_dtype, void* stream) {
     if (out_dtype != MDY_DT_BF16 && out_dtype != MDY_DT_F32) return fail(MDY_E_DTYPE, "weight_dequant: unknown out_dtype %d", out_dtype);
     if (N < 0 || K < 0 || N > kMaxDim || K > kMaxDim) return fail(MDY_E_SHAPE, "weight_dequant: bad shape");
-    if ((N + 15) / 16 > 65535) return fail(MDY_E_SHAPE, "weight_dequant: N too large");
     if (N == 0 || K == 0) return 0;
     if (!x || !s || !y) return fail(MDY_E_NULL, "weight_dequant: null pointer");
     if (!aligned(y, out_dtype == MDY_DT_BF16 ? 2 : 4) || !aligned(s, 4)) return fail(MDY_E_ALIGN, "weight_dequant: misaligned pointer");
@@ -163,7 +157,6 @@ int mdy_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int6
     if (out_dtype != MDY_DT_BF16 && out_dtype != MDY_DT_F32) return fail(MDY_E_DTYPE, "fp8_gemm_nt: unknown out_dtype %d", out_dtype);
     if (M < 0 || N < 0 || K < 1 || M > kMaxDim || N > kMaxDim || K > kMaxDim)
         return fail(MDY_E_SHAPE, "fp8_gemm_nt: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
-    if ((M + 15) / 16 > 65535) return fail(MDY_E_SHAPE, "fp8_gemm_nt: M too large");
     if (M == 0 || N == 0) return 0;
     if (!a || !a_s || !b || !b_s || !c) return fail(MDY_E_NULL, "fp8_gemm_nt: null pointer");
     if (!aligned(c, out_dtype == MDY_DT_BF16 ? 2 : 4) || !aligned(a_s, 4) || !aligned(b_s, 4) || (bias && !aligned(bias, 2)))
@@ -185,7 +178,6 @@ int mdy_fp8_gemm_nt_ws(const void* a, const float* a_s, int64_t as_row_stride, i
     if (out_dtype != MDY_DT_BF16 && out_dtype != MDY_DT_F32) return fail(MDY_E_DTYPE, "fp8_gemm_nt_ws: unknown out_dtype %d", out_dtype);
     if (M < 0 || N < 0 || K < 1 || M > kMaxDim || N > kMaxDim || K > kMaxDim)
         return fail(MDY_E_SHAPE, "fp8_gemm_nt_ws: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
-    if ((M + 15) / 16 > 65535) return fail(MDY_E_SHAPE, "fp8_gemm_nt_ws: M too large");
     if (workspace_bytes < 0) return fail(MDY_E_SHAPE, "fp8_gemm_nt_ws: workspace_bytes < 0");
     if (M == 0 || N == 0) return 0;
     if (!a || !a_s || !b || !b_s || !c) return fail(MDY_E_NULL, "fp8_gemm_nt_ws: null pointer");
@@ -211,7 +203,7 @@ int mdy_fp8_grouped_gemm_nt(const void* a, const float* a_s, int64_t as_row_stri
         if (m_splits[g] < 0 || m_splits[g] > kMaxDim) return fail(MDY_E_SHAPE, "fp8_grouped_gemm_nt: m_splits[%lld]=%lld", (long long)g, (long long)m_splits[g]);
         M += m_splits[g];
     }
-    if (M > kMaxDim || (M + 15) / 16 > 65535 * 16) return fail(MDY_E_SHAPE, "fp8_grouped_gemm_nt: too many rows (%lld)", (long long)M);
+    if (M > kMaxDim) return fail(MDY_E_SHAPE, "fp8_grouped_gemm_nt: too many rows (%lld)", (long long)M);
     if (M == 0) return 0;
     if (!a || !a_s || !b || !b_s || !c) return fail(MDY_E_NULL, "fp8_grouped_gemm_nt: null pointer");
     if (!aligned(c, out_dtype == MDY_DT_BF16 ? 2 : 4) || !aligned(a_s, 4) || !aligned(b_s, 4) || (bias && !aligned(bias, 2)))

@@ -757,7 +757,7 @@ __global__ __launch_bounds__(256) void fp8_gemm_scalar_kernel(const uint8_t* __r
                                                                const float* __restrict__ b_s, OUT* __restrict__ c,
                                                                const uint16_t* __restrict__ bias, int M, int N, int K) {
     const int n = blockIdx.x * 16 + (threadIdx.x & 15);
-    const int m = blockIdx.y * 16 + (threadIdx.x >> 4);
+    const int m = block_row() * 16 + (threadIdx.x >> 4);
     if (m >= M || n >= N) return;
     const int KB = (K + 127) >> 7;
     float acc = 0.0f;
@@ -871,7 +871,8 @@ static int dispatch(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t a
                          ((reinterpret_cast<uintptr_t>(b) & 15) == 0);
     const bool big_ok = mfma_ok && K <= (1 << 16) && as_rs >= 0 && as_cs >= 0 && as_extent < ((int64_t)1 << 31);
     if (!mfma_ok || (M > 64 && !big_ok)) {
-        dim3 grid((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16));
+        dim3 grid;
+        if (!grid_rows((N + 15) / 16, (M + 15) / 16, grid)) return kErrTooManyBlocks;
         hipLaunchKernelGGL((fp8_gemm_scalar_kernel<OUT>), grid, dim3(256), 0, stream, a, a_s, as_rs, as_cs, b, b_s, c,
                            bias, M, N, K);
         return (int)hipGetLastError();

@@ -56,7 +56,8 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
 
     const int t = threadIdx.x;
     const int lane = t & 63, wave = t >> 6;
-    const int bm = blockIdx.y, bk = blockIdx.x;
+    const int bm = block_row(), bk = blockIdx.x;
+    if (bm >= (PM >> 7)) return;
     const int cl = (t & 15) * 8;          // first local column of this thread
     const int rg = t >> 4;                // row group 0..NRG-1
     const int c0 = bk * 128 + cl;
@@ -218,9 +219,10 @@ int launch_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s
                            int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int64_t s_kb_stride,
                            int t_mode, hipStream_t stream) {
     if (PM == 0 || PK == 0) return 0;
-    dim3 grid((unsigned)(PK / 128), (unsigned)(PM / 128));
+    dim3 grid;
+    if (!grid_rows(PK / 128, PM / 128, grid)) return kErrTooManyBlocks;
     // 512 threads (4 rows each) when there are few tiles per CU: more waves to hide the load and store latency
-    const bool wide = grid.x * (long)grid.y < 256 * 24;
+    const bool wide = (PK / 128) * (PM / 128) < 256 * 24;
     dim3 block(wide ? 512 : 256);
     const bool vec = (x_col_stride == 1) && (K % 8 == 0) && (x_row_stride % 8 == 0) &&
                      ((reinterpret_cast<uintptr_t>(x) & 15) == 0);

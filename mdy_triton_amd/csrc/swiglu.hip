@@ -55,7 +55,7 @@ __device__ __forceinline__ uint4 load8_bf16(const uint16_t* p, int col, int N, b
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
-// grid.x = ceil(PN / 512), grid.y = ceil(PM / 8), block = 256.
+// ceil(PN / 512) x ceil(PM / 8) blocks (grid_rows), block = 256.
 // QUANT: write e4m3fn + scales; act may be null.  !QUANT: act only.
 template <int MODE, bool QUANT, bool VEC>
 __global__ __launch_bounds__(256) void swiglu_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ act,
@@ -65,7 +65,7 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const uint16_t* __restrict_
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int col = blockIdx.x * 512 + lane * 8;
-    const int row0 = blockIdx.y * kSgRowsPerBlock + wave * kSgRowsPerWave;
+    const int row0 = block_row() * kSgRowsPerBlock + wave * kSgRowsPerWave;
 
     uint4 ru[kSgRowsPerWave], rg[kSgRowsPerWave];
 #pragma unroll
@@ -135,7 +135,7 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const uint16_t* __restr
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int col = blockIdx.x * 512 + lane * 8;
-    const int row0 = blockIdx.y * kSgRowsPerBlock + wave * kSgRowsPerWave;
+    const int row0 = block_row() * kSgRowsPerBlock + wave * kSgRowsPerWave;
 #pragma unroll
     for (int r = 0; r < kSgRowsPerWave; ++r) {
         const int row = row0 + r;
@@ -181,8 +181,8 @@ int launch_swiglu(const void* x, void* act, void* y, float* s, int64_t M, int64_
     const bool quant = y != nullptr;
     const int64_t rows = quant ? PM : M, cols = quant ? PN : N;
     if (rows == 0 || cols == 0) return 0;
-    dim3 grid((unsigned)((cols + 511) / 512), (unsigned)((rows + kSgRowsPerBlock - 1) / kSgRowsPerBlock));
-    dim3 block(256);
+    dim3 grid, block(256);
+    if (!grid_rows((cols + 511) / 512, (rows + kSgRowsPerBlock - 1) / kSgRowsPerBlock, grid)) return kErrTooManyBlocks;
     const int up_off = gate_first ? (int)N : 0, gate_off = gate_first ? 0 : (int)N;
     const bool vec = (N % 8 == 0) && (x_row_stride % 8 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0) &&
                      (act == nullptr || (reinterpret_cast<uintptr_t>(act) & 15) == 0);
@@ -206,7 +206,8 @@ int launch_swiglu(const void* x, void* act, void* y, float* s, int64_t M, int64_
 int launch_swiglu_bwd(const void* x, const void* dy, void* dx, int64_t M, int64_t N, int64_t x_row_stride,
                       int gate_first, hipStream_t stream) {
     if (M == 0 || N == 0) return 0;
-    dim3 grid((unsigned)((N + 511) / 512), (unsigned)((M + kSgRowsPerBlock - 1) / kSgRowsPerBlock));
+    dim3 grid;
+    if (!grid_rows((N + 511) / 512, (M + kSgRowsPerBlock - 1) / kSgRowsPerBlock, grid)) return kErrTooManyBlocks;
     const int up_off = gate_first ? (int)N : 0, gate_off = gate_first ? 0 : (int)N;
     const bool vec = (N % 8 == 0) && (x_row_stride % 8 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0) &&
                      ((reinterpret_cast<uintptr_t>(dy) & 15) == 0) && ((reinterpret_cast<uintptr_t>(dx) & 15) == 0);

@@ -27,7 +27,7 @@ __global__ __launch_bounds__(256) void weight_dequant_kernel(const uint8_t* __re
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int col = blockIdx.x * kWdCols + lane * 8;
-    const int row0 = (blockIdx.y * kWdWaves + wave) * kWdRows;
+    const int row0 = (block_row() * kWdWaves + wave) * kWdRows;
     if (col >= K) return;
 
     uint2 raw[kWdRows];
@@ -88,8 +88,8 @@ __global__ __launch_bounds__(256) void weight_dequant_kernel(const uint8_t* __re
 int launch_weight_dequant(const void* x, const float* s, void* y, int64_t N, int64_t K, int out_dtype,
                           hipStream_t stream) {
     if (N == 0 || K == 0) return 0;
-    dim3 grid((unsigned)((K + kWdCols - 1) / kWdCols), (unsigned)((N + kWdRows * kWdWaves - 1) / (kWdRows * kWdWaves)));
-    dim3 block(256);
+    dim3 grid, block(256);
+    if (!grid_rows((K + kWdCols - 1) / kWdCols, (N + kWdRows * kWdWaves - 1) / (kWdRows * kWdWaves), grid)) return kErrTooManyBlocks;
     const int sK = (int)((K + kGroup - 1) / kGroup);
     const bool vec = (K % 8 == 0) && ((reinterpret_cast<uintptr_t>(x) & 7) == 0) &&
                      ((reinterpret_cast<uintptr_t>(y) & 15) == 0);

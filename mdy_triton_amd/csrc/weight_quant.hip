@@ -32,8 +32,9 @@ __global__ __launch_bounds__(2048 / RPT) void weight_quant_kernel(const uint16_t
     const int t = threadIdx.x;
     const int lane = t & 63;
     const int wave = t >> 6;
-    const int bn = blockIdx.y;  // block row (along N)
-    const int bk = blockIdx.x;  // block column (along K)
+    const int bn = block_row();  // block row (along N)
+    const int bk = blockIdx.x;   // block column (along K)
+    if (bn >= (PN >> 7)) return;
     const int c0 = bk * 128 + (t & 15) * 8;
     const int rbase = bn * 128 + (t >> 4) * RPT;
 
@@ -142,7 +143,8 @@ int launch_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t,
                         int64_t w_row_stride, int64_t w_col_stride, int64_t PN, int64_t PK, int mode,
                         hipStream_t stream) {
     if (PN == 0 || PK == 0) return 0;
-    dim3 grid((unsigned)(PK / 128), (unsigned)(PN / 128));
+    dim3 grid;
+    if (!grid_rows(PK / 128, PN / 128, grid)) return kErrTooManyBlocks;
     // 512 threads per tile: 4 rows per thread, 56 VGPRs, 8 waves per SIMD (256 threads with 8 rows each need 89
     // VGPRs and measured 1-5 % slower at every size tried)
     dim3 block(512);

@@ -136,3 +136,66 @@ def test_swiglu_beyond_4g_bytes(x_big):
         assert torch.equal(act[r:r + H], acts), r
         assert np.array_equal(u8(y[r:r + H]), u8(ys)) and torch.equal(s[r:r + H], ss), r
         assert torch.equal(dx[r:r + H], m.silu_bwd(dy[r:r + H].contiguous(), xs, "gate-up")), r
+
+
+# ---- more rows than grid.y could hold (65535 blocks): the kernels run on 1-D grids
+def _row_samples(rows, h=64):
+    return [0, rows // 2 // h * h, rows - h]
+
+
+def test_act_quant_and_swiglu_with_a_million_rows():
+    M, K = 8 * 65535 + 4104, 256                            # > 65535 blocks of 8 rows
+    x = big_bf16(M, K, 31)
+    y, s = m.act_quant(x)
+    assert y.shape == (M, K) and s.shape == (M, 2)
+    amax = x.view(M, 2, 128).abs().amax(-1).float().cpu()
+    assert torch.equal(s.cpu(), amax / 448.0)
+    for r in _row_samples(M):
+        yr, sr = O.act_quant(x[r:r + 64].cpu())
+        assert np.array_equal(u8(y[r:r + 64]), u8(yr)) and torch.equal(s[r:r + 64].cpu(), sr), r
+    yq, sq, act = m.silu_act_quant(x, "up-gate", return_act=True)
+    assert torch.equal(act, m.silu_fwd(x, "up-gate"))
+    dx = m.silu_bwd(act, x, "up-gate")
+    for r in _row_samples(M):
+        xs = x[r:r + 64].contiguous()
+        ys, ss, acts = m.silu_act_quant(xs, "up-gate", return_act=True)
+        assert torch.equal(act[r:r + 64], acts), r
+        assert np.array_equal(u8(yq[r:r + 64]), u8(ys)) and torch.equal(sq[r:r + 64], ss), r
+        assert torch.equal(dx[r:r + 64], m.silu_bwd(acts, xs, "up-gate")), r
+
+
+def test_weight_dequant_and_scalar_gemm_with_a_million_rows():
+    N, K = 16 * 65535 + 272, 128                             # > 65535 blocks of 8 (dequant) and of 16 (GEMM) rows
+    g = torch.Generator(device=DEV).manual_seed(41)
+    q = torch.randint(-8, 9, (N, K), device=DEV, generator=g, dtype=torch.int8).float().to(FP8)
+    s = torch.exp2(torch.randint(-2, 3, ((N + 127) // 128, 1), device=DEV, generator=g).float())
+    d = m.weight_dequant(q, s, out_dtype=torch.float32)
+    ref = q.float() * s.repeat_interleave(128, 0)[:N]
+    assert torch.equal(d, ref)
+    # K = 48 is not a multiple of 128: the one-thread-per-element kernel; small integers and power-of-two
+    # scales make every sum exact
+    Kg, Ng = 48, 24
+    a = q[:, :Kg].contiguous()
+    a_s = torch.exp2(torch.randint(-1, 2, (N, 1), device=DEV, generator=g).float())
+    b = torch.randint(-4, 5, (Ng, Kg), device=DEV, generator=g, dtype=torch.int8).float().to(FP8)
+    b_s = torch.full((1, 1), 0.5, device=DEV)
+    c = m.fp8_gemm(a, a_s, b, b_s, out_dtype=torch.float32)
+    ref = (a.float() @ b.float().t()) * a_s * 0.5
+    assert torch.equal(c, ref)
+
+
+def test_training_quantizers_with_more_than_65535_tile_rows():
+    M, K = 128 * 65536, 256                                  # > 65535 tile rows of 128
+    x = big_bf16(M, K, 51)
+    y, s, y_t, s_t = m.quant_grad_output(x)
+    assert y.shape == (M, K) and y_t.shape == (K, M)
+    for r in slabs(M, M // 2):
+        yr, sr, ytr, str_ = O.quant_grad_output(x[r:r + H].cpu())
+        assert np.array_equal(u8(y[r:r + H]), u8(yr)) and torch.equal(s[r:r + H].cpu(), sr), r
+        assert np.array_equal(u8(y_t[:, r:r + H]), u8(ytr)), r
+        assert torch.equal(s_t[:, r // 128:(r + H) // 128].cpu(), str_), r
+    del y, s, y_t, s_t
+    wq, ws = m.weight_quant_block(x)
+    for r in slabs(M, M // 2):
+        yr, sr = O.weight_quant_block(x[r:r + H].cpu())
+        assert np.array_equal(u8(wq[r:r + H]), u8(yr)) and torch.equal(ws[r // 128:(r + H) // 128].cpu(), sr), r
