@@ -55,17 +55,20 @@ __device__ __forceinline__ uint4 load8_bf16(const uint16_t* p, int col, int N, b
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
-// ceil(PN / 512) x ceil(PM / 8) blocks (grid_rows), block = 256.
+// Block = 8 rows x 512 columns, 256 threads; blocks arranged by grid_rows, or (by_xcd, with row-major scales)
+// as grid (8, column chunks, slabs of 8 row blocks) so that all column chunks of a row block run on one XCD and
+// the 16-byte pieces of its scale lines meet in one L2 (see act_quant_kernel).
 // QUANT: write e4m3fn + scales; act may be null.  !QUANT: act only.
 template <int MODE, bool QUANT, bool VEC>
 __global__ __launch_bounds__(256) void swiglu_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ act,
                                                      uint8_t* __restrict__ y, float* __restrict__ s, int M, int N,
                                                      int64_t x_row_stride, int up_off, int gate_off, int PM, int PN,
-                                                     int64_t s_row_stride, int64_t s_col_stride) {
+                                                     int64_t s_row_stride, int64_t s_col_stride, int by_xcd) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int col = blockIdx.x * 512 + lane * 8;
-    const int row0 = block_row() * kSgRowsPerBlock + wave * kSgRowsPerWave;
+    const int col = (by_xcd ? blockIdx.y : blockIdx.x) * 512 + lane * 8;
+    const int row_block = by_xcd ? (int)((blockIdx.z << 3) + blockIdx.x) : block_row();
+    const int row0 = row_block * kSgRowsPerBlock + wave * kSgRowsPerWave;
 
     uint4 ru[kSgRowsPerWave], rg[kSgRowsPerWave];
 #pragma unroll
@@ -181,25 +184,36 @@ int launch_swiglu(const void* x, void* act, void* y, float* s, int64_t M, int64_
     const bool quant = y != nullptr;
     const int64_t rows = quant ? PM : M, cols = quant ? PN : N;
     if (rows == 0 || cols == 0) return 0;
-    dim3 grid, block(256);
-    if (!grid_rows((cols + 511) / 512, (rows + kSgRowsPerBlock - 1) / kSgRowsPerBlock, grid)) return kErrTooManyBlocks;
     const int up_off = gate_first ? (int)N : 0, gate_off = gate_first ? 0 : (int)N;
     const bool vec = (N % 8 == 0) && (x_row_stride % 8 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0) &&
                      (act == nullptr || (reinterpret_cast<uintptr_t>(act) & 15) == 0);
-    const uint16_t* xp = static_cast<const uint16_t*>(x);
-    uint16_t* ap = static_cast<uint16_t*>(act);
-    uint8_t* yp = static_cast<uint8_t*>(y);
+    const int by_xcd = (quant && s_col_stride == 1) ? 1 : 0;    // row-major scales
+    const int64_t chunks = (cols + 511) / 512;
+    if (chunks > 65535) return kErrTooManyBlocks;
+    const int64_t slab_rows = (int64_t)kSgRowsPerBlock * 8;                  // rows per grid.z step
+    const int64_t rows_per_launch = by_xcd ? slab_rows * 65535 : rows;      // grid.z takes 65535 slabs
+    for (int64_t r0 = 0; r0 < rows; r0 += rows_per_launch) {
+        const int64_t n_rows = rows - r0 < rows_per_launch ? rows - r0 : rows_per_launch;
+        const int64_t m = M - r0 < 0 ? 0 : (M - r0 < n_rows ? M - r0 : n_rows);
+        dim3 grid(8, (unsigned)chunks, (unsigned)((n_rows + slab_rows - 1) / slab_rows)), block(256);
+        if (!by_xcd && !grid_rows(chunks, (n_rows + kSgRowsPerBlock - 1) / kSgRowsPerBlock, grid)) return kErrTooManyBlocks;
+        const uint16_t* xp = static_cast<const uint16_t*>(x) + r0 * x_row_stride;
+        uint16_t* ap = act ? static_cast<uint16_t*>(act) + r0 * N : nullptr;
+        uint8_t* yp = quant ? static_cast<uint8_t*>(y) + r0 * PN : nullptr;
+        float* sp = quant ? s + r0 * s_row_stride : nullptr;
+        const int pm = quant ? (int)n_rows : 0;
 #define MDY_SG(MODE, QUANT, VEC)                                                                                     \
-    hipLaunchKernelGGL((swiglu_kernel<MODE, QUANT, VEC>), grid, block, 0, stream, xp, ap, yp, s, (int)M, (int)N,       \
-                       x_row_stride, up_off, gate_off, (int)PM, (int)PN, s_row_stride, s_col_stride)
-    if (!quant) {
-        if (vec) MDY_SG(0, false, true); else MDY_SG(0, false, false);
-    } else if (mode == 0) {
-        if (vec) MDY_SG(0, true, true); else MDY_SG(0, true, false);
-    } else {
-        if (vec) MDY_SG(1, true, true); else MDY_SG(1, true, false);
-    }
+    hipLaunchKernelGGL((swiglu_kernel<MODE, QUANT, VEC>), grid, block, 0, stream, xp, ap, yp, sp, (int)m, (int)N,      \
+                       x_row_stride, up_off, gate_off, pm, (int)PN, s_row_stride, s_col_stride, by_xcd)
+        if (!quant) {
+            if (vec) MDY_SG(0, false, true); else MDY_SG(0, false, false);
+        } else if (mode == 0) {
+            if (vec) MDY_SG(0, true, true); else MDY_SG(0, true, false);
+        } else {
+            if (vec) MDY_SG(1, true, true); else MDY_SG(1, true, false);
+        }
 #undef MDY_SG
+    }
     return (int)hipGetLastError();
 }
 
