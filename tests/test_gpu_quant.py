@@ -158,6 +158,20 @@ def test_quant_input_bit_exact(M, K, seed):
     assert np.array_equal(u8(y), u8(y_ref))
 
 
+@pytest.mark.parametrize("M,K,seed", [(16384, 4096, 8), (8230, 8198, 9), (9001, 7552, 10)])
+def test_quant_input_large_bit_exact(M, K, seed):
+    """From 2^26 padded elements on, the forward quantizer runs 32-row blocks that stage the column-major
+    scales in LDS; ragged M (padded to 4) and K (not a multiple of 8: scalar loads) included."""
+    x = P.activations("outliers", M, K, seed)
+    x[5, 3] = 3e4; x[M - 1, K - 1] = -2e4                                    # saturating groups
+    y_ref, s_ref, _, _ = O.quant_input(x, True)
+    y, s, _, _ = m.quant_input(x.to(DEV), True)
+    assert y.shape == y_ref.shape and s.shape == s_ref.shape and s.stride() == s_ref.stride()
+    assert y.shape[0] * y.shape[1] >= 1 << 26
+    assert torch.equal(s.cpu(), s_ref)
+    assert np.array_equal(u8(y), u8(y_ref))
+
+
 def test_quant_input_strided_rows_and_saturation():
     big = P.activations("normal", 40, 1024, 7)
     x = big[:, 128:128 + 512]                      # row stride 1024, column stride 1, offset 256 bytes
