@@ -342,3 +342,34 @@ def test_add_bias_bit_exact(M, N):
     out = m.add_bias(xd, b.to(DEV))
     assert out.data_ptr() == xd.data_ptr()
     assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
+
+
+# ------------------------------------------------------------------ random ragged shapes, every quantizer
+def test_quantizers_random_shapes():
+    """40 seeded shapes with ragged sides (and, for every fourth, a strided view as the input): every
+    quantizer against the oracle, bytes, scales, shapes and strides."""
+    rng = np.random.default_rng(2024)
+    for case in range(40):
+        M = int(rng.choice([1, 3, 8, 63, 64, 65, 129, 257, 520])) + int(rng.integers(0, 5))
+        K = int(rng.choice([1, 7, 128, 130, 511, 512, 640, 1100])) + int(rng.integers(0, 9))
+        kind = ("normal", "outliers", "heavy")[case % 3]
+        x = P.activations(kind, M, K + 16, case)
+        if case % 5 == 0:
+            x[0, 8] = 3e4                                   # saturates the DeepLinear dialect
+        xd = x.to(DEV)
+        if case % 4 == 0:                                   # row stride K + 16, 16-byte offset
+            x, xd = x[:, 8:8 + K], xd[:, 8:8 + K]
+        else:
+            x, xd = x[:, :K].contiguous(), xd[:, :K].contiguous()
+        tag = (case, M, K)
+        if K % 128 == 0:                                    # the official quantizer wants whole groups
+            y, s = m.act_quant(xd)
+            yr, sr = O.act_quant(x.contiguous())
+            assert np.array_equal(u8(y), u8(yr)) and torch.equal(s.cpu(), sr), tag
+        _same_quant([t for t in m.quant_input(xd, True) if t is not None],
+                    [t for t in O.quant_input(x, True) if t is not None])
+        _same_quant(m.quant_input(xd, False), O.quant_input(x, False))
+        _same_quant(m.quant_grad_output(xd), O.quant_grad_output(x))
+        for only_forward in (True, False):
+            _same_quant([t for t in m.quant_weight(xd, only_forward) if t is not None],
+                        [t for t in O.quant_weight(x, only_forward) if t is not None])
