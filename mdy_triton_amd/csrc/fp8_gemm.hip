@@ -821,14 +821,22 @@ static bool big_tiles_pay(int64_t M, int64_t N) {
 // Tile and ring depth for the shapes that do not take 256x256 tiles:
 //   0: 128x128, 2 K blocks in LDS (two workgroups share a CU)   1: 128x128, 4 K blocks (one workgroup per CU)
 //   2: 128x64, 6 K blocks                                       3: 64x64, 8 K blocks
+//   4: 128x256, 3 K blocks, 8 waves                             5: 256x128, 3 K blocks, 8 waves
 // Measured rule: the smallest tile that still gives every workgroup a CU of its own (the time of these
 // shapes goes with the bytes each CU has to pull, not with its MFMAs), and the ring as deep as LDS allows.
-static int few_tiles_config(int M, int N) {
-    const long rows128 = (M + 127) / 128, rows64 = (M + 63) / 64;
-    const long cols128 = (N + 127) / 128, cols64 = (N + 63) / 64;
+// Between 257 and 512 tiles of 128x128 that is a 128x256 or 256x128 tile (whichever pads less), one per CU,
+// rather than two 128x128 workgroups per CU: 4096x1536x7168 77 -> 70 us, 8192x1024x7168 91 -> 75 us,
+// 1100x6000x16384 178 -> 140 us (K <= 512: 4-6 % slower, so short K keeps the 128x128 tiles).
+static int few_tiles_config(int M, int N, int K) {
+    const long rows128 = (M + 127) / 128, rows64 = (M + 63) / 64, rows256 = (M + 255) / 256;
+    const long cols128 = (N + 127) / 128, cols64 = (N + 63) / 64, cols256 = (N + 255) / 256;
     if (rows64 * cols64 <= kCUs) return 3;
     if (rows128 * cols64 <= kCUs) return 2;
     if (rows128 * cols128 <= kCUs) return 1;
+    if (K < 1024) return 0;    // a handful of K blocks: two short workgroups per CU hide each other's prologue and epilogue
+    const long wide = rows128 * cols256, tall = rows256 * cols128;
+    if (wide <= tall && wide <= kCUs) return 4;
+    if (tall <= kCUs) return 5;
     return 0;
 }
 
@@ -931,10 +939,12 @@ static int dispatch(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t a
     // K blocks in flight, and smaller tiles when even 128x128 tiles leave most CUs idle.
 #define MDY_FEW(BM_, BN_, ST_)                                                                                       \
     return launch_mfma<BM_, BN_, 2, 2, ST_, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream)
-    switch (few_tiles_config(M, N)) {
+    switch (few_tiles_config(M, N, K)) {
         case 1: MDY_FEW(128, 128, 4);
         case 2: MDY_FEW(128, 64, 6);
         case 3: MDY_FEW(64, 64, 8);
+        case 4: return launch_mfma<128, 256, 2, 4, 3, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
+        case 5: return launch_mfma<256, 128, 2, 4, 3, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
         default: MDY_FEW(128, 128, 2);
     }
 #undef MDY_FEW
