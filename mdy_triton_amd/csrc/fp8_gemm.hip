@@ -456,12 +456,12 @@ struct GroupTable {
     int tile_start[kMaxGroups + 1];  // tile rows (of BM) before group g
 };
 
-template <int BM, int BN, int WGM, int WGN, typename OUT>
+template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT>
 __global__ __launch_bounds__(WGM* WGN * 64) void fp8_grouped_gemm_kernel(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
     const uint16_t* __restrict__ bias, int N, int K, int tiles_n, const GroupTable tbl) {
-    __shared__ __attribute__((aligned(1024))) uint8_t pool[TileLds<BM, BN, WGM * WGN, 2>::bytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t pool[TileLds<BM, BN, WGM * WGN, STAGES>::bytes];
     const int G = tbl.n_groups;
     const int pid = xcd_contiguous(blockIdx.x, tbl.tile_start[G] * tiles_n);
     const int trow = pid / tiles_n;               // position in units of whole tile rows
@@ -481,7 +481,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_grouped_gemm_kernel(
     duty.b_sh = __builtin_amdgcn_readfirstlane(duty.b_sh);
     const int KB = K >> 7, NB = (N + 127) >> 7;
     const int r0 = __builtin_amdgcn_readfirstlane(tbl.row_start[g]), r1 = __builtin_amdgcn_readfirstlane(tbl.row_start[g + 1]);
-    fp8_gemm_tile<BM, BN, WGM, WGN, 2, OUT>(a, a_s, as_rs, as_cs, as_bytes, b + (size_t)g * N * K,
+    fp8_gemm_tile<BM, BN, WGM, WGN, STAGES, OUT>(a, a_s, as_rs, as_cs, as_bytes, b + (size_t)g * N * K,
                                          b_s + (size_t)g * NB * KB, c, bias ? bias + (size_t)g * N : nullptr,
                                          __builtin_amdgcn_readfirstlane(r0 + tm * BM), r1,
                                          __builtin_amdgcn_readfirstlane(tbl.row_start[G]), __builtin_amdgcn_readfirstlane(tn * BN), N, K, N,
@@ -1118,7 +1118,8 @@ static int launch_grouped(const uint8_t* a, const float* a_s, int64_t as_rs, int
     if (trow == 0) return 0;
     const int tiles_n = (N + 255) / 256;
     dim3 grid((unsigned)(trow * tiles_n)), block(512);
-    hipLaunchKernelGGL((fp8_grouped_gemm_kernel<BM, 256, 2, 4, OUT>), grid, block, 0, stream, a, a_s, (int)as_rs, (int)as_cs,
+    // the 128-row tile leaves LDS for a ring of 3 K blocks
+    hipLaunchKernelGGL((fp8_grouped_gemm_kernel<BM, 256, 2, 4, (BM == 128 ? 3 : 2), OUT>), grid, block, 0, stream, a, a_s, (int)as_rs, (int)as_cs,
                        as_bytes, b, b_s, c, bias, N, K, tiles_n, tbl);
     return (int)hipGetLastError();
 }
