@@ -456,12 +456,15 @@ struct GroupTable {
     int tile_start[kMaxGroups + 1];  // tile rows (of BM) before group g
 };
 
-template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT>
-__global__ __launch_bounds__(WGM* WGN * 64) void fp8_grouped_gemm_kernel(
+// Tile rows are 256 rows high; a group's last tile row, when it holds at most 128 rows, runs as a 128x256 tile
+// (ring of 3 K blocks in the LDS the 256x256 tile's ring of 2 would take).
+template <typename OUT>
+__global__ __launch_bounds__(512) void fp8_grouped_gemm_kernel(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
     const uint16_t* __restrict__ bias, int N, int K, int tiles_n, const GroupTable tbl) {
-    __shared__ __attribute__((aligned(1024))) uint8_t pool[TileLds<BM, BN, WGM * WGN, STAGES>::bytes];
+    constexpr int kBig = TileLds<256, 256, 8, 2>::bytes, kSmall = TileLds<128, 256, 8, 3>::bytes;
+    __shared__ __attribute__((aligned(1024))) uint8_t pool[kBig > kSmall ? kBig : kSmall];
     const int G = tbl.n_groups;
     const int pid = xcd_contiguous(blockIdx.x, tbl.tile_start[G] * tiles_n);
     const int trow = pid / tiles_n;               // position in units of whole tile rows
@@ -481,11 +484,16 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_grouped_gemm_kernel(
     duty.b_sh = __builtin_amdgcn_readfirstlane(duty.b_sh);
     const int KB = K >> 7, NB = (N + 127) >> 7;
     const int r0 = __builtin_amdgcn_readfirstlane(tbl.row_start[g]), r1 = __builtin_amdgcn_readfirstlane(tbl.row_start[g + 1]);
-    fp8_gemm_tile<BM, BN, WGM, WGN, STAGES, OUT>(a, a_s, as_rs, as_cs, as_bytes, b + (size_t)g * N * K,
-                                         b_s + (size_t)g * NB * KB, c, bias ? bias + (size_t)g * N : nullptr,
-                                         __builtin_amdgcn_readfirstlane(r0 + tm * BM), r1,
-                                         __builtin_amdgcn_readfirstlane(tbl.row_start[G]), __builtin_amdgcn_readfirstlane(tn * BN), N, K, N,
-                                         duty, 0, K >> 7, pool);
+    const int m0 = __builtin_amdgcn_readfirstlane(r0 + tm * 256);
+    const int m_total = __builtin_amdgcn_readfirstlane(tbl.row_start[G]);
+    const int n0 = __builtin_amdgcn_readfirstlane(tn * 256);
+    const uint8_t* bg = b + (size_t)g * N * K;
+    const float* bsg = b_s + (size_t)g * NB * KB;
+    const uint16_t* biasg = bias ? bias + (size_t)g * N : nullptr;
+    if (r1 - m0 <= 128)
+        fp8_gemm_tile<128, 256, 2, 4, 3, OUT>(a, a_s, as_rs, as_cs, as_bytes, bg, bsg, c, biasg, m0, r1, m_total, n0, N, K, N, duty, 0, KB, pool);
+    else
+        fp8_gemm_tile<256, 256, 2, 4, 2, OUT>(a, a_s, as_rs, as_cs, as_bytes, bg, bsg, c, biasg, m0, r1, m_total, n0, N, K, N, duty, 0, KB, pool);
 }
 
 // ---------------------------------------------------------------------------
@@ -1101,7 +1109,7 @@ int launch_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, i
                            (int)N, (int)K, stream);
 }
 
-template <int BM, typename OUT>
+template <typename OUT>
 static int launch_grouped(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, uint32_t as_bytes,
                           const uint8_t* b, const float* b_s, OUT* c, const uint16_t* bias, const int64_t* m_splits,
                           int G, int N, int K, hipStream_t stream) {
@@ -1112,15 +1120,14 @@ static int launch_grouped(const uint8_t* a, const float* a_s, int64_t as_rs, int
         tbl.row_start[g] = row;
         tbl.tile_start[g] = trow;
         row += (int)m_splits[g];
-        trow += ((int)m_splits[g] + BM - 1) / BM;
+        trow += ((int)m_splits[g] + 255) / 256;
     }
     for (int g = G; g <= kMaxGroups; ++g) { tbl.row_start[g] = row; tbl.tile_start[g] = trow; }
     if (trow == 0) return 0;
     const int tiles_n = (N + 255) / 256;
     dim3 grid((unsigned)(trow * tiles_n)), block(512);
-    // the 128-row tile leaves LDS for a ring of 3 K blocks
-    hipLaunchKernelGGL((fp8_grouped_gemm_kernel<BM, 256, 2, 4, (BM == 128 ? 3 : 2), OUT>), grid, block, 0, stream, a, a_s, (int)as_rs, (int)as_cs,
-                       as_bytes, b, b_s, c, bias, N, K, tiles_n, tbl);
+    hipLaunchKernelGGL((fp8_grouped_gemm_kernel<OUT>), grid, block, 0, stream, a, a_s, (int)as_rs, (int)as_cs, as_bytes, b, b_s,
+                       c, bias, N, K, tiles_n, tbl);
     return (int)hipGetLastError();
 }
 
@@ -1134,18 +1141,12 @@ static int dispatch_grouped(const uint8_t* a, const float* a_s, int64_t as_rs, i
                           ((reinterpret_cast<uintptr_t>(b) & 15) == 0) && K <= (1 << 16) && as_rs >= 0 && as_cs >= 0 &&
                           as_extent < ((int64_t)1 << 31) && G <= kMaxGroups;
     if (tiled_ok) {
-        bool all256 = true;
         int64_t max_rows = 0;
-        for (int g = 0; g < G; ++g) {
-            all256 = all256 && (m_splits[g] % 256 == 0);
-            max_rows = m_splits[g] > max_rows ? m_splits[g] : max_rows;
-        }
+        for (int g = 0; g < G; ++g) max_rows = m_splits[g] > max_rows ? m_splits[g] : max_rows;
         if (strip_pays(max_rows, (int64_t)G * ((N + 127) / 128)))
             return launch_strip<OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, m_splits, G, (int)max_rows, N, K,
                                      stream);
-        if (all256)
-            return launch_grouped<256, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, m_splits, G, N, K, stream);
-        return launch_grouped<128, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, m_splits, G, N, K, stream);
+        return launch_grouped<OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, m_splits, G, N, K, stream);
     }
     // any other shape / alignment: one dense call per group
     int64_t row = 0;

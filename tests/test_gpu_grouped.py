@@ -75,7 +75,8 @@ def call_f32(qa, sa, qb, sb, m_splits):
 
 
 @pytest.mark.parametrize("m_splits,N,K", [([256, 512, 0, 256], 520, 384),          # all multiples of 256: 256x256 tiles
-                                          ([100, 0, 1, 300, 129, 128], 776, 256),  # ragged groups: 128x256 tiles, tails everywhere
+                                          ([100, 0, 1, 300, 129, 128], 776, 256),  # ragged groups: 128x256 last tiles, tails everywhere
+                                          ([384, 640, 129, 257, 0, 900, 128, 1], 776, 640),   # 256-row tiles + a 128-row last tile
                                           ([16] * 32, 2048, 512),                  # decode-like: many tiny groups
                                           ([3, 5], 40, 128)])
 def test_grouped_gemm_exact_integer(m_splits, N, K):
