@@ -341,7 +341,10 @@ def table(torch, m, timer, dev):
         m.act_quant(m.silu_fwd(ug))
     line("C4 silu_fwd + act_quant (2 passes) %dx%d" % (Ms, Ns), timer.run(unfused, 20)[0], 9.03125 * Ms * Ns, "GB/s", PEAK_HBM_GBS)
     line("C4 silu_fwd %dx%d" % (Ms, Ns), timer.run(lambda: m.silu_fwd(ug), 20)[0], 6.0 * Ms * Ns, "GB/s", PEAK_HBM_GBS)
-    del ug
+    dact = (torch.randn(Ms, Ns, device=dev)).to(torch.bfloat16)
+    # backward: reads up, gate and dy, writes d_up and d_gate: 10 bytes per activation element
+    line("C4 silu_bwd %dx%d" % (Ms, Ns), timer.run(lambda: m.silu_bwd(dact, ug), 20)[0], 10.0 * Ms * Ns, "GB/s", PEAK_HBM_GBS)
+    del ug, dact
     # grouped (MoE) GEMM: 32 routed experts of the up/gate projection (N = 2 x 2048, K = 7168)
     G, Ng, Kg = 32, 4096, 7168
     bq = torch.randint(0, 120, (G, Ng, Kg), dtype=torch.uint8, device=dev).view(FP8)
@@ -360,6 +363,12 @@ def table(torch, m, timer, dev):
             us = timer.run(lambda: m.fp8_grouped_matmul(aq, asg, bq, bsg, [mg] * G), 10, cold="read")[0]
             line("   the same after a read-only cache flush", us,
                  Mt * Kg + G * Ng * Kg + 2.0 * Mt * Ng + 4.0 * Mt * Kg / 128, "GB/s", PEAK_HBM_GBS)
+    # ragged experts (8 x 1000 rows): 256-row tiles plus one 128-row tile per expert in the same launch
+    Gr, mr = 8, 1000
+    aq = torch.randint(0, 120, (Gr * mr, Kg), dtype=torch.uint8, device=dev).view(FP8)
+    asg = torch.rand(Kg // 128, Gr * mr, device=dev).t()
+    us = timer.run(lambda: m.fp8_grouped_matmul(aq, asg, bq[:Gr], bsg[:Gr], [mr] * Gr), 10)[0]
+    line("grouped fp8_gemm %d experts x %d rows, N=%d K=%d" % (Gr, mr, Ng, Kg), us, 2.0 * Gr * mr * Ng * Kg, "TFLOP/s", PEAK_FP8_TFLOPS)
     del bq, bsg, aq, asg
     for M in (1, 16, 64):
         for (N, K) in ((7168, 2048), (2048, 7168)):
