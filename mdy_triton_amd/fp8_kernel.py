@@ -133,3 +133,92 @@ def weight_quant_block(x: torch.Tensor, BLOCK_M: int = 128, BLOCK_N: int = 128,
         check(lib().mdy_weight_quant(ptr(x), ptr(y), ptr(s), None, None, M, N, x.stride(0), x.stride(1), M, N, 0,
                                      stream_ptr(dev)), "weight_quant_block")
     return y, s
+
+
+class _Fp8MlpCkptOps(torch.autograd.Function):
+    """Memory-saving MLP step (fp8_kernel.py:436-494): the forward keeps only x and the two weights; the
+    backward recomputes the up/gate projection and the activation, then runs the two weight-gradient and
+    the two input-gradient GEMMs on the quantizers' transposed copies."""
+
+    @staticmethod
+    def forward(ctx, x, w_up_gate, w_down, order="up-gate", up_gate_cache=None, down_cache=None):
+        from . import fp8 as L
+        shape = x.shape
+        x2 = x.reshape(-1, shape[-1])
+        M, H = x2.shape
+        N2, inter = w_up_gate.size(0), w_down.size(1)
+        q_x, s_x, _, _ = L.quant_input(x2, only_forward=True)
+        q_wu, s_wu = (up_gate_cache or L.quant_weight(w_up_gate, only_forward=True))[:2]
+        q_wd, s_wd = (down_cache or L.quant_weight(w_down, only_forward=True))[:2]
+        up_gate = L.fp8_matmul(q_x[:M], s_x[:M], q_wu[:N2], s_wu[:L._cdiv(N2, 128)])
+        q_act, s_act = silu_act_quant(up_gate, order, dialect="deeplinear")      # act itself is never written
+        y = L.fp8_matmul(q_act[:M], s_act[:M], q_wd[:w_down.size(0)], s_wd[:L._cdiv(w_down.size(0), 128)])
+        ctx.save_for_backward(x2, w_up_gate, w_down)
+        ctx.order, ctx.shape, ctx.dims = order, shape, (M, H, N2, inter)
+        return y.view(*shape[:-1], w_down.size(0))
+
+    @staticmethod
+    def backward(ctx, dy):
+        from . import fp8 as L
+        x2, w_up_gate, w_down = ctx.saved_tensors
+        M, H, N2, inter = ctx.dims
+        out_f = w_down.size(0)
+        dy2 = dy.reshape(-1, out_f)
+        if dy2.dtype != torch.bfloat16:
+            dy2 = dy2.to(torch.bfloat16)
+        cd = L._cdiv
+        # recompute up_gate and act; the transposed copies feed the weight gradients
+        q_x, s_x, q_xt, s_xt = L.quant_input(x2, only_forward=False)
+        q_wu, s_wu, q_wut, s_wut = L.quant_weight(w_up_gate, only_forward=False)
+        up_gate = L.fp8_matmul(q_x[:M], s_x[:M], q_wu[:N2], s_wu[:cd(N2, 128)])
+        act = silu_fwd(up_gate, ctx.order)
+        _, _, q_actt, s_actt = L.quant_input(act, only_forward=False)
+        _, _, q_wdt, s_wdt = L.quant_weight(w_down, only_forward=False)
+        q_dy, s_dy, q_dyt, s_dyt = L.quant_grad_output(dy2)
+        dact = L.fp8_matmul(q_dy[:M], s_dy[:M], q_wdt[:inter], s_wdt[:cd(inter, 128)])
+        dw_down = L.fp8_matmul(q_dyt[:out_f], s_dyt[:out_f], q_actt[:inter], s_actt[:cd(inter, 128)])
+        dup_gate = silu_bwd(dact, up_gate, ctx.order)
+        q_du, s_du, q_dut, s_dut = L.quant_grad_output(dup_gate)
+        dx = L.fp8_matmul(q_du[:M], s_du[:M], q_wut[:H], s_wut[:cd(H, 128)]).view(ctx.shape)
+        dw_up_gate = L.fp8_matmul(q_dut[:N2], s_dut[:N2], q_xt[:H], s_xt[:cd(H, 128)])
+        return dx, dw_up_gate, dw_down, None, None, None
+
+
+def fp8_ckpt_mlp(x, w_up_gate, w_down, order="up-gate"):
+    return _Fp8MlpCkptOps.apply(x, w_up_gate, w_down, order)
+
+
+class Fp8MLP(torch.nn.Module):
+    """SwiGLU MLP on the FP8 linear path (fp8_kernel.py:500-515): up/gate projection, silu(gate) * up, down
+    projection, both projections block-wise FP8 (`DeepLinear`: e4m3fn, 1x128 activation and 128x128 weight
+    scales), no biases.
+
+    Without gradients the activation goes from the up/gate GEMM to the down GEMM through the fused
+    SwiGLU + quantizer (one pass, the bf16 activation is never written).  With gradients the default is the
+    composition DeepLinear -> triton_silu -> DeepLinear; `low_memory` (attribute or call argument, as in the
+    reference) keeps only the input for the backward pass and recomputes up/gate and the activation there.
+    """
+
+    def __init__(self, hidden_size, intermediate_size, order="up-gate", fp8_dtype=FP8, low_memory=False,
+                 device=None, dtype=torch.bfloat16):
+        super().__init__()
+        if fp8_dtype != FP8:
+            raise TypeError("only torch.float8_e4m3fn is implemented")
+        assert order in _ORDERS, "please indicate the order of input, up-gate or gate-up"
+        from .fp8 import DeepLinear
+        self.up_gate_proj = DeepLinear(hidden_size, intermediate_size * 2, bias=False, device=device, dtype=dtype)
+        self.down_proj = DeepLinear(intermediate_size, hidden_size, bias=False, device=device, dtype=dtype)
+        self.order = order
+        self.fp8_dtype = fp8_dtype
+        self.low_memory = low_memory
+
+    def forward(self, hidden_states, low_memory=False):
+        up, down = self.up_gate_proj, self.down_proj
+        needs_grad = torch.is_grad_enabled() and (hidden_states.requires_grad or up.weight.requires_grad or
+                                                  down.weight.requires_grad)
+        if not needs_grad or low_memory or self.low_memory:
+            # cached quantized weights (re-quantized when a weight changes); the forward needs no transposed copies
+            return _Fp8MlpCkptOps.apply(hidden_states, up.weight, down.weight, self.order,
+                                        up._quantized_weight(False) if up.cache_weight else None,
+                                        down._quantized_weight(False) if down.cache_weight else None)
+        return down(triton_silu(up(hidden_states), self.order))

@@ -112,3 +112,73 @@ def test_swiglu_abi_rejects_bad_arguments():
     assert L.mdy_swiglu_bwd(x.data_ptr(), None, x.data_ptr(), 8, 256, 512, 0, None) == -1
     with pytest.raises(AssertionError):
         m.silu_fwd(x, "gate_up")
+
+
+# ------------------------------------------------------------------ Fp8MLP (fp8_kernel.py:436-515)
+def _within(got, want):
+    g_, w_ = got.float().cpu(), want.float()
+    return bool(((g_ - w_).abs() <= 1e-2 + 1e-2 * w_.abs()).all())
+
+
+@pytest.mark.parametrize("order", ["up-gate", "gate-up"])
+@pytest.mark.parametrize("shape,inter", [((3, 100, 512), 768), ((256, 1024), 1280)])
+def test_fp8_mlp_three_paths(shape, inter, order):
+    """Composition with gradients, the memory-saving op and the gradient-free fused path agree bit for bit
+    with each other (same kernels on the same values).  Against the CPU oracle every stage is held to the
+    GEMM tolerance (rtol = atol = 1e-2) with the oracle fed the device's own bf16 intermediates; the chain
+    as a whole cannot be held to it element by element (a one-ulp difference in up_gate or dact moves a few
+    values across an e4m3fn rounding boundary, a 6 % step in that term of the next GEMM's sums), so end to
+    end the bar is a relative Frobenius error below 0.5 %."""
+    H = shape[-1]
+    g = torch.Generator().manual_seed(inter + H)
+    x = torch.randn(*shape, generator=g).bfloat16()
+    w_ug = (torch.randn(2 * inter, H, generator=g) * 0.03).bfloat16()
+    w_d = (torch.randn(H, inter, generator=g) * 0.03).bfloat16()
+    dy = torch.randn(*shape, generator=g).bfloat16()
+
+    mlp = m.Fp8MLP(H, inter, order=order, device=DEV)
+    up, down = mlp.up_gate_proj, mlp.down_proj
+    with torch.no_grad():
+        up.weight.copy_(w_ug)
+        down.weight.copy_(w_d)
+    results = []
+    for low_memory in (False, True):
+        mlp.zero_grad()
+        xg = x.to(DEV).requires_grad_(True)
+        y = mlp(xg, low_memory=low_memory)
+        y.backward(dy.to(DEV))
+        results.append((y.detach(), xg.grad, up.weight.grad.clone(), down.weight.grad.clone()))
+    for a, b in zip(*results):
+        assert a.shape == b.shape and a.dtype == torch.bfloat16 and torch.equal(a, b)
+    with torch.no_grad():
+        assert torch.equal(mlp(x.to(DEV)), results[0][0])
+    mlp.low_memory = True                                        # the attribute switches the path as well
+    assert torch.equal(mlp(x.to(DEV).requires_grad_(True)), results[0][0])
+    y_d, dx_d, dwug_d, dwd_d = results[0]
+
+    # the same composition by hand, keeping the intermediates
+    mlp.zero_grad()
+    xg = x.to(DEV).requires_grad_(True)
+    ug_d = up(xg)
+    ug_d.retain_grad()
+    act_d = m.triton_silu(ug_d, order)
+    act_d.retain_grad()
+    y2 = down(act_d)
+    y2.backward(dy.to(DEV))
+    assert torch.equal(y2, y_d) and torch.equal(xg.grad, dx_d)
+    ug_c, act_c = ug_d.detach().cpu(), act_d.detach().cpu()
+    # stage by stage
+    assert _within(ug_d, O.deep_linear_forward(x, w_ug, None))
+    assert _within(y_d, O.deep_linear_forward(act_c, w_d, None))
+    dact_r, dwd_r, _ = O.deep_linear_backward(act_c, w_d, dy, False)
+    assert _within(act_d.grad, dact_r) and _within(dwd_d, dwd_r)
+    dx_r, dwug_r, _ = O.deep_linear_backward(x, w_ug, ug_d.grad.cpu(), False)
+    assert _within(dx_d, dx_r) and _within(dwug_d, dwug_r)
+    # end to end
+    up_gate = O.deep_linear_forward(x, w_ug, None)
+    act = O.silu_fwd(up_gate, order)
+    dact, dw_d_ref, _ = O.deep_linear_backward(act, w_d, dy, False)
+    dx_ref, dw_ug_ref, _ = O.deep_linear_backward(x, w_ug, O.silu_bwd(dact, up_gate, order), False)
+    for got, want in zip(results[0], (O.deep_linear_forward(act, w_d, None), dx_ref, dw_ug_ref, dw_d_ref)):
+        assert got.shape == want.shape
+        assert (got.float().cpu() - want.float()).norm() < 5e-3 * want.float().norm()
