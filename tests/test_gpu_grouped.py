@@ -196,3 +196,37 @@ def test_grouped_abi_rejects_bad_arguments():
     assert L.mdy_fp8_grouped_gemm_nt(*args(ok, c=c.data_ptr() + 1)) == -3
     with pytest.raises(ValueError):
         m.fp8_grouped_matmul(a.view(FP8), s, b.view(FP8), bs, [100, 100])
+
+
+def test_custom_manger_funnel_and_weight_cache():
+    """CustomManger (megatron_patchs/manger.py): the classmethods are the package's operators, and
+    get_fp8_weight re-quantizes a parameter only after set_first_micro_batch(p, True)."""
+    from mdy_triton_amd.megatron_patchs.manger import CustomManger as CM
+    g = torch.Generator().manual_seed(3)
+    w = torch.nn.Parameter((torch.randn(256, 512, generator=g) * 0.02).bfloat16().to(DEV))
+    CM.clear()
+    first = CM.get_fp8_weight(w)
+    ref = m.per_block_cast_to_fp8(w.detach(), output_transpose=True)
+    assert len(first) == 4 and all(torch.equal(a.view(torch.uint8) if a.dtype == FP8 else a,
+                                               b.view(torch.uint8) if b.dtype == FP8 else b) for a, b in zip(first, ref))
+    with torch.no_grad():
+        w.mul_(2)
+    assert CM.get_fp8_weight(w)[0].data_ptr() == first[0].data_ptr()          # not marked: the cached copies
+    CM.set_first_micro_batch(w, True)
+    again = CM.get_fp8_weight(w)
+    ref2 = m.per_block_cast_to_fp8(w.detach(), output_transpose=True)                  # re-quantized from the new weight ...
+    assert torch.equal(again[1], ref2[1]) and torch.equal(again[0].view(torch.uint8), ref2[0].view(torch.uint8))
+    assert CM.get_fp8_weight(w)[0].data_ptr() == again[0].data_ptr()          # ... and are cached again
+    # a list of expert weights is keyed by its first member
+    experts = [torch.nn.Parameter((torch.randn(256, 256, generator=g) * 0.02).bfloat16().to(DEV)) for _ in range(3)]
+    qe = CM.get_fp8_weight(experts)
+    assert qe[0].shape == (3, 256, 256) and experts[0] in CM.fp8_weight_map
+    # the funnel
+    x = torch.randn(64, 512, generator=g).bfloat16().to(DEV)
+    qx, sx, _, _ = CM.per_token_cast_to_fp8(x)
+    out = CM.fp8_matmul(qx[:64], sx[:64], again[0][:256], again[1][:2])
+    assert torch.equal(out, m.fp8_matmul(qx[:64], sx[:64], again[0][:256], again[1][:2]))
+    t = torch.arange(12, device=DEV).reshape(3, 4).t()                         # non-contiguous rows
+    assert CM.fix_tensor_shape(t, 2).is_contiguous() and CM.fix_tensor_shape(t, 2).shape == (2, 3)
+    CM.clear()
+    assert not CM.fp8_weight_map
