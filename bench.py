@@ -22,6 +22,8 @@ Prints ONE JSON line on stdout:
                and per launch of several back-to-back launches on uncached buffers (us_streamed)
   cpu_baseline the CPU oracle (dequantize + fp32 matmul, torch CPU ops) on a bounded
                sample of the same workload, on the host cores of this box
+Before the W warm-up steps the script runs the same step for 50 ms (set-up, untimed): after an idle period the
+GPU needs some 20 ms of work to reach its sustained clock, whatever W is.
 With --table a per-kernel table for every benchmark configuration goes to stderr.
 """
 import argparse
@@ -211,6 +213,13 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    # set-up, not part of the measurement: bring the GPU out of its idle power state (the first ~20 ms of work
+    # after an idle period run at a fraction of the sustained clock, whatever --warmup says)
+    t_ramp = time.perf_counter()
+    while time.perf_counter() - t_ramp < 0.05:
+        step()
+        torch.cuda.synchronize()
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -291,6 +300,11 @@ def main():
         },
         "parity_spot_check": parity_ok,
     }
+    # the same peak derived from the device the run is on: CUs x 4 SIMDs x 2048 FP8 flop per clock x max clock
+    props = torch.cuda.get_device_properties(dev)
+    clock_khz = getattr(props, "clock_rate", 0) or 2400000      # MI355X: 2.4 GHz peak engine clock
+    result["roofline"]["peak_from_device_props"] = round(props.multi_processor_count * 4 * 2048 * clock_khz * 1e3 / 1e12, 1)
+    result["roofline"]["device"] = "%s, %d CUs, %.2f GHz" % (props.name, props.multi_processor_count, clock_khz / 1e6)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch, kind, M, N, K, xq, xs, wq, ws)
 
