@@ -230,3 +230,18 @@ def test_custom_manger_funnel_and_weight_cache():
     assert CM.fix_tensor_shape(t, 2).is_contiguous() and CM.fix_tensor_shape(t, 2).shape == (2, 3)
     CM.clear()
     assert not CM.fp8_weight_map
+
+
+def test_grouped_gemm_exact_integer_random_splits():
+    """Twelve seeded group tables (empty, tiny, ragged and 256-aligned experts mixed) against the exact integer
+    reference: every expert starts a new tile row, its last tile row may be the 128-row kind, and no row of
+    one expert may see another expert's weight."""
+    rng = np.random.default_rng(77)
+    for case in range(12):
+        G = int(rng.integers(1, 9))
+        m_splits = [int(rng.choice([0, 1, 17, 100, 128, 129, 200, 256, 257, 300, 384, 385, 512, 700])) for _ in range(G)]
+        if sum(m_splits) == 0:
+            m_splits[0] = 130
+        N = int(rng.choice([128, 200, 256, 520, 776, 1024]))
+        K = 128 * int(rng.integers(1, 6))
+        exact_grouped_case(m_splits, N, K, 1000 + case, call_f32)
