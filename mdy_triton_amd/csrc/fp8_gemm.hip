@@ -832,7 +832,7 @@ static bool big_tiles_pay(int64_t M, int64_t N) {
 //   4: 128x256, 3 K blocks, 8 waves                             5: 256x128, 3 K blocks, 8 waves
 // Measured rule: the smallest tile that still gives every workgroup a CU of its own (the time of these
 // shapes goes with the bytes each CU has to pull, not with its MFMAs), and the ring as deep as LDS allows.
-// Between 257 and 512 tiles of 128x128 that is a 128x256 or 256x128 tile (whichever pads less), one per CU,
+// Between 257 and 512 tiles of 128x128 that is a 128x256 tile (else, if those are too many, 256x128), one per CU,
 // rather than two 128x128 workgroups per CU: 4096x1536x7168 77 -> 70 us, 8192x1024x7168 91 -> 75 us,
 // 1100x6000x16384 178 -> 140 us (K <= 512: 4-6 % slower, so short K keeps the 128x128 tiles).
 static int few_tiles_config(int M, int N, int K) {
@@ -843,7 +843,7 @@ static int few_tiles_config(int M, int N, int K) {
     if (rows128 * cols128 <= kCUs) return 1;
     if (K < 1024) return 0;    // a handful of K blocks: two short workgroups per CU hide each other's prologue and epilogue
     const long wide = rows128 * cols256, tall = rows256 * cols128;
-    if (wide <= tall && wide <= kCUs) return 4;
+    if (wide <= kCUs) return 4;    // also when it pads more than the tall tile: 12800x384x7168 82 against 95 us
     if (tall <= kCUs) return 5;
     return 0;
 }
