@@ -66,6 +66,43 @@ def test_argument_validation_without_device(lib):
     assert lib.mdy_add_bias(p, p, 0, 16, None) == 0
 
 
+def test_argument_validation_of_the_later_entry_points(lib):
+    buf = ctypes.create_string_buffer(8192)
+    p = (ctypes.addressof(buf) + 255) // 256 * 256
+    # GEMM with a workspace: negative size, misaligned buffer, empty problem, workspace query of a bad shape
+    assert lib.mdy_fp8_gemm_nt_ws(p, p, 1, 1, p, p, p, None, 4, 4, 128, 0, p, -1, None) == -2
+    assert lib.mdy_fp8_gemm_nt_ws(p, p, 1, 1, p, p, p, None, 4, 4, 128, 0, p + 4, 64, None) == -3
+    assert lib.mdy_fp8_gemm_nt_ws(p, p, 1, 1, p, p, p, None, 0, 4, 128, 0, None, 0, None) == 0
+    assert lib.mdy_fp8_gemm_nt_ws(p, p, 1, 1, p, p, p, None, 4, 4, 128, 5, None, 0, None) == -4
+    assert lib.mdy_fp8_gemm_workspace_bytes(-1, 4, 128) == 0 and lib.mdy_fp8_gemm_workspace_bytes(4, 4, 0) == 0
+    assert lib.mdy_fp8_gemm_workspace_bytes(128, 1536, 4096) >= 2 * 128 * 1536 * 4      # split along K
+    assert lib.mdy_fp8_gemm_workspace_bytes(1, 7168, 2048) == 0                          # decode: never
+    # grouped GEMM: no group table, a negative group, too many groups, nothing to do
+    splits = (ctypes.c_int64 * 3)(4, -1, 4)
+    assert lib.mdy_fp8_grouped_gemm_nt(p, p, 1, 1, p, p, p, None, None, 3, 4, 128, 0, None) == -1
+    assert lib.mdy_fp8_grouped_gemm_nt(p, p, 1, 1, p, p, p, None, splits, 3, 4, 128, 0, None) == -2
+    assert lib.mdy_fp8_grouped_gemm_nt(p, p, 1, 1, p, p, p, None, splits, (1 << 20) + 1, 4, 128, 0, None) == -2
+    zero = (ctypes.c_int64 * 2)(0, 0)
+    assert lib.mdy_fp8_grouped_gemm_nt(p, p, 1, 1, p, p, p, None, zero, 2, 4, 128, 0, None) == 0
+    assert lib.mdy_fp8_grouped_gemm_nt(None, None, 1, 1, None, None, None, None, None, 0, 4, 128, 0, None) == 0
+    # training quantizer: unknown transposed-scale mode, unpadded sizes, scale stride shorter than the rows
+    assert lib.mdy_quant_transpose(p, p, p, p, p, 128, 128, 128, 1, 128, 128, 128, 7, None) == -4
+    assert lib.mdy_quant_transpose(p, p, p, p, p, 100, 128, 128, 1, 100, 128, 128, 0, None) == -2
+    assert lib.mdy_quant_transpose(p, p, p, p, p, 128, 128, 128, 1, 128, 128, 64, 0, None) == -2
+    assert lib.mdy_quant_transpose(p, p, p, None, p, 128, 128, 128, 1, 128, 128, 128, 0, None) == -1
+    # SwiGLU: nothing to write, quantized output without scales, row stride shorter than the row
+    assert lib.mdy_swiglu(p, None, None, None, 4, 128, 256, 0, 4, 128, 1, 1, 0, None) == -1
+    assert lib.mdy_swiglu(p, None, p, None, 4, 128, 256, 0, 4, 128, 1, 1, 0, None) == -1
+    assert lib.mdy_swiglu(p, p, None, None, 4, 128, 200, 0, 0, 0, 1, 1, 0, None) == -2
+    assert lib.mdy_swiglu(p, None, p, p, 4, 128, 256, 0, 4, 100, 1, 1, 0, None) == -2
+    assert lib.mdy_swiglu(p, p, None, None, 0, 128, 256, 0, 0, 0, 1, 1, 0, None) == 0
+    # diagnostics
+    assert lib.mdy_quotient_selfcheck(None, 0, 16, 0, None) == -1
+    assert lib.mdy_quotient_selfcheck(p, 16, 8, 0, None) == -2
+    assert lib.mdy_cast_f32_to_e4m3(p, p, -1, 0, None) == -2 and lib.mdy_cast_f32_to_e4m3(None, None, 0, 0, None) == 0
+    assert lib.mdy_fp8_last_error()            # the last message is kept
+
+
 def test_python_wrappers_keep_reference_preconditions():
     import mdy_triton_amd as m
     x = torch.zeros(4, 130, dtype=torch.bfloat16)
