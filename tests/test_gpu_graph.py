@@ -88,3 +88,42 @@ def test_training_quantizers_and_split_gemm_replay():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, eager2), rep
+
+
+def test_calls_from_several_threads_and_streams_do_not_interfere():
+    """The library keeps no mutable state between calls: four host threads, each on its own stream, run
+    different operators on their own tensors at the same time (ctypes releases the GIL during a call) and
+    every result equals the one computed alone."""
+    import threading
+    torch.manual_seed(5)
+    jobs = []
+    for i, (M, N, K) in enumerate([(64, 512, 1024), (300, 384, 512), (1, 2048, 2048), (130, 1100, 4224)]):
+        x = bf16(M, K, 100 + i)
+        w_q, w_s = m.quant_weight(bf16(N, K, 200 + i, 0.05))[:2]
+
+        def job(x=x, w_q=w_q, w_s=w_s, M=M, N=N):
+            q, s, _, _ = m.quant_input(x)
+            return m.fp8_matmul(q[:M], s[:M], w_q[:N], w_s[:(N + 127) // 128])
+        jobs.append(job)
+    alone = [j().clone() for j in jobs]
+    torch.cuda.synchronize()
+    results, errors = [None] * len(jobs), []
+
+    def worker(i):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for _ in range(25):
+                    out = jobs[i]()
+                stream.synchronize()
+            results[i] = out
+        except Exception as e:        # surfaces in the main thread below
+            errors.append(e)
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(len(jobs))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for got, want in zip(results, alone):
+        assert torch.equal(got, want)
