@@ -66,6 +66,33 @@ __device__ __forceinline__ uint2 quantize8(const float (&f)[8], float amax, floa
     return out;
 }
 
+// 8 bf16 of row `row` from column `col` on, zeros outside the M x K matrix
+template <bool VEC>
+__device__ __forceinline__ uint4 load8(const uint16_t* __restrict__ x, int row, int col, int M, int K, int64_t x_row_stride) {
+    if (row >= M || col >= K) return make_uint4(0u, 0u, 0u, 0u);
+    const uint16_t* p = x + (int64_t)row * x_row_stride + col;
+    if (VEC) return load_nt16(p);  // K % 8 == 0: all 8 columns in range
+    uint32_t w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        if (col + i < K) w[i >> 1] |= (uint32_t)p[i] << ((i & 1) * 16);
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// the lane's 8 values as fp32 and the absmax of its 128-element group (16 lanes)
+__device__ __forceinline__ float unpack8_group_max(const uint4& raw, float (&f)[8]) {
+    f[0] = bf16_lo(raw.x); f[1] = bf16_hi(raw.x);
+    f[2] = bf16_lo(raw.y); f[3] = bf16_hi(raw.y);
+    f[4] = bf16_lo(raw.z); f[5] = bf16_hi(raw.z);
+    f[6] = bf16_lo(raw.w); f[7] = bf16_hi(raw.w);
+    float m = 0.0f;
+    m = fmaxf(fmaxf(fabsf(f[0]), fabsf(f[1])), m);
+    m = fmaxf(fmaxf(fabsf(f[2]), fabsf(f[3])), m);
+    m = fmaxf(fmaxf(fabsf(f[4]), fabsf(f[5])), m);
+    m = fmaxf(fmaxf(fabsf(f[6]), fabsf(f[7])), m);
+    return row16_max(m);
+}
+
 // Block = 8 rows x 512 columns, 256 threads.  Two block arrangements:
 //   by_xcd = 0: grid_rows(column chunks, row blocks);
 //   by_xcd = 1: grid (8, column chunks, slabs of 8 row blocks).  Consecutive workgroup ids go to consecutive
@@ -91,35 +118,14 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restri
 #pragma unroll
     for (int r = 0; r < kAqRowsPerWave; ++r) {
         const int row = row0 + r;
-        raw[r] = make_uint4(0u, 0u, 0u, 0u);
-        if (row < M && col < K) {
-            const uint16_t* p = x + (int64_t)row * x_row_stride + col;
-            if (VEC) {
-                raw[r] = load_nt16(p);  // K % 8 == 0: all 8 columns in range
-            } else {
-                uint32_t w[4] = {0u, 0u, 0u, 0u};
-#pragma unroll
-                for (int i = 0; i < 8; ++i)
-                    if (col + i < K) w[i >> 1] |= (uint32_t)p[i] << ((i & 1) * 16);
-                raw[r] = make_uint4(w[0], w[1], w[2], w[3]);
-            }
-        }
+        raw[r] = load8<VEC>(x, row, col, M, K, x_row_stride);
     }
 
 #pragma unroll
     for (int r = 0; r < kAqRowsPerWave; ++r) {
         const int row = row0 + r;
         float f[8];
-        f[0] = bf16_lo(raw[r].x); f[1] = bf16_hi(raw[r].x);
-        f[2] = bf16_lo(raw[r].y); f[3] = bf16_hi(raw[r].y);
-        f[4] = bf16_lo(raw[r].z); f[5] = bf16_hi(raw[r].z);
-        f[6] = bf16_lo(raw[r].w); f[7] = bf16_hi(raw[r].w);
-        float m = 0.0f;
-        m = fmaxf(fmaxf(fabsf(f[0]), fabsf(f[1])), m);
-        m = fmaxf(fmaxf(fabsf(f[2]), fabsf(f[3])), m);
-        m = fmaxf(fmaxf(fabsf(f[4]), fabsf(f[5])), m);
-        m = fmaxf(fmaxf(fabsf(f[6]), fabsf(f[7])), m);
-        const float amax = row16_max(m);
+        const float amax = unpack8_group_max(raw[r], f);
         float scale;
         const uint2 packed = quantize8<MODE>(f, amax, scale);
         if (row < PM && col_in_out) {
@@ -148,34 +154,13 @@ __global__ __launch_bounds__(512) void act_quant_cm_kernel(const uint16_t* __res
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const int row = row0 + r;
-        raw[r] = make_uint4(0u, 0u, 0u, 0u);
-        if (row < M && col < K) {
-            const uint16_t* p = x + (int64_t)row * x_row_stride + col;
-            if (VEC) {
-                raw[r] = load_nt16(p);
-            } else {
-                uint32_t w[4] = {0u, 0u, 0u, 0u};
-#pragma unroll
-                for (int i = 0; i < 8; ++i)
-                    if (col + i < K) w[i >> 1] |= (uint32_t)p[i] << ((i & 1) * 16);
-                raw[r] = make_uint4(w[0], w[1], w[2], w[3]);
-            }
-        }
+        raw[r] = load8<VEC>(x, row, col, M, K, x_row_stride);
     }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const int row = row0 + r;
         float f[8];
-        f[0] = bf16_lo(raw[r].x); f[1] = bf16_hi(raw[r].x);
-        f[2] = bf16_lo(raw[r].y); f[3] = bf16_hi(raw[r].y);
-        f[4] = bf16_lo(raw[r].z); f[5] = bf16_hi(raw[r].z);
-        f[6] = bf16_lo(raw[r].w); f[7] = bf16_hi(raw[r].w);
-        float m = 0.0f;
-        m = fmaxf(fmaxf(fabsf(f[0]), fabsf(f[1])), m);
-        m = fmaxf(fmaxf(fabsf(f[2]), fabsf(f[3])), m);
-        m = fmaxf(fmaxf(fabsf(f[4]), fabsf(f[5])), m);
-        m = fmaxf(fmaxf(fabsf(f[6]), fabsf(f[7])), m);
-        const float amax = row16_max(m);
+        const float amax = unpack8_group_max(raw[r], f);
         float scale;
         const uint2 packed = quantize8<MODE>(f, amax, scale);
         if (row < PM && col_in_out) store_nt8(y + (int64_t)row * PK + col, packed);
