@@ -19,11 +19,12 @@
 
 namespace mdy {
 
-template <int MODE, bool VEC, int RPT>
-__global__ __launch_bounds__(2048 / RPT) void weight_quant_kernel(const uint16_t* __restrict__ w, uint8_t* __restrict__ y,
+template <int MODE, bool VEC>
+__global__ __launch_bounds__(512) void weight_quant_kernel(const uint16_t* __restrict__ w, uint8_t* __restrict__ y,
                                                             float* __restrict__ s, uint8_t* __restrict__ y_t,
                                                             float* __restrict__ s_t, int N, int K, int64_t w_row_stride,
                                                             int64_t w_col_stride, int PN, int PK) {
+    constexpr int RPT = 4;             // rows per thread
     constexpr int NRG = 128 / RPT;     // row groups of RPT consecutive rows, 16 threads (8 columns each) per group
     constexpr int WAVES = NRG / 4;
     __shared__ float wave_max[WAVES];
@@ -107,25 +108,13 @@ __global__ __launch_bounds__(2048 / RPT) void weight_quant_kernel(const uint16_t
     if (y_t) {
         // column j of the thread's RPT x 8 bytes = RPT consecutive bytes of row (t%16)*8 + j of the transposed tile
         const int cl = (t & 15) * 8, rg = t >> 4;
-        if (RPT == 8) {
-            uint32_t tb[8][2];   // [column j][rows 0..3 | 4..7]
-            uint32_t lo8[8], hi8[8];
+        uint32_t c_lo[4], c_hi[4];
+        transpose4x4_bytes(qlo, c_lo);
+        transpose4x4_bytes(qhi, c_hi);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) { lo8[i] = qlo[i % RPT]; hi8[i] = qhi[i % RPT]; }
-            transpose8x8_bytes(lo8, hi8, tb);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) *reinterpret_cast<uint2*>(&tile[cl + j][rg * 8]) = make_uint2(tb[j][0], tb[j][1]);
-        } else {
-            const uint32_t rl[4] = {qlo[0], qlo[1 % RPT], qlo[2 % RPT], qlo[3 % RPT]};
-            const uint32_t rh[4] = {qhi[0], qhi[1 % RPT], qhi[2 % RPT], qhi[3 % RPT]};
-            uint32_t c_lo[4], c_hi[4];
-            transpose4x4_bytes(rl, c_lo);
-            transpose4x4_bytes(rh, c_hi);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                *reinterpret_cast<uint32_t*>(&tile[cl + j][rg * 4]) = c_lo[j];
-                *reinterpret_cast<uint32_t*>(&tile[cl + 4 + j][rg * 4]) = c_hi[j];
-            }
+        for (int j = 0; j < 4; ++j) {
+            *reinterpret_cast<uint32_t*>(&tile[cl + j][rg * 4]) = c_lo[j];
+            *reinterpret_cast<uint32_t*>(&tile[cl + 4 + j][rg * 4]) = c_hi[j];
         }
         __syncthreads();
         // y_t[k][n]: thread owns output columns (t%16)*8..+7 (n) of output rows t/16 + NRG*i (k)
@@ -154,7 +143,7 @@ int launch_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t,
     uint8_t* yp = static_cast<uint8_t*>(y);
     uint8_t* ytp = static_cast<uint8_t*>(y_t);
 #define MDY_WQ(MODE, VEC)                                                                                          \
-    hipLaunchKernelGGL((weight_quant_kernel<MODE, VEC, 4>), grid, block, 0, stream, wp, yp, s, ytp, s_t, (int)N, \
+    hipLaunchKernelGGL((weight_quant_kernel<MODE, VEC>), grid, block, 0, stream, wp, yp, s, ytp, s_t, (int)N, \
                        (int)K, w_row_stride, w_col_stride, (int)PN, (int)PK)
     if (mode == 0) {
         if (vec) MDY_WQ(0, true); else MDY_WQ(0, false);
