@@ -28,17 +28,6 @@ constexpr int kAqRowsPerWave = 2;
 constexpr int kAqWaves = 4;
 constexpr int kAqRowsPerBlock = kAqRowsPerWave * kAqWaves;  // 8 rows x 512 columns per block
 
-__device__ __forceinline__ float row16_max(float v) {
-    // butterfly over the 16 lanes of a DPP row: xor 1, xor 2 (quad_perm), then
-    // row_half_mirror (lane -> 7-lane inside each 8) and row_mirror (lane -> 15-lane)
-    int i = __float_as_int(v);
-    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0xB1, 0xF, 0xF, true))));   // quad_perm [1,0,3,2]
-    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0x4E, 0xF, 0xF, true))));   // quad_perm [2,3,0,1]
-    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0x141, 0xF, 0xF, true))));  // row_half_mirror
-    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0x140, 0xF, 0xF, true))));  // row_mirror
-    return __int_as_float(i);
-}
-
 template <int MODE>
 __device__ __forceinline__ uint2 quantize8(const float (&f)[8], float amax, float& scale_out) {
     float s = group_scale<MODE>(amax);

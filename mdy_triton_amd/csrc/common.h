@@ -95,6 +95,18 @@ __device__ __forceinline__ void transpose8x8_bytes(const uint32_t (&lo)[8], cons
     }
 }
 
+// max over the 16 lanes of a DPP row (one 128-element quantization group: 16 lanes x 8 values)
+__device__ __forceinline__ float row16_max(float v) {
+    // butterfly over the 16 lanes of a DPP row: xor 1, xor 2 (quad_perm), then
+    // row_half_mirror (lane -> 7-lane inside each 8) and row_mirror (lane -> 15-lane)
+    int i = __float_as_int(v);
+    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0xB1, 0xF, 0xF, true))));   // quad_perm [1,0,3,2]
+    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0x4E, 0xF, 0xF, true))));   // quad_perm [2,3,0,1]
+    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0x141, 0xF, 0xF, true))));  // row_half_mirror
+    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0x140, 0xF, 0xF, true))));  // row_mirror
+    return __int_as_float(i);
+}
+
 // Streaming (non-temporal) vector accesses: the quantizers and the dequantizer touch every
 // byte exactly once, so they bypass cache allocation; measured 1.25-1.5x over plain accesses.
 typedef unsigned uintx4_t __attribute__((ext_vector_type(4)));

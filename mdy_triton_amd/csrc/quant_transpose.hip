@@ -21,15 +21,6 @@
 
 namespace mdy {
 
-__device__ __forceinline__ float qt_row16_max(float v) {
-    int i = __float_as_int(v);
-    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0xB1, 0xF, 0xF, true))));
-    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0x4E, 0xF, 0xF, true))));
-    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0x141, 0xF, 0xF, true))));
-    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0x140, 0xF, 0xF, true))));
-    return __int_as_float(i);
-}
-
 // x / s in the DeepLinear dialect.  FAST (amax <= 1e4, so |x/s| <= 448 needs no clamp) uses the
 // reciprocal form; otherwise an IEEE division saturated at +-448 (NaN kept).
 template <bool FAST>
@@ -92,7 +83,7 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
             cmax[2 * j] = fmaxf(cmax[2 * j], fabsf(f[i][2 * j]));
             cmax[2 * j + 1] = fmaxf(cmax[2 * j + 1], fabsf(f[i][2 * j + 1]));
         }
-        rmax[i] = qt_row16_max(m);
+        rmax[i] = row16_max(m);
     }
 
     // ---- (1) row-wise quantization straight from registers

@@ -26,15 +26,6 @@ constexpr int kSgRowsPerWave = 2;
 constexpr int kSgWaves = 4;
 constexpr int kSgRowsPerBlock = kSgRowsPerWave * kSgWaves;
 
-__device__ __forceinline__ float sg_row16_max(float v) {
-    int i = __float_as_int(v);
-    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0xB1, 0xF, 0xF, true))));
-    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0x4E, 0xF, 0xF, true))));
-    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0x141, 0xF, 0xF, true))));
-    i = __float_as_int(fmaxf(__int_as_float(i), __int_as_float(__builtin_amdgcn_mov_dpp(i, 0x140, 0xF, 0xF, true))));
-    return __int_as_float(i);
-}
-
 __device__ __forceinline__ float sg_sigmoid(float g) {
     // 2^(-g * log2(e)); for g << 0 the exponential overflows to +inf and the reciprocal gives 0
     const float e = __builtin_amdgcn_exp2f(-1.44269504088896340736f * g);
@@ -110,7 +101,7 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const uint16_t* __restrict_
             float m = 0.0f;
 #pragma unroll
             for (int i = 0; i < 8; i += 2) m = fmaxf(fmaxf(fabsf(f[i]), fabsf(f[i + 1])), m);
-            const float amax = sg_row16_max(m);
+            const float amax = row16_max(m);
             const float sc = group_scale<MODE>(amax);
             const bool fast = MODE == 0 ? fast_quotient_ok<0>(amax) : (amax <= 1e4f);
             float q[8];
