@@ -28,33 +28,6 @@ constexpr int kAqRowsPerWave = 2;
 constexpr int kAqWaves = 4;
 constexpr int kAqRowsPerBlock = kAqRowsPerWave * kAqWaves;  // 8 rows x 512 columns per block
 
-template <int MODE>
-__device__ __forceinline__ uint2 quantize8(const float (&f)[8], float amax, float& scale_out) {
-    float s = group_scale<MODE>(amax);
-    scale_out = s;
-    float q[8];
-    bool fast = MODE == 0 ? fast_quotient_ok<0>(amax) : (amax <= 1e4f);
-    if (fast) {
-        float r = 1.0f / s;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) q[i] = fast_quotient(f[i], s, r);
-    } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            float v = f[i] / s;
-            if (MODE != 0) {
-                float c = __builtin_amdgcn_fmed3f(v, -kFp8Max, kFp8Max);
-                v = (v != v) ? v : c;
-            }
-            q[i] = v;
-        }
-    }
-    uint2 out;
-    out.x = pack4_e4m3(q[0], q[1], q[2], q[3]);
-    out.y = pack4_e4m3(q[4], q[5], q[6], q[7]);
-    return out;
-}
-
 // 8 bf16 of row `row` from column `col` on, zeros outside the M x K matrix
 template <bool VEC>
 __device__ __forceinline__ uint4 load8(const uint16_t* __restrict__ x, int row, int col, int M, int K, int64_t x_row_stride) {

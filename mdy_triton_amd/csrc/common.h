@@ -66,6 +66,28 @@ __device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float 
     return (uint32_t)w;
 }
 
+// One lane's 8 values of a 128-element group with absmax `amax` -> 8 e4m3fn bytes and the group's scale: the
+// reciprocal + 2-FMA quotient where it is proven bit-identical to IEEE division, plain division elsewhere.
+template <int MODE>
+__device__ __forceinline__ uint2 quantize8(const float (&f)[8], float amax, float& scale_out) {
+    float s = group_scale<MODE>(amax);
+    scale_out = s;
+    float q[8];
+    bool fast = MODE == 0 ? fast_quotient_ok<0>(amax) : (amax <= 1e4f);
+    if (fast) {
+        float r = 1.0f / s;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i] = fast_quotient(f[i], s, r);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i] = sat_for_mode<MODE>(f[i] / s);
+    }
+    uint2 out;
+    out.x = pack4_e4m3(q[0], q[1], q[2], q[3]);
+    out.y = pack4_e4m3(q[4], q[5], q[6], q[7]);
+    return out;
+}
+
 // 4x4 byte transpose with v_perm_b32: r[i] holds bytes (i,0..3); on return c[j] holds bytes (0..3, j).
 __device__ __forceinline__ void transpose4x4_bytes(const uint32_t (&r)[4], uint32_t (&c)[4]) {
     // __builtin_amdgcn_perm(s0, s1, sel): result byte k = byte sel[k] of {s1: 0..3, s0: 4..7}

@@ -102,19 +102,10 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const uint16_t* __restrict_
 #pragma unroll
             for (int i = 0; i < 8; i += 2) m = fmaxf(fmaxf(fabsf(f[i]), fabsf(f[i + 1])), m);
             const float amax = row16_max(m);
-            const float sc = group_scale<MODE>(amax);
-            const bool fast = MODE == 0 ? fast_quotient_ok<0>(amax) : (amax <= 1e4f);
-            float q[8];
-            if (fast) {
-                const float rr = 1.0f / sc;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) q[i] = fast_quotient(f[i], sc, rr);
-            } else {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) q[i] = sat_for_mode<MODE>(f[i] / sc);
-            }
+            float sc;
+            const uint2 packed = quantize8<MODE>(f, amax, sc);
             if (row < PM && col < PN) {
-                store_nt8(y + (int64_t)row * PN + col, make_uint2(pack4_e4m3(q[0], q[1], q[2], q[3]), pack4_e4m3(q[4], q[5], q[6], q[7])));
+                store_nt8(y + (int64_t)row * PN + col, packed);
                 if ((lane & 15) == 0) s[(int64_t)row * s_row_stride + (int64_t)(col >> 7) * s_col_stride] = sc;
             }
         }
