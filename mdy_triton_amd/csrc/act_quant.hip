@@ -212,7 +212,7 @@ __global__ __launch_bounds__(256) void quotient_selfcheck_kernel(unsigned long l
     const uint32_t ai = (uint32_t)amax_lo + blockIdx.x;
     const float amax = bf16_one((uint16_t)ai);
     const float s = group_scale<MODE>(amax);
-    const bool fast = MODE == 0 ? fast_quotient_ok<0>(amax) : (amax <= 1e4f);
+    const bool fast = group_is_fast<MODE>(amax);      // the quantizers' own criterion
     const float r = 1.0f / s;
     unsigned long long pairs = 0, f32_bad = 0, fp8_bad = 0, plain = 0;
     for (uint32_t t = threadIdx.x; t < 2 * (ai + 1); t += blockDim.x) {

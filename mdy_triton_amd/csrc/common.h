@@ -69,13 +69,9 @@ __device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float 
 // One lane's 8 values of a 128-element group with absmax `amax` -> 8 e4m3fn bytes and the group's scale: the
 // reciprocal + 2-FMA quotient where it is proven bit-identical to IEEE division, plain division elsewhere.
 template <int MODE>
-__device__ __forceinline__ uint2 quantize8(const float (&f)[8], float amax, float& scale_out) {
-    float s = group_scale<MODE>(amax);
-    scale_out = s;
+__device__ __forceinline__ uint2 quantize8_scaled(const float (&f)[8], float s, float r, bool fast) {
     float q[8];
-    bool fast = MODE == 0 ? fast_quotient_ok<0>(amax) : (amax <= 1e4f);
     if (fast) {
-        float r = 1.0f / s;
 #pragma unroll
         for (int i = 0; i < 8; ++i) q[i] = fast_quotient(f[i], s, r);
     } else {
@@ -86,6 +82,18 @@ __device__ __forceinline__ uint2 quantize8(const float (&f)[8], float amax, floa
     out.x = pack4_e4m3(q[0], q[1], q[2], q[3]);
     out.y = pack4_e4m3(q[4], q[5], q[6], q[7]);
     return out;
+}
+// True when a group with this absmax may take the reciprocal form in its dialect (the DeepLinear dialect also
+// needs |x / s| <= 448 without the saturating clamp, i.e. an absmax within the 1e4 clamp).
+template <int MODE>
+__device__ __forceinline__ bool group_is_fast(float amax) {
+    return MODE == 0 ? fast_quotient_ok<0>(amax) : (amax <= 1e4f);
+}
+template <int MODE>
+__device__ __forceinline__ uint2 quantize8(const float (&f)[8], float amax, float& scale_out) {
+    const float s = group_scale<MODE>(amax);
+    scale_out = s;
+    return quantize8_scaled<MODE>(f, s, 1.0f / s, group_is_fast<MODE>(amax));
 }
 
 // 4x4 byte transpose with v_perm_b32: r[i] holds bytes (i,0..3); on return c[j] holds bytes (0..3, j).

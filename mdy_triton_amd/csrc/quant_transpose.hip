@@ -93,7 +93,7 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
         const float sc = group_scale<1>(rmax[i]);
         const float r = 1.0f / sc;
         float q[8];
-        if (rmax[i] <= 1e4f) {
+        if (group_is_fast<1>(rmax[i])) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) q[j] = qt_quot<true>(f[i][j], sc, r);
         } else {
@@ -158,7 +158,7 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
     }
     bool tfast = true;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) tfast = tfast && (tamax[j] <= 1e4f);
+    for (int j = 0; j < 8; ++j) tfast = tfast && group_is_fast<1>(tamax[j]);
     uint32_t qlo[RPT], qhi[RPT];   // row i of the transposed copy's bytes: columns 0..3 | 4..7
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {

@@ -74,7 +74,7 @@ __global__ __launch_bounds__(512) void weight_quant_kernel(const uint16_t* __res
     for (int w = 1; w < WAVES; ++w) amax = fmaxf(amax, wave_max[w]);
 
     const float sc = group_scale<MODE>(amax);
-    const bool fast = MODE == 0 ? fast_quotient_ok<0>(amax) : (amax <= 1e4f);
+    const bool fast = group_is_fast<MODE>(amax);
     const float r = 1.0f / sc;
     if (t == 0) {
         s[(int64_t)bn * (PK >> 7) + bk] = sc;
@@ -83,23 +83,7 @@ __global__ __launch_bounds__(512) void weight_quant_kernel(const uint16_t* __res
     uint32_t qlo[RPT], qhi[RPT];   // row i of the quantized bytes: columns 0..3 | 4..7
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
-        float q[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            if (fast) {
-                q[j] = fast_quotient(f[i][j], sc, r);
-            } else {
-                float v = f[i][j] / sc;
-                if (MODE != 0) {
-                    float c = __builtin_amdgcn_fmed3f(v, -kFp8Max, kFp8Max);
-                    v = (v != v) ? v : c;
-                }
-                q[j] = v;
-            }
-        }
-        uint2 o;
-        o.x = pack4_e4m3(q[0], q[1], q[2], q[3]);
-        o.y = pack4_e4m3(q[4], q[5], q[6], q[7]);
+        const uint2 o = quantize8_scaled<MODE>(f[i], sc, r, fast);
         const int row = rbase + i;  // < PN because PN % 128 == 0
         store_nt8(y + (int64_t)row * PK + c0, o);
         qlo[i] = o.x;
