@@ -39,6 +39,14 @@ namespace mdy {
 // chunk swizzle of an LDS row; depends on row bits 0..3 only so that rows 16 apart share it
 __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
+// The promotion of one K block (offical_kernel.py:86): acc += (MFMA result of the block) * (its combined scale).
+__device__ __forceinline__ void fold(floatx4& acc, const floatx4& p, float sc) {
+    acc[0] = __builtin_fmaf(p[0], sc, acc[0]);
+    acc[1] = __builtin_fmaf(p[1], sc, acc[1]);
+    acc[2] = __builtin_fmaf(p[2], sc, acc[2]);
+    acc[3] = __builtin_fmaf(p[3], sc, acc[3]);
+}
+
 template <typename OUT>
 __device__ __forceinline__ void store4(OUT* c, int64_t ldc, int m, int n, int M, int N, const float (&v)[4], bool vec_ok) {
     if (m >= M || n >= N) return;
@@ -307,10 +315,7 @@ __device__ __forceinline__ void fp8_gemm_tile(
                 const int u = t - DEPTH, si = u / NH, h = u % NH;
                 const int i = HOLD_A ? h : si, j = HOLD_A ? si : h;
                 const floatx4 q = p[u % (DEPTH + 1)];
-                acc[i][j][0] = __builtin_fmaf(q[0], sc[i], acc[i][j][0]);
-                acc[i][j][1] = __builtin_fmaf(q[1], sc[i], acc[i][j][1]);
-                acc[i][j][2] = __builtin_fmaf(q[2], sc[i], acc[i][j][2]);
-                acc[i][j][3] = __builtin_fmaf(q[3], sc[i], acc[i][j][3]);
+                fold(acc[i][j], q, sc[i]);
             }
 #pragma unroll
             for (int j = 0; j < NDMA; ++j) {
@@ -585,10 +590,7 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_kernel(const ui
                 const float sc = cur.sa[i] * cur.sb[j];
                 const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
                 const floatx4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, zero, 0, 0, 0, 0, 0, 0);
-                acc[j][i][0] = __builtin_fmaf(p[0], sc, acc[j][i][0]);
-                acc[j][i][1] = __builtin_fmaf(p[1], sc, acc[j][i][1]);
-                acc[j][i][2] = __builtin_fmaf(p[2], sc, acc[j][i][2]);
-                acc[j][i][3] = __builtin_fmaf(p[3], sc, acc[j][i][3]);
+                fold(acc[j][i], p, sc);
             }
         }
         if (more) cur = nxt;
@@ -724,10 +726,7 @@ __global__ __launch_bounds__(512) void fp8_gemm_strip_kernel(
                     const float sc = lds_sa[buf][kc][i * 16 + frow] * sb;
                     const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
                     const floatx4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, zero, 0, 0, 0, 0, 0, 0);
-                    acc[i][0] = __builtin_fmaf(p[0], sc, acc[i][0]);
-                    acc[i][1] = __builtin_fmaf(p[1], sc, acc[i][1]);
-                    acc[i][2] = __builtin_fmaf(p[2], sc, acc[i][2]);
-                    acc[i][3] = __builtin_fmaf(p[3], sc, acc[i][3]);
+                    fold(acc[i], p, sc);
                 }
             }
         }
