@@ -39,6 +39,14 @@ namespace mdy {
 // chunk swizzle of an LDS row; depends on row bits 0..3 only so that rows 16 apart share it
 __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
+// One 128-deep scale block of a 16x16 sub-tile, from zero: v_mfma_f32_16x16x128_f8f6f4 with e4m3 operands and unit
+// hardware scales.  The weight rows go in as the MFMA's rows and the activation rows as its columns, so a lane's
+// four results are four consecutive n of one m.
+__device__ __forceinline__ floatx4 mfma_block(const intx8& weight_rows, const intx8& act_rows) {
+    const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(weight_rows, act_rows, zero, 0, 0, 0, 0, 0, 0);
+}
+
 // The promotion of one K block (offical_kernel.py:86): acc += (MFMA result of the block) * (its combined scale).
 __device__ __forceinline__ void fold(floatx4& acc, const floatx4& p, float sc) {
     acc[0] = __builtin_fmaf(p[0], sc, acc[0]);
@@ -297,9 +305,7 @@ __device__ __forceinline__ void fp8_gemm_tile(
                 if (h == 0 && si + 1 < NS) fx[(si + 1) & 1] = read_frag(lx, x0, x1, si + 1);
                 const intx8 fa_ = HOLD_A ? fh[h] : fx[si & 1];
                 const intx8 fb_ = HOLD_A ? fx[si & 1] : fh[h];
-                const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
-                // rows of the MFMA = n (B panel), columns = m (A panel)
-                p[t % (DEPTH + 1)] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb_, fa_, zero, 0, 0, 0, 0, 0, 0);
+                p[t % (DEPTH + 1)] = mfma_block(fb_, fa_);
                 if (t == TB) {
                     // K block kb+1 has landed once only the younger loads are left in flight
                     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(YOUNGER) : "memory");
@@ -588,8 +594,7 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_kernel(const ui
                 const intx8 fa = intx8{cur.alo[i][0], cur.alo[i][1], cur.alo[i][2], cur.alo[i][3],
                                        cur.ahi[i][0], cur.ahi[i][1], cur.ahi[i][2], cur.ahi[i][3]};
                 const float sc = cur.sa[i] * cur.sb[j];
-                const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
-                const floatx4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, zero, 0, 0, 0, 0, 0, 0);
+                const floatx4 p = mfma_block(fb, fa);
                 fold(acc[j][i], p, sc);
             }
         }
@@ -724,8 +729,7 @@ __global__ __launch_bounds__(512) void fp8_gemm_strip_kernel(
                     const intx4 hi = *reinterpret_cast<const intx4*>(la + a_rd1);
                     const intx8 fa = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                     const float sc = lds_sa[buf][kc][i * 16 + frow] * sb;
-                    const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
-                    const floatx4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, zero, 0, 0, 0, 0, 0, 0);
+                    const floatx4 p = mfma_block(fb, fa);
                     fold(acc[i], p, sc);
                 }
             }
