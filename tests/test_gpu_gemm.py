@@ -465,3 +465,34 @@ def test_deep_linear_backward_partial_requirements():
     xg = x.clone().requires_grad_(True)
     lin(xg).sum().backward()                      # only dgrad
     assert close(xg.grad, ref[0])
+
+
+# ------------------------------------------------------------------ non-finite values
+@pytest.mark.parametrize("M,N,K", [(256, 384, 512),       # MFMA tiles
+                                   (8, 256, 512),         # weight-streaming kernel
+                                   (130, 1100, 4224),     # split along K
+                                   (16, 25600, 256),      # strip kernel
+                                   (40, 48, 100)])        # one thread per element
+def test_gemm_non_finite_values_follow_the_block_formula(M, N, K):
+    """A NaN operand byte poisons exactly its output row / column, an infinite scale makes its row infinite
+    with the sign of the block's partial sum: the same pattern as the reference's accumulation
+    (offical_kernel.py:80-91) evaluated block by block on the CPU, in every kernel."""
+    g = torch.Generator().manual_seed(M * 7 + N)
+    a = torch.randint(-6, 7, (M, K), generator=g).float().to(FP8)
+    b = torch.randint(-6, 7, (N, K), generator=g).float().to(FP8)
+    KB, NB = (K + 127) // 128, (N + 127) // 128
+    a_s = torch.rand(M, KB, generator=g) + 0.5
+    b_s = torch.rand(NB, KB, generator=g) + 0.5
+    au, bu = a.view(torch.uint8), b.view(torch.uint8)
+    au[1, 3] = 0x7F                                     # NaN in activation row 1
+    bu[5, K - 1] = 0xFF                                 # NaN in weight row 5 (last K element)
+    a_s[2, KB - 1] = float("inf")                       # row 2: +-inf, or NaN where the block's partial sum is 0
+    a_s[3, 0] = 0.0                                     # a zero scale drops the block
+    ref = O.fp8_gemm_blockwise(a, a_s, b, b_s, dtype=torch.float32)
+    got = m.fp8_gemm(a.to(DEV), a_s.to(DEV), b.to(DEV), b_s.to(DEV), out_dtype=torch.float32).cpu()
+    assert torch.equal(torch.isnan(got), torch.isnan(ref))
+    assert torch.isnan(got[1]).all() and torch.isnan(got[:, 5]).all()
+    assert torch.equal(torch.isinf(got), torch.isinf(ref)) and torch.equal(got[torch.isinf(ref)], ref[torch.isinf(ref)])
+    fin = torch.isfinite(ref)
+    # fp32 sums of ~1e3-sized terms in a different order (and scale products rounded differently): a few ulps of 1e3
+    assert fin[4:].any() and torch.allclose(got[fin], ref[fin], rtol=1e-4, atol=1e-2)
