@@ -11,6 +11,10 @@
  *     mdy_fp8_last_error() returns a thread-local message for the last non-zero
  *     return on the calling thread.
  *
+ * Sizes: every row / column count up to 2^30 (MDY_E_SHAPE beyond); operands may exceed 2^32 bytes (all
+ * addressing is 64-bit).  A launch whose block count does not fit the grid limits (more than 33 million columns)
+ * returns hipErrorInvalidConfiguration.
+ *
  * Reference interfaces are cited as file:line under the reference tree
  * (triton_kernels/deepseekv3/offical_kernel.py = "offical_kernel.py",
  *  triton_kernels/dpsk_fp8linear/fp8.py        = "fp8.py").
