@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define MDY_FP8_ABI_VERSION 2
+#define MDY_FP8_ABI_VERSION 3
 
 /* error codes (negative = argument rejected before any launch) */
 #define MDY_OK 0
@@ -176,6 +176,21 @@ int64_t mdy_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int mdy_fp8_gemm_nt_ws(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
                        const void* b, const float* b_s, void* c, const void* bias, int64_t M, int64_t N,
                        int64_t K, int out_dtype, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Which kernel family mdy_fp8_gemm_nt (with_workspace = 0) or mdy_fp8_gemm_nt_ws with a sufficient workspace
+ * (with_workspace = 1) runs for these operands; launches nothing, needs no GPU.  No counterpart in the reference
+ * (its Triton kernel has one code path); the Python wrappers use it to warn when a large shape would take the
+ * scalar kernel, which exists for K % 128 != 0 and unaligned operands and is ~100x slower than the MFMA kernels
+ * (aligned shapes reach it only with K > 65536, or activation scales spanning 2^31 bytes or more, and M > 64).
+ * a and b are only inspected for 16-byte alignment (NULL counts as aligned).
+ */
+#define MDY_PATH_SCALAR 0
+#define MDY_PATH_SMALL_M 1
+#define MDY_PATH_STRIP 2
+#define MDY_PATH_TILES 3
+#define MDY_PATH_TILES_SPLIT_K 4
+int mdy_fp8_gemm_path(const void* a, const void* b, int64_t as_row_stride, int64_t as_col_stride, int64_t M,
+                      int64_t N, int64_t K, int with_workspace);
 
 /* Grouped (mixture-of-experts) block-scaled FP8 GEMM, NT layout: the rows of a are split into G
  * consecutive groups of m_splits[g] rows and group g is multiplied with its own weight,

@@ -10,7 +10,7 @@ import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libmdyfp8.so")
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _lock = threading.Lock()
 _lib = None
@@ -31,6 +31,7 @@ SIGNATURES = {
     "mdy_fp8_gemm_nt": [_p, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p],
     "mdy_fp8_gemm_nt_ws": [_p, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p, _i64, _p],
     "mdy_fp8_gemm_workspace_bytes": [_i64, _i64, _i64],
+    "mdy_fp8_gemm_path": [_p, _p, _i64, _i64, _i64, _i64, _i64, _int],
     "mdy_add_bias": [_p, _p, _i64, _i64, _p],
     "mdy_cast_f32_to_e4m3": [_p, _p, _i64, _int, _p],
     "mdy_quotient_selfcheck": [_p, _int, _int, _int, _p],
@@ -60,7 +61,8 @@ def load():
             fn = getattr(lib, name)
             fn.argtypes = argtypes
             fn.restype = (ctypes.c_char_p if name == "mdy_fp8_last_error" else
-                          ctypes.c_int64 if name == "mdy_fp8_gemm_workspace_bytes" else ctypes.c_int)
+                          ctypes.c_int64 if name in ("mdy_fp8_gemm_workspace_bytes", "mdy_fp8_gemm_static_workspace_bytes")
+                          else ctypes.c_int)
         got = lib.mdy_fp8_abi_version()
         if got != ABI_VERSION:
             raise MdyFp8Error("libmdyfp8.so ABI version %d, expected %d: rebuild" % (got, ABI_VERSION))

@@ -1,5 +1,7 @@
 """Tensor plumbing shared by the operator modules: device checks, raw pointers,
 the current HIP stream.  PyTorch is used for memory and streams only."""
+import warnings
+
 import torch
 
 from . import _lib
@@ -81,3 +83,27 @@ def gemm_workspace(device, M, N, K):
     if nbytes <= 0:
         return None
     return torch.empty(nbytes, device=device, dtype=torch.uint8)
+
+
+_SLOW_WARNED = set()
+
+
+def warn_if_scalar_gemm(a, b, as_rs, as_cs, M, N, K, who):
+    """One warning per shape when a LARGE aligned-K GEMM would run on the scalar kernel (one thread per output
+    element, ~100x slower than the MFMA kernels).  That kernel is the intended path for K % 128 != 0; a shape
+    with K % 128 == 0 reaches it only when K > 65536, when the activation scales span 2^31 bytes or more, or
+    when an operand is not 16-byte aligned - none of which should pass silently.  The test that decides is the
+    library's own (mdy_fp8_gemm_path); the cheap checks in front of it keep the common case free."""
+    if M <= 64 or K % 128 != 0:
+        return
+    extent = ((M - 1) * as_rs + (K // 128 - 1) * as_cs + 1) * 4
+    if K <= 65536 and 0 <= extent < (1 << 31) and as_rs >= 0 and as_cs >= 0 and not ((a.data_ptr() | b.data_ptr()) & 15):
+        return
+    key = (M, N, K, as_rs, as_cs)
+    if key in _SLOW_WARNED:
+        return
+    if _lib.load().mdy_fp8_gemm_path(a.data_ptr(), b.data_ptr(), as_rs, as_cs, M, N, K, 1) == 0:
+        _SLOW_WARNED.add(key)
+        warnings.warn("%s: M=%d N=%d K=%d runs on the scalar fallback kernel (K > 65536, activation scales spanning "
+                      ">= 2^31 bytes, or an operand that is not 16-byte aligned); expect ~100x the time of the MFMA "
+                      "path - split K or the rows into several calls" % (who, M, N, K), RuntimeWarning, stacklevel=3)

@@ -190,6 +190,13 @@ int mdy_fp8_gemm_nt_ws(const void* a, const float* a_s, int64_t as_row_stride, i
                     "fp8_gemm_nt_ws");
 }
 
+int mdy_fp8_gemm_path(const void* a, const void* b, int64_t as_row_stride, int64_t as_col_stride, int64_t M, int64_t N,
+                      int64_t K, int with_workspace) {
+    if (M < 1 || N < 1 || K < 1 || M > kMaxDim || N > kMaxDim || K > kMaxDim)
+        return fail(MDY_E_SHAPE, "fp8_gemm_path: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+    return mdy::fp8_gemm_path(a, b, as_row_stride, as_col_stride, M, N, K, with_workspace);
+}
+
 int mdy_fp8_grouped_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,
                             const float* b_s, void* c, const void* bias, const int64_t* m_splits, int64_t G, int64_t N,
                             int64_t K, int out_dtype, void* stream) {

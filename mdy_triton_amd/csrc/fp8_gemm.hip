@@ -787,15 +787,28 @@ __global__ __launch_bounds__(256) void fp8_gemm_scalar_kernel(const uint8_t* __r
         reinterpret_cast<float*>(c)[(int64_t)m * N + n] = acc;
 }
 
-constexpr int kCUs = 256;   // workgroups of the big tile that run at once (one per CU)
+// Compute units of the current device (workgroups of the big tile that run at once, one per CU): read from the
+// device properties once per device and thread, 256 on a full MI355X, fewer on a partitioned part.
+static int cu_count() {
+    static thread_local int cached_dev = -1, cached_cus = 256;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return cached_cus;
+    if (dev != cached_dev) {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0) cached_cus = cus;
+        cached_dev = dev;
+    }
+    return cached_cus;
+}
 
 template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT>
 static int launch_mfma(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, uint32_t as_bytes,
                        const uint8_t* b, const float* b_s, OUT* c, const uint16_t* bias, int M, int N, int K,
                        int ldc, hipStream_t stream) {
+    const int cus = cu_count();
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     // the 256x256 tile fills a CU's LDS: one workgroup per CU that walks its tiles itself
-    const int wgs = (BM * BN >= 256 * 256 && tiles_m * tiles_n > kCUs) ? kCUs : tiles_m * tiles_n;
+    const int wgs = (BM * BN >= 256 * 256 && tiles_m * tiles_n > cus) ? cus : tiles_m * tiles_n;
     dim3 grid((unsigned)wgs), block(WGM * WGN * 64);
     hipLaunchKernelGGL((fp8_gemm_mfma_kernel<BM, BN, WGM, WGN, STAGES, OUT>), grid, block, 0, stream, a, a_s, (int)as_rs,
                        (int)as_cs, as_bytes, b, b_s, c, bias, M, N, K, ldc, tiles_m, tiles_n);
@@ -809,24 +822,26 @@ static int launch_mfma(const uint8_t* a, const float* a_s, int64_t as_rs, int64_
 // the time), which fills the machine for one short round instead of half-filling a long one.
 // Returns tiles_n when no split pays.
 static int main_tile_columns(int tiles_m, int tiles_n) {
+    const int cus = cu_count();
     const long total = (long)tiles_m * tiles_n;
-    const long full_rounds = total / kCUs;
-    if (full_rounds < 1 || total % kCUs == 0) return tiles_n;
-    const int cols_main = (int)(full_rounds * kCUs / tiles_m);
+    const long full_rounds = total / cus;
+    if (full_rounds < 1 || total % cus == 0) return tiles_n;
+    const int cols_main = (int)(full_rounds * cus / tiles_m);
     if (cols_main <= 0 || cols_main >= tiles_n) return tiles_n;
-    const long rounds_main = ((long)cols_main * tiles_m + kCUs - 1) / kCUs;
+    const long rounds_main = ((long)cols_main * tiles_m + cus - 1) / cus;
     const long rem_small = 2L * (tiles_n - cols_main) * tiles_m;
-    const double cost_split = (double)rounds_main + 0.6 * (double)((rem_small + kCUs - 1) / kCUs);
-    const double cost_plain = (double)((total + kCUs - 1) / kCUs);
+    const double cost_split = (double)rounds_main + 0.6 * (double)((rem_small + cus - 1) / cus);
+    const double cost_plain = (double)((total + cus - 1) / cus);
     return cost_split < cost_plain - 0.05 ? cols_main : tiles_n;
 }
 
 // 256x256 tiles (one workgroup per CU) when they fill most of the CUs, or when 128x128 tiles (two workgroups
 // per CU) would need a second round: 144..199 tiles of 256x256 measured 20-26 % faster than 577..796 of 128x128.
 static bool big_tiles_pay(int64_t M, int64_t N) {
+    const int cus = cu_count();
     const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
     const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128);
-    return t256 >= 200 || t128 > 2 * kCUs;
+    return t256 >= 200 || t128 > 2 * cus;
 }
 
 // Tile and ring depth for the shapes that do not take 256x256 tiles:
@@ -839,15 +854,16 @@ static bool big_tiles_pay(int64_t M, int64_t N) {
 // rather than two 128x128 workgroups per CU: 4096x1536x7168 77 -> 70 us, 8192x1024x7168 91 -> 75 us,
 // 1100x6000x16384 178 -> 140 us (K <= 512: 4-6 % slower, so short K keeps the 128x128 tiles).
 static int few_tiles_config(int M, int N, int K) {
+    const int cus = cu_count();
     const long rows128 = (M + 127) / 128, rows64 = (M + 63) / 64, rows256 = (M + 255) / 256;
     const long cols128 = (N + 127) / 128, cols64 = (N + 63) / 64, cols256 = (N + 255) / 256;
-    if (rows64 * cols64 <= kCUs) return 3;
-    if (rows128 * cols64 <= kCUs) return 2;
-    if (rows128 * cols128 <= kCUs) return 1;
+    if (rows64 * cols64 <= cus) return 3;
+    if (rows128 * cols64 <= cus) return 2;
+    if (rows128 * cols128 <= cus) return 1;
     if (K < 1024) return 0;    // a handful of K blocks: two short workgroups per CU hide each other's prologue and epilogue
     const long wide = rows128 * cols256, tall = rows256 * cols128;
-    if (wide <= kCUs) return 4;    // also when it pads more than the tall tile: 12800x384x7168 82 against 95 us
-    if (tall <= kCUs) return 5;
+    if (wide <= cus) return 4;    // also when it pads more than the tall tile: 12800x384x7168 82 against 95 us
+    if (tall <= cus) return 5;
     return 0;
 }
 
@@ -969,6 +985,7 @@ struct SplitPlan {
 };
 
 static SplitPlan plan_split(int64_t M, int64_t N, int64_t K) {
+    const int cus = cu_count();
     SplitPlan p{0, 1, 0};
     // up to 32 rows the weight-streaming kernel is as fast; below 32 K blocks the second pass costs more than
     // the split gains
@@ -982,10 +999,10 @@ static SplitPlan plan_split(int64_t M, int64_t N, int64_t K) {
     const long tiles[4] = {0, rows128 * cols128, rows128 * cols64, rows64 * cols64};
     for (int cfg = 1; cfg <= 3; ++cfg) {
         if (cfg != 3 && M <= 64) continue;                       // 128-row tiles would be half empty
-        long ks = kCUs / tiles[cfg];
+        long ks = cus / tiles[cfg];
         if (ks > KB / 8) ks = KB / 8;
         if (ks < 2) continue;
-        if (tiles[cfg] * ks < kCUs * 3 / 4 && cfg != 3) continue;  // a smaller tile fills the machine better
+        if (tiles[cfg] * ks < cus * 3 / 4 && cfg != 3) continue;  // a smaller tile fills the machine better
         p.config = cfg;
         p.kb_per = (int)((KB + ks - 1) / ks);
         p.ksplit = (KB + p.kb_per - 1) / p.kb_per;
@@ -1096,6 +1113,24 @@ int launch_fp8_gemm_nt_ws(const void* a, const float* a_s, int64_t as_row_stride
         return launch_fp8_gemm_nt(a, ts, 1, M, b, b_s, c, bias, M, N, K, out_dtype, stream);
     }
     return launch_fp8_gemm_nt(a, a_s, as_row_stride, as_col_stride, b, b_s, c, bias, M, N, K, out_dtype, stream);
+}
+
+// Which kernel family a call would run (the same tests as dispatch() / launch_splitk(), no launch):
+//   0 scalar (one thread per output element)   1 small-M weight streaming   2 strip   3 MFMA tiles
+//   4 MFMA tiles split along K (needs the workspace)
+int fp8_gemm_path(const void* a, const void* b, int64_t as_rs, int64_t as_cs, int64_t M, int64_t N, int64_t K,
+                  int with_workspace) {
+    const int64_t KB = (K + 127) / 128;
+    const int64_t as_extent = ((M - 1) * as_rs + (KB - 1) * as_cs + 1) * 4;
+    const bool mfma_ok = (K % 128 == 0) && ((reinterpret_cast<uintptr_t>(a) & 15) == 0) &&
+                         ((reinterpret_cast<uintptr_t>(b) & 15) == 0);
+    const bool big_ok = mfma_ok && K <= (1 << 16) && as_rs >= 0 && as_cs >= 0 && as_extent < ((int64_t)1 << 31);
+    if (with_workspace && big_ok && plan_split(M, N, K).ksplit > 1) return 4;
+    if (!mfma_ok || (M > 64 && !big_ok)) return 0;
+    if (M <= 64 && big_ok && strip_pays(M, (N + 127) / 128)) return 2;
+    if (M >= 32 && M <= 64 && big_ok && ((N + 127) / 128 >= 128 || (N + 63) / 64 >= 100)) return 3;
+    if (M <= 64) return 1;
+    return 3;
 }
 
 int launch_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,

@@ -10,7 +10,7 @@ from typing import Optional, Tuple
 
 import torch
 
-from ._torch_glue import FP8, check, gemm_workspace, lib, on_device, ptr, require_gpu, stream_ptr
+from ._torch_glue import FP8, check, gemm_workspace, lib, on_device, ptr, require_gpu, stream_ptr, warn_if_scalar_gemm
 
 
 def _cdiv(a: int, b: int) -> int:
@@ -151,6 +151,7 @@ def fp8_matmul(qa: torch.Tensor, sa: torch.Tensor, qb: torch.Tensor, sb: torch.T
     if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != N or not bias.is_contiguous()):
         raise ValueError("bias must be a contiguous bfloat16 [N] tensor")
     with on_device(dev):
+        warn_if_scalar_gemm(qa, qb, sa.stride(0), sa.stride(1), M, N, K, "fp8_matmul")
         ws = gemm_workspace(dev, M, N, K)      # scratch for shapes that are split along K, else None
         check(lib().mdy_fp8_gemm_nt_ws(ptr(qa), ptr(sa), sa.stride(0), sa.stride(1), ptr(qb), ptr(sb), ptr(out),
                                        ptr(bias), M, N, K, 0, ptr(ws), ws.numel() if ws is not None else 0,
@@ -218,24 +219,59 @@ class _DeepLinear(torch.autograd.Function):
 class DeepLinear(torch.nn.Linear):
     """nn.Linear whose forward and backward run the block-wise FP8 path (fp8.py:347-349).
 
-    The bf16 master weight is quantized per 128x128 block; the result is cached
-    and reused until the weight tensor changes (its version counter or storage),
-    which removes the per-call re-quantization the reference notebook subtracts by
-    hand.  Set `cache_weight=False` to re-quantize on every call as the reference
-    does, `fuse_bias=True` to add the bias inside the GEMM epilogue.
+    By default the bf16 master weight is quantized per 128x128 block on every call, as the
+    reference does (fp8.py:320).  `cache_weight = True` keeps the quantized copies between
+    calls; the owner of the weight then says when it changed:
+
+      * `invalidate_weight_cache()` (or `set_first_micro_batch(True)`, the name the reference's
+        Megatron patch uses for the same signal, megatron_patchs/manger.py:77-86) after every
+        optimizer step.  It is REQUIRED after updates that go through `weight.data`
+        (`weight.data.copy_(main_param)`, `weight.data.mul_(...)`: what Megatron's, apex's and
+        DeepSpeed's optimizers do): those do not bump the tensor's version counter, so nothing
+        else can see them;
+      * in-place updates through the tensor itself (`weight.mul_()`, `optimizer.step()` of
+        torch.optim) bump the version counter and a new storage changes the data pointer; both are
+        noticed without a call.
+
+    `check_weight_cache = True` (or the environment variable MDY_FP8_CHECK_WEIGHT_CACHE=1)
+    verifies every cache hit against a checksum of the weight taken when it was quantized and
+    raises if they differ - a debugging aid (one reduction and one host synchronisation per call).
+    `fuse_bias = True` adds the bias inside the GEMM epilogue.
     """
 
-    cache_weight = True
+    cache_weight = False
     fuse_bias = False
+    check_weight_cache = False
+
+    @staticmethod
+    def _fingerprint(w: torch.Tensor) -> int:
+        """Exact 64-bit sum of the weight's 16-bit patterns (integer arithmetic, so order does not matter)."""
+        return int(torch.sum(w.detach().contiguous().view(torch.int16), dtype=torch.int64).item())
+
+    def invalidate_weight_cache(self) -> None:
+        """Forget the cached quantized weight: the next forward quantizes the current one."""
+        self._wq_cache = None
+
+    def set_first_micro_batch(self, flag: bool = True) -> None:
+        """flag=True marks the weight as updated since it was last quantized (the first micro-batch
+        of a step in the reference's Megatron patch); False leaves the cache as it is."""
+        if flag:
+            self.invalidate_weight_cache()
 
     def _quantized_weight(self, with_transpose: bool):
+        import os
         w = self.weight
         key = (w.data_ptr(), w._version, tuple(w.shape), w.device)
+        checking = self.check_weight_cache or os.environ.get("MDY_FP8_CHECK_WEIGHT_CACHE", "0") not in ("", "0")
         cached = getattr(self, "_wq_cache", None)
         if cached is not None and cached[0] == key and (cached[1][2] is not None or not with_transpose):
+            if checking and cached[2] is not None and cached[2] != self._fingerprint(w):
+                raise RuntimeError(
+                    "DeepLinear: the weight changed since its quantized copy was cached (an update through "
+                    "`.data`, which bumps no version counter); call invalidate_weight_cache() after such updates")
             return cached[1]
         quantized = quant_weight(w.detach(), only_forward=not with_transpose)
-        self._wq_cache = (key, quantized)
+        self._wq_cache = (key, quantized, self._fingerprint(w) if checking else None)
         return quantized
 
     def forward(self, input):

@@ -16,6 +16,12 @@ from ._torch_glue import FP8, check, lib, on_device, ptr, require_gpu, stream_pt
 _ORDERS = ("up-gate", "gate-up")
 
 
+def _require_e4m3(fp8_dtype, who: str):
+    if fp8_dtype != FP8:
+        raise TypeError("%s: only torch.float8_e4m3fn is implemented, got %s (the reference defaults to "
+                        "float8_e5m2; pass fp8_dtype=torch.float8_e4m3fn)" % (who, fp8_dtype))
+
+
 def _flatten_up_gate(x: torch.Tensor, order: str, who: str):
     assert order in _ORDERS, "please indicate the order of input, up-gate or gate-up"
     if x.dtype != torch.bfloat16:
@@ -141,8 +147,9 @@ class _Fp8MlpCkptOps(torch.autograd.Function):
     the two input-gradient GEMMs on the quantizers' transposed copies."""
 
     @staticmethod
-    def forward(ctx, x, w_up_gate, w_down, order="up-gate", up_gate_cache=None, down_cache=None):
+    def forward(ctx, x, w_up_gate, w_down, fp8_dtype=FP8, order="up-gate", up_gate_cache=None, down_cache=None):
         from . import fp8 as L
+        _require_e4m3(fp8_dtype, "fp8_ckpt_mlp")
         shape = x.shape
         x2 = x.reshape(-1, shape[-1])
         M, H = x2.shape
@@ -181,11 +188,14 @@ class _Fp8MlpCkptOps(torch.autograd.Function):
         q_du, s_du, q_dut, s_dut = L.quant_grad_output(dup_gate)
         dx = L.fp8_matmul(q_du[:M], s_du[:M], q_wut[:H], s_wut[:cd(H, 128)]).view(ctx.shape)
         dw_up_gate = L.fp8_matmul(q_dut[:N2], s_dut[:N2], q_xt[:H], s_xt[:cd(H, 128)])
-        return dx, dw_up_gate, dw_down, None, None, None
+        return dx, dw_up_gate, dw_down, None, None, None, None
 
 
-def fp8_ckpt_mlp(x, w_up_gate, w_down, order="up-gate"):
-    return _Fp8MlpCkptOps.apply(x, w_up_gate, w_down, order)
+def fp8_ckpt_mlp(x, w_up_gate, w_down, fp8_dtype=FP8, order="up-gate"):
+    """Memory-saving FP8 MLP step with the reference's positional order (fp8_kernel.py:436-494:
+    `fp8_ckpt_mlp(h, w1, w2, self.fp8_dtype, self.order)`).  Only float8_e4m3fn is implemented: the reference's
+    default, float8_e5m2, raises TypeError here."""
+    return _Fp8MlpCkptOps.apply(x, w_up_gate, w_down, fp8_dtype, order)
 
 
 class Fp8MLP(torch.nn.Module):
@@ -202,8 +212,7 @@ class Fp8MLP(torch.nn.Module):
     def __init__(self, hidden_size, intermediate_size, order="up-gate", fp8_dtype=FP8, low_memory=False,
                  device=None, dtype=torch.bfloat16):
         super().__init__()
-        if fp8_dtype != FP8:
-            raise TypeError("only torch.float8_e4m3fn is implemented")
+        _require_e4m3(fp8_dtype, "Fp8MLP")
         assert order in _ORDERS, "please indicate the order of input, up-gate or gate-up"
         from .fp8 import DeepLinear
         self.up_gate_proj = DeepLinear(hidden_size, intermediate_size * 2, bias=False, device=device, dtype=dtype)
@@ -218,7 +227,7 @@ class Fp8MLP(torch.nn.Module):
                                                   down.weight.requires_grad)
         if not needs_grad or low_memory or self.low_memory:
             # cached quantized weights (re-quantized when a weight changes); the forward needs no transposed copies
-            return _Fp8MlpCkptOps.apply(hidden_states, up.weight, down.weight, self.order,
+            return _Fp8MlpCkptOps.apply(hidden_states, up.weight, down.weight, self.fp8_dtype, self.order,
                                         up._quantized_weight(False) if up.cache_weight else None,
                                         down._quantized_weight(False) if down.cache_weight else None)
         return down(triton_silu(up(hidden_states), self.order))

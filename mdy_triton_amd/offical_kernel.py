@@ -8,7 +8,7 @@ from typing import Optional, Tuple
 
 import torch
 
-from ._torch_glue import FP8, check, gemm_workspace, lib, on_device, out_code, ptr, require_gpu, stream_ptr
+from ._torch_glue import FP8, check, gemm_workspace, lib, on_device, out_code, ptr, require_gpu, stream_ptr, warn_if_scalar_gemm
 
 
 def act_quant(x: torch.Tensor, block_size: int = 128) -> Tuple[torch.Tensor, torch.Tensor]:
@@ -85,6 +85,7 @@ def fp8_gemm(a: torch.Tensor, a_s: torch.Tensor, b: torch.Tensor, b_s: torch.Ten
     dtype = out_dtype or torch.get_default_dtype()
     c = a.new_empty(*a.size()[:-1], N, dtype=dtype)
     with on_device(dev):
+        warn_if_scalar_gemm(a, b, KB, 1, M, N, K, "fp8_gemm")
         ws = gemm_workspace(dev, M, N, K)      # scratch for shapes that are split along K, else None
         check(lib().mdy_fp8_gemm_nt_ws(ptr(a), ptr(a_s), KB, 1, ptr(b), ptr(b_s), ptr(c), ptr(bias), M, N, K,
                                        out_code(dtype), ptr(ws), ws.numel() if ws is not None else 0,

@@ -125,3 +125,17 @@ def test_product_never_imports_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert not re.search(r"^\s*(from|import)\s+oracle\b", text, flags=re.M), f
+
+
+def test_gemm_path_query_needs_no_gpu(lib):
+    """mdy_fp8_gemm_path only inspects sizes, strides and pointer alignment."""
+    q = lib.mdy_fp8_gemm_path
+    assert q(None, None, 56, 1, 4096, 18432, 7168, 1) == 3          # MFMA tiles
+    assert q(None, None, 56, 1, 4096, 18432, 7168, 0) == 3
+    assert q(None, None, 16, 1, 16, 7168, 2048, 1) == 1             # weight streaming
+    assert q(None, None, 2, 1, 300, 200, 200, 1) == 0               # K % 128 != 0: scalar
+    assert q(None, None, 1025, 1, 100, 256, 131200, 1) == 0         # K > 65536 and M > 64: scalar
+    assert q(8, None, 56, 1, 4096, 1536, 7168, 1) == 0              # misaligned operand: scalar
+    assert q(None, None, 32, 1, 128, 1536, 4096, 1) == 4            # split along K with a workspace ...
+    assert q(None, None, 32, 1, 128, 1536, 4096, 0) == 3            # ... plain tiles without
+    assert q(None, None, 56, 1, 0, 5, 128, 0) == -2

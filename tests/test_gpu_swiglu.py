@@ -182,3 +182,26 @@ def test_fp8_mlp_three_paths(shape, inter, order):
     for got, want in zip(results[0], (O.deep_linear_forward(act, w_d, None), dx_ref, dw_ug_ref, dw_d_ref)):
         assert got.shape == want.shape
         assert (got.float().cpu() - want.float()).norm() < 5e-3 * want.float().norm()
+
+
+def test_fp8_ckpt_mlp_reference_call_order():
+    """The reference calls `fp8_ckpt_mlp(h, w1, w2, self.fp8_dtype, self.order)` (fp8_kernel.py:510): the
+    fourth positional argument is the fp8 dtype, the fifth the order; float8_e5m2 (the reference's default)
+    is refused with a clear error."""
+    g = torch.Generator().manual_seed(5)
+    H, inter = 256, 384
+    x = torch.randn(32, H, generator=g).bfloat16().to(DEV)
+    w_ug = (torch.randn(2 * inter, H, generator=g) * 0.03).bfloat16().to(DEV)
+    w_d = (torch.randn(H, inter, generator=g) * 0.03).bfloat16().to(DEV)
+    mlp = m.Fp8MLP(H, inter, order="gate-up", device=DEV)
+    with torch.no_grad():
+        mlp.up_gate_proj.weight.copy_(w_ug)
+        mlp.down_proj.weight.copy_(w_d)
+        want = mlp(x)
+        got = m.fp8_ckpt_mlp(x, w_ug, w_d, torch.float8_e4m3fn, "gate-up")
+        assert torch.equal(got, want)
+        assert torch.equal(m.fp8_ckpt_mlp(x, w_ug, w_d, order="gate-up"), want)
+        with pytest.raises(TypeError, match="float8_e4m3fn"):
+            m.fp8_ckpt_mlp(x, w_ug, w_d, torch.float8_e5m2, "gate-up")
+        with pytest.raises(TypeError, match="float8_e4m3fn"):
+            m.Fp8MLP(H, inter, fp8_dtype=torch.float8_e5m2, device=DEV)

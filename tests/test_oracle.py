@@ -250,6 +250,29 @@ def test_add_bias_and_deep_linear_composition():
     assert torch.equal(out, O.add_bias(nb, bias))
 
 
+def test_add_bias_numpy_pin():
+    """add_bias (fp8.py:283-305) from outside the oracle: bf16 bits -> fp32, one fp32 add, round to nearest
+    even back to bf16, all in numpy with the from-definition conversions.  Includes ties (a bias of half an
+    ulp of x), cancellation to zero, a sum that overflows bf16 and a dropped-term check (a zero bias must be
+    the identity)."""
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(37, 200, generator=g).bfloat16()
+    b = torch.randn(200, generator=g).bfloat16()
+    x[0, :4] = torch.tensor([1.0, 1.0, 256.0, 3.0e38]).bfloat16()
+    b[:4] = torch.tensor([2.0 ** -8, -1.0, 1.0, 3.0e38]).bfloat16()       # tie to even, exact zero, tie, overflow
+    xb = x.view(torch.int16).numpy().view(np.uint16)
+    bb = b.view(torch.int16).numpy().view(np.uint16)
+    want = F.f32_to_bf16_bits_rne(F.bf16_bits_to_f32(xb) + F.bf16_bits_to_f32(bb)[None, :])
+    got = O.add_bias(x.clone(), b)
+    assert got.dtype == torch.bfloat16 and got.shape == x.shape
+    assert np.array_equal(got.view(torch.int16).numpy().view(np.uint16), want)
+    assert got[0, 0].item() == 1.0 and got[0, 1].item() == 0.0 and np.isinf(got[0, 3].item())
+    assert torch.equal(O.add_bias(x.clone(), torch.zeros(200).bfloat16()), x)
+    # leading dimensions broadcast over the last one only
+    x3 = x[:36].reshape(3, 12, 200)
+    assert torch.equal(O.add_bias(x3.clone(), b).reshape(36, 200), got[:36])
+
+
 def test_quant_input_training_outputs():
     # the transposed copy is a 128x128 block quantization: it must coincide with the block weight quantizer's
     g = torch.Generator().manual_seed(11)
