@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define MDY_FP8_ABI_VERSION 3
+#define MDY_FP8_ABI_VERSION 4
 
 /* error codes (negative = argument rejected before any launch) */
 #define MDY_OK 0
@@ -191,6 +191,28 @@ int mdy_fp8_gemm_nt_ws(const void* a, const float* a_s, int64_t as_row_stride, i
 #define MDY_PATH_TILES_SPLIT_K 4
 int mdy_fp8_gemm_path(const void* a, const void* b, int64_t as_row_stride, int64_t as_col_stride, int64_t M,
                       int64_t N, int64_t K, int with_workspace);
+
+/* mdy_fp8_gemm_nt_ws for callers that cannot allocate device memory and so cannot bring a workspace: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.
+ * Same arguments, kernels and results as mdy_fp8_gemm_nt_ws minus the workspace pair: the scratch memory is a
+ * static device array of mdy_fp8_gemm_static_workspace_bytes() (32 MiB) inside the library, which every GPU the
+ * library has run this call on holds until the process ends.  The call allocates nothing and frees nothing
+ * (no hipMalloc / hipFree, no allocating library routine).
+ *
+ *   - a shape whose mdy_fp8_gemm_workspace_bytes(M, N, K) exceeds the static buffer is rejected with MDY_E_SHAPE
+ *     (nothing launched): use mdy_fp8_gemm_nt_ws or mdy_fp8_gemm_nt for it;
+ *   - every call on a GPU shares that GPU's buffer and leaves its partial sums in it: calls that overlap in time
+ *     on one GPU (two streams, two threads) race - serialise them, or give the others their own workspace
+ *     through mdy_fp8_gemm_nt_ws.  Nothing in the buffer has to be cleared between calls;
+ *   - the buffer's device address is looked up on the first call on each device (one symbol query, no
+ *     allocation); mdy_fp8_gemm_static_workspace_init() does that lookup for the current device ahead of time,
+ *     e.g. before a stream capture begins.
+ */
+int64_t mdy_fp8_gemm_static_workspace_bytes(void);
+int mdy_fp8_gemm_static_workspace_init(void);
+int mdy_fp8_gemm_nt_static_ws(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
+                              const void* b, const float* b_s, void* c, const void* bias, int64_t M, int64_t N,
+                              int64_t K, int out_dtype, void* stream);
 
 /* Grouped (mixture-of-experts) block-scaled FP8 GEMM, NT layout: the rows of a are split into G
  * consecutive groups of m_splits[g] rows and group g is multiplied with its own weight,

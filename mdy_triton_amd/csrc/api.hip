@@ -197,6 +197,35 @@ int mdy_fp8_gemm_path(const void* a, const void* b, int64_t as_row_stride, int64
     return mdy::fp8_gemm_path(a, b, as_row_stride, as_col_stride, M, N, K, with_workspace);
 }
 
+int64_t mdy_fp8_gemm_static_workspace_bytes(void) { return mdy::kStaticScratchBytes; }
+
+int mdy_fp8_gemm_static_workspace_init(void) {
+    if (int e = check_device()) return e;
+    void* p = nullptr;
+    return launched(mdy::static_scratch_ptr(&p), "fp8_gemm_static_workspace_init");
+}
+
+int mdy_fp8_gemm_nt_static_ws(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,
+                              const float* b_s, void* c, const void* bias, int64_t M, int64_t N, int64_t K, int out_dtype,
+                              void* stream) {
+    if (out_dtype != MDY_DT_BF16 && out_dtype != MDY_DT_F32) return fail(MDY_E_DTYPE, "fp8_gemm_nt_static_ws: unknown out_dtype %d", out_dtype);
+    if (M < 0 || N < 0 || K < 1 || M > kMaxDim || N > kMaxDim || K > kMaxDim)
+        return fail(MDY_E_SHAPE, "fp8_gemm_nt_static_ws: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+    if (M == 0 || N == 0) return 0;
+    if (!a || !a_s || !b || !b_s || !c) return fail(MDY_E_NULL, "fp8_gemm_nt_static_ws: null pointer");
+    if (!aligned(c, out_dtype == MDY_DT_BF16 ? 2 : 4) || !aligned(a_s, 4) || !aligned(b_s, 4) || (bias && !aligned(bias, 2)))
+        return fail(MDY_E_ALIGN, "fp8_gemm_nt_static_ws: misaligned pointer");
+    const int64_t need = mdy::fp8_gemm_workspace_bytes(M, N, K);
+    if (need > mdy::kStaticScratchBytes)
+        return fail(MDY_E_SHAPE, "fp8_gemm_nt_static_ws: M=%lld N=%lld K=%lld needs %lld bytes of scratch, the static buffer holds %lld; "
+                    "use mdy_fp8_gemm_nt_ws with a caller-owned workspace (or mdy_fp8_gemm_nt)",
+                    (long long)M, (long long)N, (long long)K, (long long)need, (long long)mdy::kStaticScratchBytes);
+    if (int e = check_device()) return e;
+    return launched(mdy::launch_fp8_gemm_nt_static(a, a_s, as_row_stride, as_col_stride, b, b_s, c, bias, M, N, K, out_dtype,
+                                                   static_cast<hipStream_t>(stream)),
+                    "fp8_gemm_nt_static_ws");
+}
+
 int mdy_fp8_grouped_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,
                             const float* b_s, void* c, const void* bias, const int64_t* m_splits, int64_t G, int64_t N,
                             int64_t K, int out_dtype, void* stream) {

@@ -206,6 +206,12 @@ int launch_fp8_gemm_nt_ws(const void* a, const float* a_s, int64_t as_row_stride
                           int64_t K, int out_dtype, void* workspace, int64_t workspace_bytes, hipStream_t stream);
 int fp8_gemm_path(const void* a, const void* b, int64_t as_rs, int64_t as_cs, int64_t M, int64_t N, int64_t K,
                   int with_workspace);
+// static device scratch of the no-allocation GEMM entry point (defined in fp8_gemm.hip)
+constexpr int64_t kStaticScratchBytes = (int64_t)32 << 20;
+int static_scratch_ptr(void** out);
+int launch_fp8_gemm_nt_static(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
+                              const void* b, const float* b_s, void* c, const void* bias, int64_t M, int64_t N,
+                              int64_t K, int out_dtype, hipStream_t stream);
 int launch_fp8_grouped_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
                                const void* b, const float* b_s, void* c, const void* bias, const int64_t* m_splits,
                                int64_t G, int64_t M, int64_t N, int64_t K, int out_dtype, hipStream_t stream);

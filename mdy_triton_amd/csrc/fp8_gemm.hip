@@ -32,6 +32,8 @@
 // Small-M kernel (M <= 64): weight streaming, one workgroup of 8 waves per 16 columns,
 // waves split K (next block prefetched) and reduce through LDS.  Strip kernel: 5..64 rows against
 // many 128-column strips.  Scalar kernel: any other shape/alignment.
+#include <mutex>
+
 #include "common.h"
 
 namespace mdy {
@@ -1131,6 +1133,49 @@ int fp8_gemm_path(const void* a, const void* b, int64_t as_rs, int64_t as_cs, in
     if (M >= 32 && M <= 64 && big_ok && ((N + 127) / 128 >= 128 || (N + 63) / 64 >= 100)) return 3;
     if (M <= 64) return 1;
     return 3;
+}
+
+// ---------------------------------------------------------------------------
+// The workspace call for callers that cannot allocate (HIP graph capture, serving loops, harnesses that forbid
+// hipMalloc): the scratch memory is a file-scope device array of kStaticScratchBytes that every GPU the library
+// runs on holds until the process ends.  In host code the array's name is only a stand-in: its device address
+// is resolved once per device with hipGetSymbolAddress (each GPU has its own copy at its own address) and that
+// pointer, never the name, goes to the kernels.  Nothing has to start at zero: the K-split kernels write every
+// element of the slabs they use before the reduction reads them, and the scale transposition writes all of its
+// output.  All calls on one GPU share the array, so calls that overlap in time on one GPU race.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) uint8_t scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mu;
+static void* g_scratch_ptr[kMaxDevices] = {};
+
+// device address of `scratch` on the current device; resolves it on the first call per device
+int static_scratch_ptr(void** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return (int)hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (p == nullptr) return (int)hipErrorInvalidSymbol;
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
+
+int launch_fp8_gemm_nt_static(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,
+                              const float* b_s, void* c, const void* bias, int64_t M, int64_t N, int64_t K, int out_dtype,
+                              hipStream_t stream) {
+    void* ws = nullptr;
+    const int rc = static_scratch_ptr(&ws);
+    if (rc != 0) return rc;
+    return launch_fp8_gemm_nt_ws(a, a_s, as_row_stride, as_col_stride, b, b_s, c, bias, M, N, K, out_dtype, ws,
+                                 kStaticScratchBytes, stream);
 }
 
 int launch_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,
