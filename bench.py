@@ -1,13 +1,15 @@
 #!/usr/bin/env python3
 """Benchmark of the block-wise FP8 linear path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3] [--table]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3] [--table] [--ablation]
 
 One "step" is one pass of the hot path over one batch of synthetic input that is
 already resident in HBM: act_quant(X) followed by fp8_gemm(Xq, Xs, Wq, Ws) -> bf16,
 i.e. the FP8 linear forward with a pre-quantized weight.  The default workload is
 the headline shape of the benchmark definition: DeepSeek-V3 dense MLP up/gate,
 X[4096, 7168] bf16 ~ N(0,1), W[18432, 7168] e4m3fn with 128x128 fp32 block scales.
+Inputs are generated on the CPU from torch.Generator().manual_seed(config index)
+and copied to the device, so that the CPU oracle and the device see the same bits.
 
 Prints ONE JSON line on stdout:
   value        whole-step throughput in TFLOP/s (2*M*N*K / step time, quantizer included)
@@ -15,21 +17,32 @@ Prints ONE JSON line on stdout:
                duration, measured with HIP events on the launch stream inside the timed
                region, against the dense FP8 MFMA peak (a call is fp8_gemm() as a user
                makes it: the wrapper passes a scratch buffer, so at this shape the library
-               runs a 4 us scale-transposition kernel and two tile launches)
-  kernels      the same for act_quant and weight_dequant against the HBM peak
+               runs a 4 us scale-transposition kernel and two tile launches); `traffic` is
+               read from the tracked rocprofv3 summary profiles/bench_C3_hbm_traffic.txt
+  kernels      act_quant and weight_dequant of the workload against the HBM peak
                (algorithmic bytes: 3.03125*M*K and 3*N*K + 4*ceil(N/128)*ceil(K/128)),
                each timed alone, cold cache (a 512 MiB buffer is rewritten before every launch),
-               and per launch of several back-to-back launches on uncached buffers (us_streamed)
+               and per launch of several back-to-back launches on uncached buffers (us_streamed);
+               the same three kernels at the other large configurations (C2, C4; cold, one
+               event pair per launch); the six decode shapes (C5) as the per-call time of a
+               replayed HIP graph of 20 calls (the Python call is not in the number)
+  power        socket power and shader clock while the GEMM runs back to back for about a
+               second (amd-smi readings), next to the board's power cap
   cpu_baseline the CPU oracle (dequantize + fp32 matmul, torch CPU ops) on a bounded
                sample of the same workload, on the host cores of this box
 Before the W warm-up steps the script runs the same step for 50 ms (set-up, untimed): after an idle period the
 GPU needs some 20 ms of work to reach its sustained clock, whatever W is.
-With --table a per-kernel table for every benchmark configuration goes to stderr.
+With --table a per-kernel table for every benchmark configuration and for the shapes the reference
+publishes numbers for goes to stderr; with --ablation the tile kernel is timed with parts of its K loop
+switched off (mdy_fp8_gemm_probe), power and clock beside each line (stdout, no JSON).
 """
 import argparse
 import json
 import os
+import re
+import subprocess
 import sys
+import threading
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
@@ -38,21 +51,16 @@ if ROOT not in sys.path:
 
 PEAK_FP8_TFLOPS = 5000.0   # MI355X dense FP8 MFMA, published
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E, published
-
-# HBM bytes per fp8_gemm call at the C3 shape (both of its launches), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (KiB per dispatch, scaled by the same counters read on a plain copy kernel of known size); the runs are
-# summarised in profiles/bench_C3_hbm_traffic.txt: FETCH_SIZE (347 857 + 72 233) KiB x 1.9997 (copy-kernel
-# calibration) = 860.2 MB read, WRITE_SIZE (134 131 + 16 418) KiB x 1.0 = 154.2 MB written; algorithmic bytes are
-# 313 MB (the A and B panels are re-fetched by the eight XCD-local L2s).
-GEMM_C3_HBM_TRAFFIC_BYTES = 1014.4e6
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "bench_C3_hbm_traffic.txt")
 
 WORKLOADS = {
-    # name: (activation kind, M, N, K, description)
-    "C1": ("normal", 128, 1024, 1024, "CPU reference case: X[128,1024], W[1024,1024]"),
-    "C2": ("outliers", 4096, 1536, 7168, "DeepSeek-V3 attention q_a proj: X[4096,7168] (1% outliers x10), W[1536,7168]"),
-    "C3": ("normal", 4096, 18432, 7168, "DeepSeek-V3 dense MLP up/gate: X[4096,7168], W[18432,7168] (headline GEMM shape)"),
-    "C4": ("heavy", 4096, 7168, 18432, "DeepSeek-V3 dense MLP down: X[4096,18432] heavy-tailed, W[7168,18432]"),
+    # name: (seed, activation kind, M, N, K, description)
+    "C1": (1, "normal", 128, 1024, 1024, "CPU reference case: X[128,1024], W[1024,1024]"),
+    "C2": (2, "outliers", 4096, 1536, 7168, "DeepSeek-V3 attention q_a proj: X[4096,7168] (1% outliers x10), W[1536,7168]"),
+    "C3": (3, "normal", 4096, 18432, 7168, "DeepSeek-V3 dense MLP up/gate: X[4096,7168], W[18432,7168] (headline GEMM shape)"),
+    "C4": (4, "heavy", 4096, 7168, 18432, "DeepSeek-V3 dense MLP down: X[4096,18432] heavy-tailed, W[7168,18432]"),
 }
+DECODE_SHAPES = [(M, N, K) for M in (1, 16, 64) for (N, K) in ((7168, 2048), (2048, 7168))]
 
 
 def parse_args():
@@ -62,24 +70,46 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="C3", choices=sorted(WORKLOADS))
     ap.add_argument("--table", action="store_true", help="also print a per-kernel table for all configurations to stderr")
+    ap.add_argument("--ablation", action="store_true",
+                    help="time the tile kernel with parts of its K loop switched off, with power and clock (no JSON)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="only the headline workload (skip C2, C4, C5 and the power loop)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="first run one plain 256 MiB device-to-device copy kernel (counter calibration for rocprofv3 --pmc)")
     return ap.parse_args()
 
 
 def make_inputs(torch, kind, M, N, K, seed, dev):
-    """Synthetic tensors of the configuration, generated on the device (values follow the
-    benchmark definition; the parity tests use CPU-generated seeded inputs instead)."""
-    g = torch.Generator(device=dev).manual_seed(seed)
-    x = torch.randn(M, K, generator=g, device=dev)
+    """Synthetic tensors of a configuration: generated on the CPU from a seeded generator (values follow the
+    benchmark definition), then copied to the device."""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, K, generator=g)
     if kind == "outliers":
-        x = torch.where(torch.rand(M, K, generator=g, device=dev) < 0.01, x * 10, x)
+        x = torch.where(torch.rand(M, K, generator=g) < 0.01, x * 10, x)
     elif kind == "heavy":
-        x = x * torch.randn(M, K, generator=g, device=dev).abs()
+        x = x * torch.randn(M, K, generator=g).abs()
     x = x.bfloat16()
-    w = (torch.randn(N, K, generator=g, device=dev) * 0.02).bfloat16()
-    return x, w
+    w = torch.randn(N, K, generator=g).mul_(0.02).bfloat16()
+    return x.to(dev), w.to(dev)
+
+
+def quantize_weight(torch, w, dev):
+    """Block-quantize a bf16 weight once with the official-dialect quantizer (amax/448, no eps): set-up, untimed."""
+    from mdy_triton_amd import _lib
+    N, K = w.shape
+    wq = torch.empty(N, K, dtype=torch.float8_e4m3fn, device=dev)
+    ws = torch.empty((N + 127) // 128, K // 128, dtype=torch.float32, device=dev)
+    PN = (N + 127) // 128 * 128
+    if PN != N:
+        wq_p = torch.empty(PN, K, dtype=torch.float8_e4m3fn, device=dev)
+        _lib.check(_lib.load().mdy_weight_quant(w.data_ptr(), wq_p.data_ptr(), ws.data_ptr(), None, None, N, K, K, 1,
+                                                PN, K, 0, None), "weight_quant")
+        wq.copy_(wq_p[:N])
+    else:
+        _lib.check(_lib.load().mdy_weight_quant(w.data_ptr(), wq.data_ptr(), ws.data_ptr(), None, None, N, K, K, 1,
+                                                N, K, 0, None), "weight_quant")
+    torch.cuda.synchronize()
+    return wq, ws
 
 
 class ColdTimer:
@@ -135,6 +165,114 @@ def streamed_us(torch, timer, fns, reps):
     return ts[len(ts) // 2]
 
 
+def graph_replay_us(torch, fn, calls=20, reps=7):
+    """Per-call time of `fn` inside a replayed HIP graph of `calls` calls (the median of `reps` replays): kernel
+    durations plus the gaps between dependent kernels, no host launch cost."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        for _ in range(calls):
+            out = fn()
+    graph.replay()
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        ts.append(e0.elapsed_time(e1) * 1e3 / calls)
+    del out, graph
+    ts.sort()
+    return ts[len(ts) // 2]
+
+
+class SmiSampler(threading.Thread):
+    """Socket power (W) and the mean shader clock of the XCDs (MHz) from `amd-smi metric --clock --power --json`,
+    sampled in the background while a loop runs on the GPU.  Readings are best effort: no amd-smi, no samples."""
+
+    def __init__(self, period=0.1):
+        super().__init__(daemon=True)
+        self.period = period
+        self.halt = False
+        self.samples = []
+
+    @staticmethod
+    def read():
+        try:
+            r = subprocess.run(["amd-smi", "metric", "--clock", "--power", "--json"], stdout=subprocess.PIPE,
+                               stderr=subprocess.DEVNULL, text=True, timeout=5)
+            d = json.loads(r.stdout)
+            g = (d["gpu_data"] if isinstance(d, dict) else d)[0]
+            power = g["power"]["socket_power"]["value"]
+            clks = [v["clk"]["value"] for k, v in g["clock"].items() if k.startswith("gfx_") and isinstance(v, dict)
+                    and isinstance(v.get("clk"), dict) and isinstance(v["clk"].get("value"), (int, float))]
+            return float(power), (sum(clks) / len(clks) if clks else None)
+        except Exception:
+            return None
+
+    def run(self):
+        while not self.halt:
+            s = self.read()
+            if s is not None:
+                self.samples.append((time.perf_counter(),) + s)
+            time.sleep(self.period)
+
+    def summary(self, t_from):
+        rows = [s for s in self.samples if s[0] >= t_from]
+        if not rows:
+            return None
+        ps = [s[1] for s in rows]
+        cs = [s[2] for s in rows if s[2] is not None]
+        return {"socket_power_w": round(sum(ps) / len(ps), 1), "socket_power_max_w": round(max(ps), 1),
+                "gfx_clock_mhz": round(sum(cs) / len(cs), 0) if cs else None, "samples": len(rows)}
+
+
+def power_cap_w():
+    import glob
+    for f in glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_cap"):
+        try:
+            return float(open(f).read()) / 1e6
+        except (OSError, ValueError):
+            pass
+    return None
+
+
+def sustained(torch, fn, seconds=2.0, batch=10):
+    """Runs fn back to back for `seconds`; returns (us per call over the second half, amd-smi summary of the same half)."""
+    sampler = SmiSampler()
+    sampler.start()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    half = None
+    n_half = 0
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    while True:
+        now = time.perf_counter()
+        if half is None and now - t0 >= seconds / 2:
+            half = now
+            e0.record()
+        if now - t0 >= seconds:
+            break
+        for _ in range(batch):
+            fn()
+        if half is not None:
+            n_half += batch
+        torch.cuda.synchronize()
+    e1.record()
+    torch.cuda.synchronize()
+    sampler.halt = True
+    sampler.join()
+    us = e0.elapsed_time(e1) * 1e3 / max(n_half, 1)
+    return us, sampler.summary(half)
+
+
 def cpu_baseline(torch, kind, M, N, K, xq, xs, wq, ws):
     """The CPU oracle (dequantize activations + dequantize weights + fp32 matmul -> bf16) on a
     bounded sample: `rows` activation rows (all of them up to 4096) against the full weight,
@@ -173,7 +311,62 @@ def cpu_baseline(torch, kind, M, N, K, xq, xs, wq, ws):
                    "fp32 matmul %.2f s; row-proportional parts extrapolated to %d rows -> %.1f s per step; cpu: %s"
                    % (rows, M, N, K, t_w, t_a, t_mm, M, full, model)),
         "checksum": float(c.float().abs().mean()),
+    }, c
+
+
+def traffic_from_profile():
+    """HBM-side bytes of one fp8_gemm call at the C3 shape, from the line `fp8_gemm_call_traffic_bytes <n>` of the
+    tracked rocprofv3 summary (FETCH_SIZE + WRITE_SIZE of the call's launches, calibrated on a copy kernel)."""
+    try:
+        m = re.search(r"^fp8_gemm_call_traffic_bytes\s+([0-9.eE+]+)", open(TRAFFIC_PROFILE).read(), re.M)
+        return float(m.group(1)) if m else None
+    except OSError:
+        return None
+
+
+def gemm_bytes(M, N, K):
+    return M * K + N * K + 4 * M * (K // 128) + 4 * ((N + 127) // 128) * (K // 128) + 2 * M * N
+
+
+def kernel_entries(torch, m, timer, x, wq, ws, reps=12):
+    """act_quant / weight_dequant / fp8_gemm of one configuration, cold cache, one event pair per launch."""
+    M, K = x.shape
+    N = wq.size(0)
+    xq, xs = m.act_quant(x)
+    aq_us, _ = timer.run(lambda: m.act_quant(x), reps)
+    wd_us, _ = timer.run(lambda: m.weight_dequant(wq, ws, out_dtype=torch.bfloat16), reps)
+    g_us, _ = timer.run(lambda: m.fp8_gemm(xq, xs, wq, ws, out_dtype=torch.bfloat16), reps)
+    aq_b = 3.03125 * M * K
+    wd_b = 3.0 * N * K + 4.0 * ((N + 127) // 128) * (K // 128)
+    fl = 2.0 * M * N * K
+    return {
+        "act_quant": {"us": round(aq_us, 2), "GB/s": round(aq_b / aq_us / 1e3, 1),
+                      "frac_hbm_peak": round(aq_b / aq_us / 1e3 / PEAK_HBM_GBS, 4)},
+        "weight_dequant": {"us": round(wd_us, 2), "GB/s": round(wd_b / wd_us / 1e3, 1),
+                           "frac_hbm_peak": round(wd_b / wd_us / 1e3 / PEAK_HBM_GBS, 4)},
+        "fp8_gemm": {"us": round(g_us, 2), "TFLOP/s": round(fl / g_us / 1e6, 1),
+                     "frac_mfma_peak": round(fl / g_us / 1e6 / PEAK_FP8_TFLOPS, 4)},
     }
+
+
+def decode_entries(torch, m, dev):
+    """The six decode / routed-expert shapes: per-call time inside a replayed HIP graph, against the HBM peak on the
+    algorithmic bytes (weights + activations + scales + output).  The weights (14.7 MB) stay in the caches between
+    the calls of a graph, so this is the kernel's speed, not a cold-memory figure."""
+    out = {}
+    for i, (M, N, K) in enumerate(DECODE_SHAPES):
+        g = torch.Generator().manual_seed(50 + i)
+        x = torch.randn(M, K, generator=g).bfloat16().to(dev)
+        w = torch.randn(N, K, generator=g).mul_(0.02).bfloat16().to(dev)
+        wq, ws = quantize_weight(torch, w, dev)
+        xq, xs = m.act_quant(x)
+        us = graph_replay_us(torch, lambda: m.fp8_gemm(xq, xs, wq, ws, out_dtype=torch.bfloat16))
+        aq_us = graph_replay_us(torch, lambda: m.act_quant(x))
+        b = gemm_bytes(M, N, K)
+        out["M=%d,N=%d,K=%d" % (M, N, K)] = {"fp8_gemm_us": round(us, 2), "GB/s": round(b / us / 1e3, 1),
+                                              "frac_hbm_peak": round(b / us / 1e3 / PEAK_HBM_GBS, 4),
+                                              "act_quant_us": round(aq_us, 2)}
+    return out
 
 
 def main():
@@ -187,20 +380,17 @@ def main():
         print("bench.py needs a GPU (torch.cuda.is_available() is False)", file=sys.stderr)
         sys.exit(2)
     import mdy_triton_amd as m
-    from mdy_triton_amd.fp8 import quant_weight  # noqa: F401  (weight side is prepared once, untimed)
     from oracle import oracle as O
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    kind, M, N, K, desc = WORKLOADS[args.workload]
-    x, w = make_inputs(torch, kind, M, N, K, 0, dev)
-    # weight: block-quantized once with the official-dialect quantizer (amax/448, no eps)
-    wq = torch.empty(N, K, dtype=torch.float8_e4m3fn, device=dev)
-    ws = torch.empty((N + 127) // 128, K // 128, dtype=torch.float32, device=dev)
-    from mdy_triton_amd import _lib
-    _lib.check(_lib.load().mdy_weight_quant(w.data_ptr(), wq.data_ptr(), ws.data_ptr(), None, None, N, K, K, 1,
-                                            N, K, 0, None), "weight_quant")
-    torch.cuda.synchronize()
+    if args.ablation:
+        ablation(torch, m, dev)
+        return
+    seed, kind, M, N, K, desc = WORKLOADS[args.workload]
+    x, w = make_inputs(torch, kind, M, N, K, seed, dev)
+    wq, ws = quantize_weight(torch, w, dev)
+    del w
 
     def step():
         xq, xs = m.act_quant(x)
@@ -253,14 +443,6 @@ def main():
     aq_bytes = 3.03125 * M * K
     wd_bytes = 3.0 * N * K + 4.0 * ((N + 127) // 128) * (K // 128)
 
-    # ---- parity spot check of this very run against the oracle (a few rows)
-    rows = torch.tensor([0, M // 2, M - 1])
-    ref = O.fp8_gemm(xq[rows.to(dev)].cpu(), xs[rows.to(dev)].cpu(), wq.cpu(), ws.cpu(), dtype=torch.bfloat16)
-    parity_ok = bool(torch.allclose(out[rows.to(dev)].float().cpu(), ref.float(), rtol=1e-2, atol=1e-2))
-    yq_ref, s_ref = O.act_quant(x[rows.to(dev)].cpu())
-    parity_ok = parity_ok and bool(torch.equal(xq[rows.to(dev)].cpu().view(torch.uint8), yq_ref.view(torch.uint8))) \
-        and bool(torch.equal(xs[rows.to(dev)].cpu(), s_ref))
-
     achieved = flops / (gemm_us * 1e-6) / 1e12
     result = {
         "metric": "fp8_gemm TFLOPS + % FP8 MFMA peak; act_quant/dequant GB/s + % HBM, 1 GPU",
@@ -274,7 +456,7 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "fp8_e4m3fn x fp8_e4m3fn -> fp32 accumulate -> bf16",
-        "data": "synthetic",
+        "data": "synthetic (CPU-seeded, copied to the device)",
         "config": {"workload": "%s %s; step = act_quant + fp8_gemm (pre-quantized weight)" % (args.workload, desc),
                    "M": M, "N": N, "K": K},
         "roofline": {"bound": "mfma",
@@ -283,7 +465,7 @@ def main():
                      "achieved": round(achieved, 2), "peak": PEAK_FP8_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP8_TFLOPS, 4),
                      "launch_us": round(gemm_us, 2), "flops_per_launch": flops,
-                     "traffic": GEMM_C3_HBM_TRAFFIC_BYTES if args.workload == "C3" else None},
+                     "traffic": traffic_from_profile() if args.workload == "C3" else None},
         "kernels": {
             "fp8_gemm_cold": {"us": round(gemm_cold_us, 2), "TFLOP/s": round(flops / gemm_cold_us / 1e6, 2),
                               "frac_mfma_peak": round(flops / gemm_cold_us / 1e6 / PEAK_FP8_TFLOPS, 4)},
@@ -298,19 +480,93 @@ def main():
                                "us_streamed": round(wd_stream_us, 2),
                                "frac_hbm_peak_streamed": round(wd_bytes / wd_stream_us / 1e3 / PEAK_HBM_GBS, 4)},
         },
-        "parity_spot_check": parity_ok,
     }
     # the same peak derived from the device the run is on: CUs x 4 SIMDs x 2048 FP8 flop per clock x max clock
     props = torch.cuda.get_device_properties(dev)
     clock_khz = getattr(props, "clock_rate", 0) or 2400000      # MI355X: 2.4 GHz peak engine clock
     result["roofline"]["peak_from_device_props"] = round(props.multi_processor_count * 4 * 2048 * clock_khz * 1e3 / 1e12, 1)
     result["roofline"]["device"] = "%s, %d CUs, %.2f GHz" % (props.name, props.multi_processor_count, clock_khz / 1e6)
+
+    if not args.no_extra:
+        # power and clock while the dominant kernel runs back to back (what bounds it: see the power cap beside it)
+        us, smi = sustained(torch, lambda: m.fp8_gemm(xq, xs, wq, ws, out_dtype=torch.bfloat16))
+        result["power"] = {"loop": "fp8_gemm %s back to back for 2 s, second half" % args.workload,
+                           "gemm_us": round(us, 1), "power_cap_w": power_cap_w()}
+        if smi:
+            result["power"].update(smi)
+
+    # ---- parity of this very run against the oracle: act_quant bit-exact on sampled rows, GEMM on the CPU leg's rows
+    rows = torch.tensor([0, M // 2, M - 1])
+    yq_ref, s_ref = O.act_quant(x[rows.to(dev)].cpu())
+    parity_ok = bool(torch.equal(xq[rows.to(dev)].cpu().view(torch.uint8), yq_ref.view(torch.uint8))) \
+        and bool(torch.equal(xs[rows.to(dev)].cpu(), s_ref))
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(torch, kind, M, N, K, xq, xs, wq, ws)
+        result["cpu_baseline"], c_ref = cpu_baseline(torch, kind, M, N, K, xq, xs, wq, ws)
+        got = out[:c_ref.size(0)].float().cpu()
+        parity_ok = parity_ok and bool(torch.allclose(got, c_ref.float(), rtol=1e-2, atol=1e-2))
+        result["parity_rows_checked"] = int(c_ref.size(0))
+        del c_ref, got
+    else:
+        ref = O.fp8_gemm(xq[rows.to(dev)].cpu(), xs[rows.to(dev)].cpu(), wq.cpu(), ws.cpu(), dtype=torch.bfloat16)
+        parity_ok = parity_ok and bool(torch.allclose(out[rows.to(dev)].float().cpu(), ref.float(), rtol=1e-2, atol=1e-2))
+        result["parity_rows_checked"] = 3
+    result["parity_spot_check"] = parity_ok
+
+    if not args.no_extra:
+        del out, xq, xs
+        for name in ("C2", "C3", "C4"):
+            if name == args.workload:
+                continue
+            s2, k2, M2, N2, K2, _ = WORKLOADS[name]
+            x2, w2 = make_inputs(torch, k2, M2, N2, K2, s2, dev)
+            wq2, ws2 = quantize_weight(torch, w2, dev)
+            del w2
+            result["kernels"][name] = kernel_entries(torch, m, timer, x2, wq2, ws2)
+            result["kernels"][name]["shape"] = {"M": M2, "N": N2, "K": K2}
+            del x2, wq2, ws2
+        result["kernels"]["C5_graph_replay"] = decode_entries(torch, m, dev)
 
     if args.table:
         table(torch, m, timer, dev)
     print(json.dumps(result))
+
+
+def ablation(torch, m, dev):
+    """The tile kernel with parts of its K loop switched off, each variant run back to back for ~1.5 s on the
+    product's own operands; per launch: time, the rate the same FLOPs would mean, socket power, shader clock."""
+    from mdy_triton_amd import _lib
+    L = _lib.load()
+    names = {0: "full kernel (the product)", 8: "no pre-touches", 4: "no FMA fold (MFMAs accumulate in place)",
+             2: "no LDS fragment reads", 1: "no global->LDS copies (ring replayed)", 5: "no copies, no fold",
+             3: "no copies, no LDS reads", 7: "MFMA only (no copies, no LDS reads, no fold)"}
+    cap = power_cap_w()
+    print("power cap %s W; idle reading: %s" % (cap, SmiSampler.read()))
+    for tile, (label, wl, N_use) in enumerate((("256x256 tiles", "C3", 16384), ("128x256 tiles", "C2", 2048))):
+        seed, kind, M, N, K, _ = WORKLOADS[wl]
+        N = N_use
+        x, w = make_inputs(torch, kind, M, N, K, seed, dev)
+        wq, ws = quantize_weight(torch, w, dev)
+        xq, xs = m.act_quant(x)
+        xst = xs.t().contiguous()              # [K/128, M]: the layout the tile kernel is given by fp8_gemm
+        c = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+        for const in (False, True):
+            a_op, b_op = xq, wq
+            if const:       # every operand byte 0x38 (= 1.0): no data toggling in the matrix cores
+                a_op = torch.full_like(xq.view(torch.uint8), 0x38).view(torch.float8_e4m3fn)
+                b_op = torch.full_like(wq.view(torch.uint8), 0x38).view(torch.float8_e4m3fn)
+            bm = 256 if tile == 0 else 128
+            print("%s, M=%d N=%d K=%d (%d tiles), %s operands" % (label, M, N, K, ((M + bm - 1) // bm) * ((N + 255) // 256),
+                                                               "constant" if const else "quantized N(0,1) x N(0,0.02)"))
+            for abl in ((0, 8, 4, 2, 1, 5, 3, 7) if not const else (0, 7)):
+                def fn(abl=abl):
+                    _lib.check(L.mdy_fp8_gemm_probe(tile, abl, a_op.data_ptr(), xst.data_ptr(), 1, M, b_op.data_ptr(),
+                                                    ws.data_ptr(), c.data_ptr(), M, N, K, None), "probe")
+                us, smi = sustained(torch, fn, seconds=1.5)
+                smi = smi or {}
+                print("  %-46s %8.1f us  %7.1f TFLOP/s-equivalent (%4.1f %% of peak)   %6s W   %5s MHz" % (
+                    names[abl], us, 2.0 * M * N * K / us / 1e6, 2.0 * M * N * K / us / 1e6 / PEAK_FP8_TFLOPS * 100,
+                    smi.get("socket_power_w"), smi.get("gfx_clock_mhz")), flush=True)
+        del x, w, wq, ws, xq, xs, xst, c
 
 
 def table(torch, m, timer, dev):
@@ -321,8 +577,8 @@ def table(torch, m, timer, dev):
         rate = work / us / (1e6 if unit == "TFLOP/s" else 1e3)
         print("%-46s %9.1f us %10.2f %-8s %5.1f %% of peak" % (name, us, rate, unit, 100 * rate / peak), file=sys.stderr)
 
-    for name, (kind, M, N, K, _) in WORKLOADS.items():
-        x, w = make_inputs(torch, kind, M, N, K, 1, dev)
+    for name, (seed, kind, M, N, K, _) in WORKLOADS.items():
+        x, w = make_inputs(torch, kind, M, N, K, seed, dev)
         wq, ws, _, _ = m.quant_weight(w)
         xq, xs = m.act_quant(x)
         line("%s act_quant %dx%d" % (name, M, K), timer.run(lambda: m.act_quant(x), 20)[0], 3.03125 * M * K, "GB/s", PEAK_HBM_GBS)
@@ -330,14 +586,35 @@ def table(torch, m, timer, dev):
              3.0 * N * K + 4.0 * ((N + 127) // 128) * (K // 128), "GB/s", PEAK_HBM_GBS)
         line("%s fp8_gemm %dx%dx%d" % (name, M, N, K), timer.run(lambda: m.fp8_gemm(xq, xs, wq, ws, out_dtype=torch.bfloat16), 10)[0],
              2.0 * M * N * K, "TFLOP/s", PEAK_FP8_TFLOPS)
+    # ---- the shapes the reference publishes numbers for (H800 there; same shapes, this GPU, same cold-cache protocol)
+    xr = torch.randn(16384, 4096, device=dev).bfloat16()
+    line("ref act_quant 16384x4096 (fp8-benchmark.ipynb:141)", timer.run(lambda: m.act_quant(xr), 20)[0], 3.03125 * 16384 * 4096, "GB/s", PEAK_HBM_GBS)
+    del xr
+    for (Mr, Nr, Kr) in ((8192, 8192, 8192), (16384, 4096, 4096), (16384, 4096, 7168), (16384, 4096, 16384)):
+        lin = m.DeepLinear(Kr, Nr, bias=False, dtype=torch.bfloat16, device=dev)
+        lin.cache_weight = True
+        xg = torch.randn(Mr, Kr, device=dev).bfloat16().requires_grad_(True)
+        dy = torch.randn(Mr, Nr, device=dev).bfloat16()
+        with torch.no_grad():
+            line("ref DeepLinear fwd %dx%dx%d (test_fp8.ipynb:169)" % (Mr, Nr, Kr), timer.run(lambda: lin(xg), 8)[0],
+                 2.0 * Mr * Nr * Kr, "TFLOP/s", PEAK_FP8_TFLOPS)
+
+        def fwd_bwd():
+            lin.zero_grad(set_to_none=True)
+            xg.grad = None
+            lin(xg).backward(dy)
+        line("ref DeepLinear fwd+bwd %dx%dx%d (test_fp8.ipynb:172)" % (Mr, Nr, Kr), timer.run(fwd_bwd, 6)[0],
+             6.0 * Mr * Nr * Kr, "TFLOP/s", PEAK_FP8_TFLOPS)
+        del lin, xg, dy
     # training-time operators at the C3 shapes (DeepLinear dialect): bytes = 2 in + 1 out + 1 transposed out per element
-    kind, M, N, K, _ = WORKLOADS["C3"]
-    x, w = make_inputs(torch, kind, M, N, K, 2, dev)
+    seed, kind, M, N, K, _ = WORKLOADS["C3"]
+    x, w = make_inputs(torch, kind, M, N, K, seed, dev)
     dy = torch.randn(M, N, device=dev, dtype=torch.bfloat16)
     line("C3 quant_input(train) %dx%d" % (M, K), timer.run(lambda: m.quant_input(x, False), 20)[0], 4.0 * M * K, "GB/s", PEAK_HBM_GBS)
     line("C3 quant_grad_output %dx%d" % (M, N), timer.run(lambda: m.quant_grad_output(dy), 20)[0], 4.0 * M * N, "GB/s", PEAK_HBM_GBS)
     line("C3 quant_weight(train) %dx%d" % (N, K), timer.run(lambda: m.quant_weight(w, False), 20)[0], 4.0 * N * K, "GB/s", PEAK_HBM_GBS)
     lin = m.DeepLinear(K, N, bias=False, dtype=torch.bfloat16, device=dev)
+    lin.cache_weight = True
     xg = x.clone().requires_grad_(True)
 
     def train_step():
@@ -387,19 +664,19 @@ def table(torch, m, timer, dev):
     us = timer.run(lambda: m.fp8_grouped_matmul(aq, asg, bq[:Gr], bsg[:Gr], [mr] * Gr), 10)[0]
     line("grouped fp8_gemm %d experts x %d rows, N=%d K=%d" % (Gr, mr, Ng, Kg), us, 2.0 * Gr * mr * Ng * Kg, "TFLOP/s", PEAK_FP8_TFLOPS)
     del bq, bsg, aq, asg
-    for M in (1, 16, 64):
-        for (N, K) in ((7168, 2048), (2048, 7168)):
-            a = torch.randint(0, 120, (M, K), dtype=torch.uint8, device=dev).view(FP8)
-            b = torch.randint(0, 120, (N, K), dtype=torch.uint8, device=dev).view(FP8)
-            a_s = torch.rand(M, K // 128, device=dev)
-            b_s = torch.rand(N // 128, K // 128, device=dev)
-            byts = M * K + N * K + 4 * M * K / 128 + 4 * (N // 128) * (K // 128) + 2 * M * N
+    for (M, N, K) in DECODE_SHAPES:
+        a = torch.randint(0, 120, (M, K), dtype=torch.uint8, device=dev).view(FP8)
+        b = torch.randint(0, 120, (N, K), dtype=torch.uint8, device=dev).view(FP8)
+        a_s = torch.rand(M, K // 128, device=dev)
+        b_s = torch.rand(N // 128, K // 128, device=dev)
 
-            def many():
-                for _ in range(20):
-                    m.fp8_gemm(a, a_s, b, b_s, out_dtype=torch.bfloat16)
-            us = timer.run(many, 10, cold=False)[0] / 20
-            line("C5 fp8_gemm M=%d N=%d K=%d (warm, back-to-back)" % (M, N, K), us, byts, "GB/s", PEAK_HBM_GBS)
+        def many():
+            for _ in range(20):
+                m.fp8_gemm(a, a_s, b, b_s, out_dtype=torch.bfloat16)
+        us = timer.run(many, 10, cold=False)[0] / 20
+        line("C5 fp8_gemm M=%d N=%d K=%d (warm, back-to-back, Python calls)" % (M, N, K), us, gemm_bytes(M, N, K), "GB/s", PEAK_HBM_GBS)
+        us = graph_replay_us(torch, lambda: m.fp8_gemm(a, a_s, b, b_s, out_dtype=torch.bfloat16))
+        line("   the same inside a replayed HIP graph", us, gemm_bytes(M, N, K), "GB/s", PEAK_HBM_GBS)
     # few rows against a long K (small-batch prefill / large-batch decode): tiles do not fill the GPU, the
     # wrapper hands the library a workspace and the shape is split along K; weight bytes bound these
     for (M, N, K) in ((128, 7168, 16384), (128, 2112, 7168), (256, 7168, 18432), (512, 4096, 7168)):
@@ -407,7 +684,7 @@ def table(torch, m, timer, dev):
         b = torch.randint(0, 120, (N, K), dtype=torch.uint8, device=dev).view(FP8)
         a_s = torch.rand(M, K // 128, device=dev)
         b_s = torch.rand((N + 127) // 128, K // 128, device=dev)
-        byts = M * K + N * K + 4 * M * K / 128 + 4 * ((N + 127) // 128) * (K // 128) + 2 * M * N
+        byts = gemm_bytes(M, N, K)
         us = timer.run(lambda: m.fp8_gemm(a, a_s, b, b_s, out_dtype=torch.bfloat16), 10)[0]
         line("fp8_gemm M=%d N=%d K=%d (split along K)" % (M, N, K), us, byts, "GB/s", PEAK_HBM_GBS)
         us = timer.run(lambda: m.fp8_gemm(a, a_s, b, b_s, out_dtype=torch.bfloat16), 10, cold="read")[0]

@@ -1,0 +1,402 @@
+// The MFMA tile body of the block-scaled FP8 GEMM and the kernel that walks tiles with it (gfx950 only).
+// Shared by fp8_gemm.hip (the product kernels) and gemm_probe.hip (the timing probe that switches parts of the
+// K loop off); the description of the kernel is at the top of fp8_gemm.hip.
+#pragma once
+#include "common.h"
+
+namespace mdy {
+
+// chunk swizzle of an LDS row; depends on row bits 0..3 only so that rows 16 apart share it
+__device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+// One 128-deep scale block of a 16x16 sub-tile, from zero: v_mfma_f32_16x16x128_f8f6f4 with e4m3 operands and unit
+// hardware scales.  The weight rows go in as the MFMA's rows and the activation rows as its columns, so a lane's
+// four results are four consecutive n of one m.
+__device__ __forceinline__ floatx4 mfma_block(const intx8& weight_rows, const intx8& act_rows) {
+    const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(weight_rows, act_rows, zero, 0, 0, 0, 0, 0, 0);
+}
+
+// The promotion of one K block (offical_kernel.py:86): acc += (MFMA result of the block) * (its combined scale).
+__device__ __forceinline__ void fold(floatx4& acc, const floatx4& p, float sc) {
+    acc[0] = __builtin_fmaf(p[0], sc, acc[0]);
+    acc[1] = __builtin_fmaf(p[1], sc, acc[1]);
+    acc[2] = __builtin_fmaf(p[2], sc, acc[2]);
+    acc[3] = __builtin_fmaf(p[3], sc, acc[3]);
+}
+
+template <typename OUT>
+__device__ __forceinline__ void store4(OUT* c, int64_t ldc, int m, int n, int M, int N, const float (&v)[4], bool vec_ok) {
+    if (m >= M || n >= N) return;
+    OUT* p = c + (int64_t)m * ldc + n;
+    if (vec_ok && n + 3 < N) {
+        // plain (cached) stores: the 8-byte pieces of a line written by different instructions are
+        // merged in L2; non-temporal stores measured ~5 % slower here
+        if (sizeof(OUT) == 2) {
+            *reinterpret_cast<uint2*>(p) = make_uint2(pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]));
+        } else {
+            *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (n + i < N) {
+                if (sizeof(OUT) == 2)
+                    reinterpret_cast<uint16_t*>(p)[i] = (uint16_t)(pack2_bf16(v[i], 0.0f) & 0xFFFFu);
+                else
+                    reinterpret_cast<float*>(p)[i] = v[i];
+            }
+        }
+    }
+}
+
+// raw buffer descriptor: base, byte range, no stride, no swizzle
+__device__ __forceinline__ intx4 make_rsrc(const void* base, uint32_t bytes) {
+    const uint64_t p = reinterpret_cast<uint64_t>(base);
+    intx4 r;
+    r[0] = (int)(uint32_t)p;
+    r[1] = (int)((uint32_t)(p >> 32) & 0xFFFFu);
+    r[2] = (int)bytes;
+    r[3] = 0x00020000;
+    return r;
+}
+__device__ __forceinline__ uint32_t lds_addr(const void* p) {
+    return (uint32_t)(uintptr_t)((__attribute__((address_space(3))) const void*)p);
+}
+// 64 lanes x 16 bytes, global (descriptor base + voff + soff) -> LDS (lds + lane*16).
+// Issued as inline asm so that the copy stays asynchronous: the kernel waits for it
+// with an explicit s_waitcnt vmcnt + barrier once per K block, nowhere else.
+// rsrc, soff and lds must be wave-uniform.
+__device__ __forceinline__ void dma16(const intx4& rsrc, int voff, int soff, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
+                 :: "v"(voff), "s"(rsrc), "s"(soff), "s"(lds) : "memory");
+}
+__device__ __forceinline__ void dma4(const intx4& rsrc, int voff, int soff, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dword %0, %1, %2 offen lds"
+                 :: "v"(voff), "s"(rsrc), "s"(soff), "s"(lds) : "memory");
+}
+
+// Shares of the panel pre-touches: the A panel of a tile row is cut into 2^a_sh shares among the tiles of
+// that row that run side by side, the B panel of a tile column into 2^b_sh shares among its tile rows.
+struct Duty {
+    int a_duty, a_sh, b_duty, b_sh;
+};
+
+// LDS of one tile workgroup, carved out of a pool that the kernel declares: the ring of A and B panels, the ring of activation scales, the tile's weight
+// scales for all K blocks, and a dummy area for copies that must go nowhere.
+template <int BM, int BN, int WAVES, int STAGES>
+struct TileLds {
+    static constexpr int NBS = (BN + 127) / 128;
+    static constexpr int a_off = 0;
+    static constexpr int b_off = a_off + STAGES * BM * 128;
+    static constexpr int s_off = b_off + STAGES * BN * 128;
+    static constexpr int bs_off = s_off + (STAGES * BM * 4 + 255) / 256 * 256;
+    static constexpr int dummy_off = bs_off + NBS * 512 * 4;
+    static constexpr int bytes = dummy_off + WAVES * 512;
+};
+
+// One BM x BN tile of C: WGM x WGN waves, each wave (BM/WGM) x (BN/WGN).
+//   rows m0 .. min(m0+BM, m_end) of a (m_end = end of the matrix, or of the expert group the tile belongs to),
+//   columns n0 .. of b / b_s / bias (already offset to the group's weight), K % 128 == 0, K <= 65536,
+//   K blocks kb0 .. kb1-1 of them (all of them except in the split-K kernel).
+// as_bytes = byte size of the addressed part of a_s (host computed, < 2^31); m_total = rows of a_s.
+// duty: which share of the A / B panel lines this workgroup pre-touches for the workgroups that copy the same
+// panels (those with the same tile row / tile column), and into how many shares the panels are cut.
+//
+// Schedule of one K block (NT = TI*TJ MFMA slots, each followed DEPTH slots later by its 4 FMAs):
+//   slots 0..      the last copies of K block kb+1 (those that did not fit into the tail below), one per GAP
+//                  slots, then one "duty touch" load for K block kb+3;
+//   slot TB        = first MFMA of the last streamed fragment: every LDS read of this K block has been
+//                  consumed, so the wave waits for its copies of kb+1 and meets the others at THE barrier
+//                  of the K block; behind it buffer `cur` is free and buffer `cur^1` is complete;
+//   slots TB..     while the last MFMAs and FMAs of kb still run: reload the held fragments, the first
+//                  streamed fragment and the scales from buffer cur^1, and issue the first copies of kb+2
+//                  into buffer cur, one per GAP slots.
+// So the LDS latency after the barrier and the issue time of the copies sit in the shadow of the matrix
+// pipe instead of in front of the first MFMA of the next K block.
+template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT, int GAP_ = 0, int TD_ = 0, int ABL_ = 0>
+__device__ __forceinline__ void fp8_gemm_tile(
+    const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
+    const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
+    const uint16_t* __restrict__ bias, int m0, int m_end, int m_total, int n0, int N, int K, int ldc, const Duty duty,
+    int kb0, int kb1, uint8_t* __restrict__ pool) {
+    // ABL_ switches parts of the K loop off for the timing probe (mdy_fp8_gemm_probe); the product uses 0.
+    //   1: no global->LDS copies in the loop (the ring is filled once and replayed)   2: no LDS fragment / scale reads
+    //   4: no FMA fold (the MFMAs accumulate in place, no block scales)                8: no pre-touches
+    constexpr bool NO_COPY = (ABL_ & 1) != 0, NO_LDS = (ABL_ & 2) != 0, NO_FOLD = (ABL_ & 4) != 0;
+    constexpr bool NO_TOUCH = (ABL_ & 8) != 0 || NO_COPY;
+    constexpr int WAVES = WGM * WGN;
+    constexpr int WM = BM / WGM, WN = BN / WGN, TI = WM / 16, TJ = WN / 16;
+    constexpr int PASS_ROWS = WAVES * 8;  // rows copied by one DMA instruction of every wave
+    constexpr int A_PASSES = BM / PASS_ROWS, B_PASSES = BN / PASS_ROWS;
+    constexpr int S_WAVES = BM / 64;      // waves that also copy the activation scales
+    constexpr int DEPTH = 4;              // MFMAs in flight before their results are folded
+    static_assert(BM % PASS_ROWS == 0 && BN % PASS_ROWS == 0 && PASS_ROWS % 16 == 0, "tile/threads mismatch");
+    static_assert(WN <= 128 && 128 % WN == 0 && S_WAVES <= WAVES && WAVES >= 2, "one weight-scale block per wave column");
+    constexpr bool HOLD_A = TI <= TJ;
+    constexpr int NH = HOLD_A ? TI : TJ, NS = HOLD_A ? TJ : TI;
+    constexpr int NT = TI * TJ;
+    constexpr int NDMA = 1 + A_PASSES + B_PASSES;       // copies per K block and wave: scales, A passes, B passes
+    constexpr int TB = NT - NH;                         // slot of the barrier
+    constexpr int NSLOT = NT + DEPTH;                   // slots of a K block (the last DEPTH hold FMAs only)
+    // Copy j of a K block goes out in slot TB+1 + GAP*j, counted on from the barrier of the block two before it
+    // and running over into the first slots of the next block.  With 8 waves one copy per slot and wave is
+    // twice what the CU's address unit takes (64 lanes x 16 bytes = 16 clocks each, a slot is 64 clocks for
+    // the two waves of a SIMD): the waves then queue on the copy instruction and their MFMAs behind it wait.
+    // Measured: 256x256 tiles 1-5 % faster with every second slot, 128x256 tiles (half as many slots) not.
+    constexpr int GAP = GAP_ > 0 ? GAP_ : (WAVES >= 8 && NT >= 32) ? 2 : 1;
+    constexpr int TAIL = (NSLOT - TB - 1 + GAP - 1) / GAP;   // copies that still fit behind the barrier
+    constexpr int FIRST = TAIL < NDMA ? TAIL : NDMA;         // copies of K block kb+2 issued in the tail of kb
+    constexpr int TOUCH = FIRST < NDMA ? TB + 1 + GAP * (NDMA - 1) - NSLOT + 1 : 0;   // slot after the last copy
+    constexpr int TD = TD_ > 0 ? TD_ : STAGES + 1;      // duty touches run this many K blocks ahead (in front of the copies)
+    // loads younger than the last copy of K block kb+1 when the wave waits for it in K block kb: the copies of
+    // blocks kb+2 .. kb+STAGES-1 and one touch per K block since (loads complete in order, so vmcnt(YOUNGER)
+    // means "block kb+1 has landed")
+    constexpr int YOUNGER = (STAGES - 2) * NDMA + STAGES - 1;
+    static_assert(STAGES >= 2 && YOUNGER <= 63, "vmcnt is a 6-bit counter");
+    static_assert(NS % 2 == 0 && NS >= 2, "the first streamed fragment of the next K block reuses queue slot 0");
+    static_assert(TOUCH < TB, "not enough slots in front of the barrier");
+
+    using L = TileLds<BM, BN, WAVES, STAGES>;
+    constexpr int NBS = L::NBS;
+    uint8_t(*lds_a)[BM * 128] = reinterpret_cast<uint8_t(*)[BM * 128]>(pool + L::a_off);     // [STAGES]
+    uint8_t(*lds_b)[BN * 128] = reinterpret_cast<uint8_t(*)[BN * 128]>(pool + L::b_off);     // [STAGES]
+    float(*lds_s)[BM] = reinterpret_cast<float(*)[BM]>(pool + L::s_off);                      // [STAGES]
+    float(*lds_bs)[512] = reinterpret_cast<float(*)[512]>(pool + L::bs_off);                  // [NBS] weight scales, all K blocks
+    uint8_t* lds_dummy = pool + L::dummy_off;                                                 // target of copies that must go nowhere
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int M = m_end;
+    const int KB = K >> 7;
+
+    // ---- DMA: descriptors limited to the rows of this tile, so that the M and N tails read 0
+    const intx4 ra = make_rsrc(a + (size_t)m0 * K, (uint32_t)min(BM, M - m0) * (uint32_t)K);
+    const intx4 rb = make_rsrc(b + (size_t)n0 * K, (uint32_t)min(BN, N - n0) * (uint32_t)K);
+    intx4 rs = make_rsrc(a_s, as_bytes);
+    if (wave >= S_WAVES) rs[2] = 0;                                   // these waves copy no scales: always out of range
+    const int prow = wave * 8 + (lane >> 3);                          // row inside a pass
+    const int voff = prow * K + (((lane & 7) ^ swz(prow)) << 4);      // permuted chunk of that row
+    const int s_voff = min(m0 + (wave % S_WAVES) * 64 + lane, m_total - 1) * as_rs * 4;
+    const uint32_t ld_base = lds_addr(&lds_dummy[0]) + wave * 512;
+    const uint32_t la_base = lds_addr(&lds_a[0][0]) + wave * 1024;
+    const uint32_t lb_base = lds_addr(&lds_b[0][0]) + wave * 1024;
+    const uint32_t ls_base = wave < S_WAVES ? lds_addr(&lds_s[0][0]) + wave * 256 : ld_base;
+    const uint32_t ls_buf = wave < S_WAVES ? BM * 4 : 0;
+
+    // copy i (0: scales, then the A passes, then the B passes) of K block kb into buffer buf.  Past the last K
+    // block the offsets run beyond the descriptors: no memory access, zeros into a buffer nobody reads any more.
+    auto issue = [&](int i, int kb, int buf) {
+        const bool more = kb < kb1;
+        if (i == 0)
+            dma4(rs, s_voff, more ? kb * as_cs * 4 : (int)as_bytes, ls_base + buf * ls_buf);
+        else if (i <= A_PASSES)
+            dma16(ra, voff, (i - 1) * PASS_ROWS * K + (more ? kb * 128 : ra[2]), la_base + buf * (BM * 128) + (i - 1) * PASS_ROWS * 128);
+        else
+            dma16(rb, voff, (i - 1 - A_PASSES) * PASS_ROWS * K + (more ? kb * 128 : rb[2]),
+                  lb_base + buf * (BN * 128) + (i - 1 - A_PASSES) * PASS_ROWS * 128);
+    };
+    // duty touch: the even waves load one dword of every line of this workgroup's share of the B panel (64
+    // rows per wave), the odd waves of the A panel, TD K blocks ahead, into the dummy area: the lines are in L2
+    // when this workgroup and its neighbours copy them.  Waves beyond the share run the same instruction on an
+    // empty descriptor.
+    const bool touch_b = (wave & 1) == 0;
+    const int share = touch_b ? (BN >> duty.b_sh) : (BM >> duty.a_sh);      // rows of the share, a power of two
+    const int t_idx = (wave >> 1) * 64 + lane;
+    intx4 rt = touch_b ? rb : ra;
+    // nobody to share with: touching one's own lines ahead of the copy only adds requests (measured)
+    if ((wave >> 1) * 64 >= share || (touch_b ? duty.b_sh : duty.a_sh) == 0) rt[2] = 0;
+    const int touch_off = ((touch_b ? duty.b_duty : duty.a_duty) * share + (t_idx & (share - 1))) * K;
+
+    // ---- fragment reads: lane -> row (lane%16) and the 32-byte K slice (lane/16) of a 16-row sub-tile
+    const int frow = lane & 15, fk = lane >> 4;
+    const int a_rd0 = (wm * WM + frow) * 128 + (((2 * fk) ^ swz(frow)) << 4);
+    const int a_rd1 = (wm * WM + frow) * 128 + (((2 * fk + 1) ^ swz(frow)) << 4);
+    const int b_rd0 = (wn * WN + frow) * 128 + (((2 * fk) ^ swz(frow)) << 4);
+    const int b_rd1 = (wn * WN + frow) * 128 + (((2 * fk + 1) ^ swz(frow)) << 4);
+    const int h0 = HOLD_A ? a_rd0 : b_rd0, h1 = HOLD_A ? a_rd1 : b_rd1;   // held operand
+    const int x0 = HOLD_A ? b_rd0 : a_rd0, x1 = HOLD_A ? b_rd1 : a_rd1;   // streamed operand
+    const int s_rd = wm * WM + frow;
+    const float* my_bs = lds_bs[(wn * WN) >> 7];
+
+    floatx4 acc[TI][TJ];
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    auto read_frag = [&](const uint8_t* base, int rd0, int rd1, int idx) {
+        const intx4 lo = *reinterpret_cast<const intx4*>(base + rd0 + idx * 2048);
+        const intx4 hi = *reinterpret_cast<const intx4*>(base + rd1 + idx * 2048);
+        return intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    };
+
+    auto touch = [&](int kb) { dma4(rt, touch_off, kb < kb1 ? kb * 128 : rt[2], ld_base + 256); };
+
+    // ---- prologue: the tile's weight scales, then the copies in the order the K loop keeps up: for every K
+    // block its first FIRST copies, the rest, one touch; K blocks 0 .. STAGES-2 whole and the first copies of
+    // block STAGES-1.  Then wait for block 0 and load the registers of step 0.
+    if (wave < NBS) {
+        const int nb = min((n0 >> 7) + wave, ((N + 127) >> 7) - 1);
+        const intx4 rbs = make_rsrc(b_s + (size_t)nb * KB, (uint32_t)KB * 4u);
+        for (int cc = 0; cc < KB; cc += 64) dma4(rbs, lane * 4, cc * 4, lds_addr(&lds_bs[wave][cc]));
+    }
+#pragma unroll
+    for (int blk = 0; blk < STAGES - 1; ++blk) {
+#pragma unroll
+        for (int i = 0; i < NDMA; ++i) issue(i, kb0 + blk, blk);
+        if (!NO_TOUCH) touch(kb0 + blk + 1 + TD - STAGES);
+        else touch(1 << 20);      // same load count for the waits below: a copy of nothing
+    }
+#pragma unroll
+    for (int i = 0; i < FIRST; ++i) issue(i, kb0 + STAGES - 1, STAGES - 1);
+    if (NO_COPY) {     // probe: the whole ring up front, nothing is copied later
+#pragma unroll
+        for (int i = FIRST; i < NDMA; ++i) issue(i, kb0 + STAGES - 1, STAGES - 1);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 2) * (NDMA + 1) + 1 + FIRST) : "memory");
+    __syncthreads();
+    intx8 fh[NH], fx[2];
+    float sc[TI];
+#pragma unroll
+    for (int h = 0; h < NH; ++h) fh[h] = read_frag(HOLD_A ? lds_a[0] : lds_b[0], h0, h1, h);
+    {
+        const float sb = my_bs[kb0];
+#pragma unroll
+        for (int i = 0; i < TI; ++i) sc[i] = lds_s[0][s_rd + i * 16] * sb;
+    }
+    fx[0] = read_frag(HOLD_A ? lds_b[0] : lds_a[0], x0, x1, 0);
+
+    int cur = 0;                                             // buffer of K block kb: kb % STAGES
+    for (int kb = kb0; kb < kb1; ++kb) {
+        const int nxt = cur + 1 == STAGES ? 0 : cur + 1;     // buffer of K block kb+1
+        const int last = cur == 0 ? STAGES - 1 : cur - 1;    // buffer of K block kb+STAGES-1
+        const uint8_t* lx = HOLD_A ? lds_b[cur] : lds_a[cur];            // streamed operand of this K block
+        const uint8_t* lh_n = HOLD_A ? lds_a[nxt] : lds_b[nxt];          // operands and scales of the next one
+        const uint8_t* lx_n = HOLD_A ? lds_b[nxt] : lds_a[nxt];
+        const float* ls_n = lds_s[nxt];
+        float sc_n[TI];
+        floatx4 p[DEPTH + 1];
+#pragma unroll
+        for (int t = 0; t < NT + DEPTH; ++t) {
+            if (t < NT) {
+                const int si = t / NH, h = t % NH;
+                if (h == 0 && si + 1 < NS) {
+                    if (!NO_LDS) fx[(si + 1) & 1] = read_frag(lx, x0, x1, si + 1);
+                    else asm volatile("" : "+v"(fx[(si + 1) & 1]));      // probe: keep the operand opaque to the optimizer
+                }
+                const intx8 fa_ = HOLD_A ? fh[h] : fx[si & 1];
+                const intx8 fb_ = HOLD_A ? fx[si & 1] : fh[h];
+                if (!NO_FOLD) {
+                    p[t % (DEPTH + 1)] = mfma_block(fb_, fa_);
+                } else {
+                    floatx4& d = acc[HOLD_A ? h : si][HOLD_A ? si : h];
+                    d = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb_, fa_, d, 0, 0, 0, 0, 0, 0);
+                }
+                if (t == TB) {
+                    // K block kb+1 has landed once only the younger loads are left in flight
+                    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(YOUNGER) : "memory");
+                    __syncthreads();
+                    if (!NO_LDS) {
+                        fx[0] = read_frag(lx_n, x0, x1, 0);      // queue slot 0 was last used by streamed fragment NS-2
+                        const float sb = my_bs[min(kb + 1, KB - 1)];
+#pragma unroll
+                        for (int i = 0; i < TI; ++i) sc_n[i] = ls_n[s_rd + i * 16] * sb;
+                    } else {
+                        asm volatile("" : "+v"(fx[0]));
+#pragma unroll
+                        for (int i = 0; i < TI; ++i) sc_n[i] = sc[i];
+                    }
+                }
+                if (t >= TB) {
+                    if (!NO_LDS) fh[h] = read_frag(lh_n, h0, h1, h);   // fh[h] had its last use just above
+                    else asm volatile("" : "+v"(fh[h]));
+                }
+            }
+            if (t >= DEPTH && !NO_FOLD) {
+                const int u = t - DEPTH, si = u / NH, h = u % NH;
+                const int i = HOLD_A ? h : si, j = HOLD_A ? si : h;
+                const floatx4 q = p[u % (DEPTH + 1)];
+                fold(acc[i][j], q, sc[i]);
+            }
+            if (!NO_COPY) {
+#pragma unroll
+                for (int j = 0; j < NDMA; ++j) {
+                    const int v = TB + 1 + GAP * j;
+                    if (v < NSLOT && v == t) issue(j, kb + STAGES, cur);                    // behind the barrier: buffer cur is free
+                    if (v >= NSLOT && v - NSLOT == t) issue(j, kb + STAGES - 1, last);      // the rest of the block started in kb-1
+                }
+            }
+            if (t == TOUCH && !NO_TOUCH) touch(kb + TD);
+            __builtin_amdgcn_sched_barrier(0);  // keep the MFMA / FMA / ds_read / copy interleaving as written
+        }
+#pragma unroll
+        for (int i = 0; i < TI; ++i) sc[i] = sc_n[i];
+        cur = nxt;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing may still be writing LDS when the wave ends
+
+    // ---- epilogue: lane holds c[m][n..n+3], m = .. + lane%16, n = .. + 4*(lane/16)
+    const bool vec_ok = (ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
+#pragma unroll
+    for (int i = 0; i < TI; ++i) {
+        const int m = m0 + wm * WM + i * 16 + frow;
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+            const int n = n0 + wn * WN + j * 16 + 4 * fk;
+            float v[4] = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+            if (bias != nullptr) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (n + e < N) v[e] += bf16_one(bias[n + e]);
+            }
+            store4<OUT>(c, ldc, m, n, M, N, v, vec_ok);
+        }
+    }
+}
+
+// Tile order shared by the kernels below: consecutive workgroup ids land on different XCDs (8 of
+// them); give each XCD a contiguous run of tiles, walked in groups of 4 tile rows.
+__device__ __forceinline__ int xcd_contiguous(int pid, int ntiles) {
+    return (ntiles % 8 == 0) ? (pid & 7) * (ntiles >> 3) + (pid >> 3) : pid;
+}
+__device__ __forceinline__ Duty tile_of(int local, int tiles_m, int tiles_n, int& tm, int& tn) {
+    constexpr int GM = 4;
+    const int group = local / (GM * tiles_n);
+    const int first_m = group * GM;
+    const int gsz = min(tiles_m - first_m, GM);
+    const int in_group = (local % (GM * tiles_n)) % gsz;
+    tm = first_m + in_group;
+    tn = (local % (GM * tiles_n)) / gsz;
+    // the workgroups of an XCD run a gsz x (up to 8) block of tiles at a time
+    Duty d;
+    d.b_sh = gsz >= 4 ? 2 : gsz >= 2 ? 1 : 0;
+    d.a_sh = tiles_n >= 8 ? 3 : tiles_n >= 4 ? 2 : tiles_n >= 2 ? 1 : 0;
+    d.b_duty = in_group & ((1 << d.b_sh) - 1);
+    d.a_duty = tn & ((1 << d.a_sh) - 1);
+    return d;
+}
+
+template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT, int GAP_ = 0, int TD_ = 0, int ABL_ = 0>
+__global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
+    const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
+    const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
+    const uint16_t* __restrict__ bias, int M, int N, int K, int ldc, int tiles_m, int tiles_n) {
+    // The grid may be smaller than the number of tiles (one workgroup per CU for the 256x256 tile): a workgroup
+    // then walks tiles blockIdx.x, blockIdx.x + gridDim.x, ... itself, which saves the ~4.5 us that pass between
+    // the end of a workgroup and the start of its successor on the same CU.  Workgroup ids keep their XCD
+    // (id % 8) from tile to tile when gridDim.x is a multiple of 8.
+    __shared__ __attribute__((aligned(1024))) uint8_t pool[TileLds<BM, BN, WGM * WGN, STAGES>::bytes];
+    const int ntiles = tiles_m * tiles_n;
+    for (int pid = blockIdx.x; pid < ntiles; pid += gridDim.x) {
+        int tm, tn;
+        const Duty duty = tile_of(xcd_contiguous(pid, ntiles), tiles_m, tiles_n, tm, tn);
+        fp8_gemm_tile<BM, BN, WGM, WGN, STAGES, OUT, GAP_, TD_, ABL_>(a, a_s, as_rs, as_cs, as_bytes, b, b_s, c, bias, tm * BM, M, M,
+                                                                      tn * BN, N, K, ldc, duty, 0, K >> 7, pool);
+        __syncthreads();   // every wave has left the tile's LDS buffers before the next tile's copies land in them
+    }
+}
+
+}  // namespace mdy

@@ -1,0 +1,57 @@
+// Timing probe of the MFMA tile kernel: one tile configuration with parts of its K loop switched off.
+// It exists so that the cost of each part (global->LDS copies, LDS fragment reads, the FMA fold of the block
+// scales, the pre-touches) can be measured on the product's own code, with the product's own operands, and the
+// power / clock readings taken while it runs; the results of a probe with anything switched off are NOT a GEMM.
+// No counterpart in the reference.
+#include "fp8_gemm_tile.h"
+
+namespace mdy {
+
+template <int BM, int BN, int WGM, int WGN, int STAGES, int GAP, int ABL>
+static int probe_launch(const uint8_t* a, const float* a_s, int as_rs, int as_cs, uint32_t as_bytes, const uint8_t* b,
+                        const float* b_s, uint16_t* c, int M, int N, int K, int max_wgs, hipStream_t stream) {
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    const int wgs = (BM * BN >= 256 * 256 && tiles_m * tiles_n > max_wgs) ? max_wgs : tiles_m * tiles_n;
+    hipLaunchKernelGGL((fp8_gemm_mfma_kernel<BM, BN, WGM, WGN, STAGES, uint16_t, GAP, 0, ABL>), dim3((unsigned)wgs),
+                       dim3(WGM * WGN * 64), 0, stream, a, a_s, as_rs, as_cs, as_bytes, b, b_s, c,
+                       static_cast<const uint16_t*>(nullptr), M, N, K, N, tiles_m, tiles_n);
+    return (int)hipGetLastError();
+}
+
+// tile: 0 = 256x256 (ring of 2 K blocks), 1 = 128x256 (ring of 3).  ablation: bit set of
+// 1 no copies in the loop, 2 no LDS reads, 4 no FMA fold, 8 no pre-touches; the combinations built are
+// 0, 8, 1, 2, 4, 3, 5, 7.  Returns -1 for a combination that is not built.
+int launch_fp8_gemm_probe(int tile, int ablation, const void* a, const float* a_s, int64_t as_rs, int64_t as_cs,
+                          const void* b, const float* b_s, void* c, int64_t M, int64_t N, int64_t K, hipStream_t stream) {
+    const int KB = (int)(K / 128);
+    const int64_t as_extent = ((M - 1) * as_rs + (int64_t)(KB - 1) * as_cs + 1) * 4;
+    int cus = 256;
+    int dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus = n;
+    }
+#define MDY_PROBE(BM, BN, ST, GAP, ABL)                                                                            \
+    return probe_launch<BM, BN, 2, 4, ST, GAP, ABL>(static_cast<const uint8_t*>(a), a_s, (int)as_rs, (int)as_cs,   \
+                                                    (uint32_t)as_extent, static_cast<const uint8_t*>(b), b_s,      \
+                                                    static_cast<uint16_t*>(c), (int)M, (int)N, (int)K, cus, stream)
+#define MDY_PROBE_TILE(BM, BN, ST, GAP)                  \
+    switch (ablation) {                                  \
+        case 0: MDY_PROBE(BM, BN, ST, GAP, 0);           \
+        case 8: MDY_PROBE(BM, BN, ST, GAP, 8);           \
+        case 1: MDY_PROBE(BM, BN, ST, GAP, 1);           \
+        case 2: MDY_PROBE(BM, BN, ST, GAP, 2);           \
+        case 4: MDY_PROBE(BM, BN, ST, GAP, 4);           \
+        case 3: MDY_PROBE(BM, BN, ST, GAP, 3);           \
+        case 5: MDY_PROBE(BM, BN, ST, GAP, 5);           \
+        case 7: MDY_PROBE(BM, BN, ST, GAP, 7);           \
+        default: return -1;                              \
+    }
+    if (tile == 0) { MDY_PROBE_TILE(256, 256, 2, 0) }
+    if (tile == 1) { MDY_PROBE_TILE(128, 256, 3, 0) }
+#undef MDY_PROBE_TILE
+#undef MDY_PROBE
+    return -1;
+}
+
+}  // namespace mdy
