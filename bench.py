@@ -536,7 +536,7 @@ def ablation(torch, m, dev):
     product's own operands; per launch: time, the rate the same FLOPs would mean, socket power, shader clock."""
     from mdy_triton_amd import _lib
     L = _lib.load()
-    names = {0: "full kernel (the product)", 8: "no pre-touches", 4: "no FMA fold (MFMAs accumulate in place)",
+    names = {0: "full kernel, pre-touches on", 8: "full kernel, no pre-touches", 4: "no FMA fold (MFMAs accumulate in place)",
              2: "no LDS fragment reads", 1: "no global->LDS copies (ring replayed)", 5: "no copies, no fold",
              3: "no copies, no LDS reads", 7: "MFMA only (no copies, no LDS reads, no fold)"}
     cap = power_cap_w()

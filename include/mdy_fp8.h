@@ -184,7 +184,7 @@ int mdy_fp8_gemm_nt_ws(const void* a, const float* a_s, int64_t as_row_stride, i
  *             1 no global->LDS copies inside the K loop (the LDS ring is filled once and replayed),
  *             2 no LDS fragment reads inside the loop, 4 no FMA fold of the block scales (the matrix cores
  *             accumulate in place), 8 no pre-touches of the shared panels; built: 0, 8, 1, 2, 4, 3, 5, 7.
- *             With anything switched off c is NOT the GEMM result.
+ *             With 1, 2 or 4 in the set c is NOT the GEMM result.
  * K % 128 == 0, K <= 65536, N % 4 == 0, a / b / c 16-byte aligned; MDY_E_DTYPE for a combination that is not built.
  */
 int mdy_fp8_gemm_probe(int tile, int ablation, const void* a, const float* a_s, int64_t as_row_stride,

@@ -144,7 +144,7 @@ __device__ __forceinline__ void fp8_gemm_tile(
     // twice what the CU's address unit takes (64 lanes x 16 bytes = 16 clocks each, a slot is 64 clocks for
     // the two waves of a SIMD): the waves then queue on the copy instruction and their MFMAs behind it wait.
     // Measured: 256x256 tiles 1-5 % faster with every second slot, 128x256 tiles (half as many slots) not.
-    constexpr int GAP = GAP_ > 0 ? GAP_ : (WAVES >= 8 && NT >= 32) ? 2 : 1;
+    constexpr int GAP = GAP_ > 0 ? GAP_ : (WAVES >= 8 && NT >= 16) ? 2 : 1;
     constexpr int TAIL = (NSLOT - TB - 1 + GAP - 1) / GAP;   // copies that still fit behind the barrier
     constexpr int FIRST = TAIL < NDMA ? TAIL : NDMA;         // copies of K block kb+2 issued in the tail of kb
     constexpr int TOUCH = FIRST < NDMA ? TB + 1 + GAP * (NDMA - 1) - NSLOT + 1 : 0;   // slot after the last copy
@@ -171,43 +171,77 @@ __device__ __forceinline__ void fp8_gemm_tile(
     const int M = m_end;
     const int KB = K >> 7;
 
-    // ---- DMA: descriptors limited to the rows of this tile, so that the M and N tails read 0
-    const intx4 ra = make_rsrc(a + (size_t)m0 * K, (uint32_t)min(BM, M - m0) * (uint32_t)K);
-    const intx4 rb = make_rsrc(b + (size_t)n0 * K, (uint32_t)min(BN, N - n0) * (uint32_t)K);
-    intx4 rs = make_rsrc(a_s, as_bytes);
-    if (wave >= S_WAVES) rs[2] = 0;                                   // these waves copy no scales: always out of range
+    // ---- DMA.  What depends on the tile: the descriptors (limited to the rows of the tile, so that the M and N
+    // tails read 0), the rows whose scales a lane copies, and the share of the panels this workgroup pre-touches.
+    struct TileAddr {
+        intx4 ra, rb, rt;
+        int s_voff, touch_off, n0;
+    };
     const int prow = wave * 8 + (lane >> 3);                          // row inside a pass
     const int voff = prow * K + (((lane & 7) ^ swz(prow)) << 4);      // permuted chunk of that row
-    const int s_voff = min(m0 + (wave % S_WAVES) * 64 + lane, m_total - 1) * as_rs * 4;
+    intx4 rs = make_rsrc(a_s, as_bytes);
+    if (wave >= S_WAVES) rs[2] = 0;                                   // these waves copy no scales: always out of range
     const uint32_t ld_base = lds_addr(&lds_dummy[0]) + wave * 512;
     const uint32_t la_base = lds_addr(&lds_a[0][0]) + wave * 1024;
     const uint32_t lb_base = lds_addr(&lds_b[0][0]) + wave * 1024;
     const uint32_t ls_base = wave < S_WAVES ? lds_addr(&lds_s[0][0]) + wave * 256 : ld_base;
     const uint32_t ls_buf = wave < S_WAVES ? BM * 4 : 0;
-
-    // copy i (0: scales, then the A passes, then the B passes) of K block kb into buffer buf.  Past the last K
-    // block the offsets run beyond the descriptors: no memory access, zeros into a buffer nobody reads any more.
-    auto issue = [&](int i, int kb, int buf) {
-        const bool more = kb < kb1;
-        if (i == 0)
-            dma4(rs, s_voff, more ? kb * as_cs * 4 : (int)as_bytes, ls_base + buf * ls_buf);
-        else if (i <= A_PASSES)
-            dma16(ra, voff, (i - 1) * PASS_ROWS * K + (more ? kb * 128 : ra[2]), la_base + buf * (BM * 128) + (i - 1) * PASS_ROWS * 128);
-        else
-            dma16(rb, voff, (i - 1 - A_PASSES) * PASS_ROWS * K + (more ? kb * 128 : rb[2]),
-                  lb_base + buf * (BN * 128) + (i - 1 - A_PASSES) * PASS_ROWS * 128);
-    };
     // duty touch: the even waves load one dword of every line of this workgroup's share of the B panel (64
     // rows per wave), the odd waves of the A panel, TD K blocks ahead, into the dummy area: the lines are in L2
     // when this workgroup and its neighbours copy them.  Waves beyond the share run the same instruction on an
     // empty descriptor.
     const bool touch_b = (wave & 1) == 0;
-    const int share = touch_b ? (BN >> duty.b_sh) : (BM >> duty.a_sh);      // rows of the share, a power of two
     const int t_idx = (wave >> 1) * 64 + lane;
-    intx4 rt = touch_b ? rb : ra;
-    // nobody to share with: touching one's own lines ahead of the copy only adds requests (measured)
-    if ((wave >> 1) * 64 >= share || (touch_b ? duty.b_sh : duty.a_sh) == 0) rt[2] = 0;
-    const int touch_off = ((touch_b ? duty.b_duty : duty.a_duty) * share + (t_idx & (share - 1))) * K;
+    auto tile_addr = [&](int tm0, int tn0, const Duty& d) {
+        TileAddr t;
+        t.ra = make_rsrc(a + (size_t)tm0 * K, (uint32_t)min(BM, M - tm0) * (uint32_t)K);
+        t.rb = make_rsrc(b + (size_t)tn0 * K, (uint32_t)min(BN, N - tn0) * (uint32_t)K);
+        t.s_voff = min(tm0 + (wave % S_WAVES) * 64 + lane, m_total - 1) * as_rs * 4;
+        const int share = touch_b ? (BN >> d.b_sh) : (BM >> d.a_sh);      // rows of the share, a power of two
+        t.rt = touch_b ? t.rb : t.ra;
+        // nobody to share with: touching one's own lines ahead of the copy only adds requests (measured)
+        if ((wave >> 1) * 64 >= share || (touch_b ? d.b_sh : d.a_sh) == 0) t.rt[2] = 0;
+        t.touch_off = ((touch_b ? d.b_duty : d.a_duty) * share + (t_idx & (share - 1))) * K;
+        t.n0 = tn0;
+        return t;
+    };
+    const TileAddr me = tile_addr(m0, n0, duty);
+
+    // copy i (0: scales, then the A passes, then the B passes) of K block kb into buffer buf.  Past the last K
+    // block the offsets run beyond the descriptors: no memory access, zeros into a buffer nobody reads any more.
+    auto issue = [&](const TileAddr& t, int i, int kb, int buf) {
+        const bool more = kb < kb1;
+        if (i == 0)
+            dma4(rs, t.s_voff, more ? kb * as_cs * 4 : (int)as_bytes, ls_base + buf * ls_buf);
+        else if (i <= A_PASSES)
+            dma16(t.ra, voff, (i - 1) * PASS_ROWS * K + (more ? kb * 128 : t.ra[2]), la_base + buf * (BM * 128) + (i - 1) * PASS_ROWS * 128);
+        else
+            dma16(t.rb, voff, (i - 1 - A_PASSES) * PASS_ROWS * K + (more ? kb * 128 : t.rb[2]),
+                  lb_base + buf * (BN * 128) + (i - 1 - A_PASSES) * PASS_ROWS * 128);
+    };
+    auto touch = [&](const TileAddr& t, int kb) { dma4(t.rt, t.touch_off, kb < kb1 ? kb * 128 : t.rt[2], ld_base + 256); };
+    // The start of a tile: its weight scales, then the copies in the order the K loop keeps up: for every K block its
+    // first FIRST copies, the rest, one touch; K blocks 0 .. STAGES-2 whole and the first copies of block STAGES-1.
+    auto prologue = [&](const TileAddr& t) {
+        if (wave < NBS) {
+            const int nb = min((t.n0 >> 7) + wave, ((N + 127) >> 7) - 1);
+            const intx4 rbs = make_rsrc(b_s + (size_t)nb * KB, (uint32_t)KB * 4u);
+            for (int cc = 0; cc < KB; cc += 64) dma4(rbs, lane * 4, cc * 4, lds_addr(&lds_bs[wave][cc]));
+        }
+#pragma unroll
+        for (int blk = 0; blk < STAGES - 1; ++blk) {
+#pragma unroll
+            for (int i = 0; i < NDMA; ++i) issue(t, i, kb0 + blk, blk);
+            if (!NO_TOUCH) touch(t, kb0 + blk + 1 + TD - STAGES);
+            else touch(t, 1 << 20);      // same load count for the waits below: a copy of nothing
+        }
+#pragma unroll
+        for (int i = 0; i < FIRST; ++i) issue(t, i, kb0 + STAGES - 1, STAGES - 1);
+        if (NO_COPY) {     // probe: the whole ring up front, nothing is copied later
+#pragma unroll
+            for (int i = FIRST; i < NDMA; ++i) issue(t, i, kb0 + STAGES - 1, STAGES - 1);
+        }
+    };
 
     // ---- fragment reads: lane -> row (lane%16) and the 32-byte K slice (lane/16) of a 16-row sub-tile
     const int frow = lane & 15, fk = lane >> 4;
@@ -232,31 +266,10 @@ __device__ __forceinline__ void fp8_gemm_tile(
         return intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     };
 
-    auto touch = [&](int kb) { dma4(rt, touch_off, kb < kb1 ? kb * 128 : rt[2], ld_base + 256); };
-
-    // ---- prologue: the tile's weight scales, then the copies in the order the K loop keeps up: for every K
-    // block its first FIRST copies, the rest, one touch; K blocks 0 .. STAGES-2 whole and the first copies of
-    // block STAGES-1.  Then wait for block 0 and load the registers of step 0.
-    if (wave < NBS) {
-        const int nb = min((n0 >> 7) + wave, ((N + 127) >> 7) - 1);
-        const intx4 rbs = make_rsrc(b_s + (size_t)nb * KB, (uint32_t)KB * 4u);
-        for (int cc = 0; cc < KB; cc += 64) dma4(rbs, lane * 4, cc * 4, lds_addr(&lds_bs[wave][cc]));
-    }
-#pragma unroll
-    for (int blk = 0; blk < STAGES - 1; ++blk) {
-#pragma unroll
-        for (int i = 0; i < NDMA; ++i) issue(i, kb0 + blk, blk);
-        if (!NO_TOUCH) touch(kb0 + blk + 1 + TD - STAGES);
-        else touch(1 << 20);      // same load count for the waits below: a copy of nothing
-    }
-#pragma unroll
-    for (int i = 0; i < FIRST; ++i) issue(i, kb0 + STAGES - 1, STAGES - 1);
-    if (NO_COPY) {     // probe: the whole ring up front, nothing is copied later
-#pragma unroll
-        for (int i = FIRST; i < NDMA; ++i) issue(i, kb0 + STAGES - 1, STAGES - 1);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    }
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 2) * (NDMA + 1) + 1 + FIRST) : "memory");
+    // ---- prologue, wait for block 0, load the registers of step 0
+    prologue(me);
+    if (NO_COPY) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 2) * (NDMA + 1) + 1 + FIRST) : "memory");
     __syncthreads();
     intx8 fh[NH], fx[2];
     float sc[TI];
@@ -325,11 +338,11 @@ __device__ __forceinline__ void fp8_gemm_tile(
 #pragma unroll
                 for (int j = 0; j < NDMA; ++j) {
                     const int v = TB + 1 + GAP * j;
-                    if (v < NSLOT && v == t) issue(j, kb + STAGES, cur);                    // behind the barrier: buffer cur is free
-                    if (v >= NSLOT && v - NSLOT == t) issue(j, kb + STAGES - 1, last);      // the rest of the block started in kb-1
+                    if (v < NSLOT && v == t) issue(me, j, kb + STAGES, cur);                    // behind the barrier: buffer cur is free
+                    if (v >= NSLOT && v - NSLOT == t) issue(me, j, kb + STAGES - 1, last);      // the rest of the block started in kb-1
                 }
             }
-            if (t == TOUCH && !NO_TOUCH) touch(kb + TD);
+            if (t == TOUCH && !NO_TOUCH) touch(me, kb + TD);
             __builtin_amdgcn_sched_barrier(0);  // keep the MFMA / FMA / ds_read / copy interleaving as written
         }
 #pragma unroll
@@ -383,7 +396,7 @@ template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT, int GAP_ =
 __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
-    const uint16_t* __restrict__ bias, int M, int N, int K, int ldc, int tiles_m, int tiles_n) {
+    const uint16_t* __restrict__ bias, int M, int N, int K, int ldc, int tiles_m, int tiles_n, int pretouch) {
     // The grid may be smaller than the number of tiles (one workgroup per CU for the 256x256 tile): a workgroup
     // then walks tiles blockIdx.x, blockIdx.x + gridDim.x, ... itself, which saves the ~4.5 us that pass between
     // the end of a workgroup and the start of its successor on the same CU.  Workgroup ids keep their XCD
@@ -392,7 +405,8 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
     const int ntiles = tiles_m * tiles_n;
     for (int pid = blockIdx.x; pid < ntiles; pid += gridDim.x) {
         int tm, tn;
-        const Duty duty = tile_of(xcd_contiguous(pid, ntiles), tiles_m, tiles_n, tm, tn);
+        Duty duty = tile_of(xcd_contiguous(pid, ntiles), tiles_m, tiles_n, tm, tn);
+        if (!pretouch) duty.a_sh = duty.b_sh = 0;
         fp8_gemm_tile<BM, BN, WGM, WGN, STAGES, OUT, GAP_, TD_, ABL_>(a, a_s, as_rs, as_cs, as_bytes, b, b_s, c, bias, tm * BM, M, M,
                                                                       tn * BN, N, K, ldc, duty, 0, K >> 7, pool);
         __syncthreads();   // every wave has left the tile's LDS buffers before the next tile's copies land in them

@@ -14,13 +14,13 @@ static int probe_launch(const uint8_t* a, const float* a_s, int as_rs, int as_cs
     const int wgs = (BM * BN >= 256 * 256 && tiles_m * tiles_n > max_wgs) ? max_wgs : tiles_m * tiles_n;
     hipLaunchKernelGGL((fp8_gemm_mfma_kernel<BM, BN, WGM, WGN, STAGES, uint16_t, GAP, 0, ABL>), dim3((unsigned)wgs),
                        dim3(WGM * WGN * 64), 0, stream, a, a_s, as_rs, as_cs, as_bytes, b, b_s, c,
-                       static_cast<const uint16_t*>(nullptr), M, N, K, N, tiles_m, tiles_n);
+                       static_cast<const uint16_t*>(nullptr), M, N, K, N, tiles_m, tiles_n, 1);
     return (int)hipGetLastError();
 }
 
 // tile: 0 = 256x256 (ring of 2 K blocks), 1 = 128x256 (ring of 3).  ablation: bit set of
 // 1 no copies in the loop, 2 no LDS reads, 4 no FMA fold, 8 no pre-touches; the combinations built are
-// 0, 8, 1, 2, 4, 3, 5, 7.  Returns -1 for a combination that is not built.
+// 0, 8, 1, 2, 4, 3, 5, 7 (0 and 8 give the exact GEMM result).  Returns -1 for a combination that is not built.
 int launch_fp8_gemm_probe(int tile, int ablation, const void* a, const float* a_s, int64_t as_rs, int64_t as_cs,
                           const void* b, const float* b_s, void* c, int64_t M, int64_t N, int64_t K, hipStream_t stream) {
     const int KB = (int)(K / 128);
