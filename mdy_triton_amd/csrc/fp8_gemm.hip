@@ -507,6 +507,7 @@ static bool big_tiles_pay(int64_t M, int64_t N) {
 //   0: 128x128, 2 K blocks in LDS (two workgroups share a CU)   1: 128x128, 4 K blocks (one workgroup per CU)
 //   2: 128x64, 6 K blocks                                       3: 64x64, 8 K blocks
 //   4: 128x256, 3 K blocks, 8 waves                             5: 256x128, 3 K blocks, 8 waves
+//   6: 128x192, 3 K blocks, 8 waves (wave tile 64x48)
 // Measured rule: the smallest tile that still gives every workgroup a CU of its own (the time of these
 // shapes goes with the bytes each CU has to pull, not with its MFMAs), and the ring as deep as LDS allows.
 // Between 257 and 512 tiles of 128x128 that is a 128x256 tile (else, if those are too many, 256x128), one per CU,
@@ -521,6 +522,9 @@ static int few_tiles_config(int M, int N, int K) {
     if (rows128 * cols128 <= cus) return 1;
     if (K < 1024) return 0;    // a handful of K blocks: two short workgroups per CU hide each other's prologue and epilogue
     const long wide = rows128 * cols256, tall = rows256 * cols128;
+    // more 128x256 tiles than 3/4 of the CUs and 128x192 tiles still one per CU: the smaller tile puts the idle CUs to
+    // work (4096x1536x7168: 256 tiles of 128x192 instead of 192 of 128x256)
+    if (wide <= cus && rows128 * ((N + 191) / 192) <= cus && rows128 * ((N + 191) / 192) > wide) return 6;
     if (wide <= cus) return 4;    // also when it pads more than the tall tile: 12800x384x7168 82 against 95 us
     if (tall <= cus) return 5;
     return 0;
@@ -631,6 +635,7 @@ static int dispatch(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t a
         case 3: MDY_FEW(64, 64, 8);
         case 4: return launch_mfma<128, 256, 2, 4, 3, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
         case 5: return launch_mfma<256, 128, 2, 4, 3, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
+        case 6: return launch_mfma<128, 192, 2, 4, 3, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
         default: MDY_FEW(128, 128, 2);
     }
 #undef MDY_FEW

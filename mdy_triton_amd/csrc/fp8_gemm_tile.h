@@ -132,7 +132,11 @@ __device__ __forceinline__ void fp8_gemm_tile(
     constexpr int S_WAVES = BM / 64;      // waves that also copy the activation scales
     constexpr int DEPTH = 4;              // MFMAs in flight before their results are folded
     static_assert(BM % PASS_ROWS == 0 && BN % PASS_ROWS == 0 && PASS_ROWS % 16 == 0, "tile/threads mismatch");
-    static_assert(WN <= 128 && 128 % WN == 0 && S_WAVES <= WAVES && WAVES >= 2, "one weight-scale block per wave column");
+    // A wave's WN columns lie in one 128-column weight-scale block when WN divides 128 (tiles then start on multiples
+    // of WN); the 192-wide tile (WN = 48, tiles start on multiples of 64) can straddle two: its 16-column sub-tiles never
+    // do, so such a wave keeps two combined scales per row and each sub-tile takes the one of its block.
+    constexpr bool STRADDLE = (128 % WN) != 0;
+    static_assert(WN <= 128 && (!STRADDLE || BN == 192) && S_WAVES <= WAVES && WAVES >= 2, "weight-scale blocks per wave column");
     constexpr bool HOLD_A = TI <= TJ;
     constexpr int NH = HOLD_A ? TI : TJ, NS = HOLD_A ? TJ : TI;
     constexpr int NT = TI * TJ;
@@ -143,8 +147,8 @@ __device__ __forceinline__ void fp8_gemm_tile(
     // and running over into the first slots of the next block.  With 8 waves one copy per slot and wave is
     // twice what the CU's address unit takes (64 lanes x 16 bytes = 16 clocks each, a slot is 64 clocks for
     // the two waves of a SIMD): the waves then queue on the copy instruction and their MFMAs behind it wait.
-    // Measured: 256x256 tiles 1-5 % faster with every second slot, 128x256 tiles (half as many slots) not.
-    constexpr int GAP = GAP_ > 0 ? GAP_ : (WAVES >= 8 && NT >= 16) ? 2 : 1;
+    // Measured: 256x256 tiles 1-5 % faster with every second slot; 128x256 and 128x192 tiles 2-7 % at 4096x1536x7168.
+    constexpr int GAP = GAP_ > 0 ? GAP_ : (WAVES >= 8 && NT >= 12) ? 2 : 1;
     constexpr int TAIL = (NSLOT - TB - 1 + GAP - 1) / GAP;   // copies that still fit behind the barrier
     constexpr int FIRST = TAIL < NDMA ? TAIL : NDMA;         // copies of K block kb+2 issued in the tail of kb
     constexpr int TOUCH = FIRST < NDMA ? TB + 1 + GAP * (NDMA - 1) - NSLOT + 1 : 0;   // slot after the last copy
@@ -197,11 +201,11 @@ __device__ __forceinline__ void fp8_gemm_tile(
         t.ra = make_rsrc(a + (size_t)tm0 * K, (uint32_t)min(BM, M - tm0) * (uint32_t)K);
         t.rb = make_rsrc(b + (size_t)tn0 * K, (uint32_t)min(BN, N - tn0) * (uint32_t)K);
         t.s_voff = min(tm0 + (wave % S_WAVES) * 64 + lane, m_total - 1) * as_rs * 4;
-        const int share = touch_b ? (BN >> d.b_sh) : (BM >> d.a_sh);      // rows of the share, a power of two
+        const int share = touch_b ? (BN >> d.b_sh) : (BM >> d.a_sh);      // rows of the share
         t.rt = touch_b ? t.rb : t.ra;
         // nobody to share with: touching one's own lines ahead of the copy only adds requests (measured)
         if ((wave >> 1) * 64 >= share || (touch_b ? d.b_sh : d.a_sh) == 0) t.rt[2] = 0;
-        t.touch_off = ((touch_b ? d.b_duty : d.a_duty) * share + (t_idx & (share - 1))) * K;
+        t.touch_off = ((touch_b ? d.b_duty : d.a_duty) * share + t_idx % share) * K;
         t.n0 = tn0;
         return t;
     };
@@ -252,7 +256,10 @@ __device__ __forceinline__ void fp8_gemm_tile(
     const int h0 = HOLD_A ? a_rd0 : b_rd0, h1 = HOLD_A ? a_rd1 : b_rd1;   // held operand
     const int x0 = HOLD_A ? b_rd0 : a_rd0, x1 = HOLD_A ? b_rd1 : a_rd1;   // streamed operand
     const int s_rd = wm * WM + frow;
-    const float* my_bs = lds_bs[(wn * WN) >> 7];
+    const int bs_col = (n0 & 127) + wn * WN;                        // first column of the wave inside the tile's first scale block
+    const float* my_bs = lds_bs[bs_col >> 7];
+    const float* my_bs_hi = lds_bs[(bs_col + WN - 1) >> 7];         // STRADDLE: the block of the wave's last columns
+    const int jsplit = STRADDLE ? min(TJ, (128 - (bs_col & 127)) >> 4) : TJ;   // sub-tiles j < jsplit lie in the first block
 
     floatx4 acc[TI][TJ];
 #pragma unroll
@@ -272,13 +279,17 @@ __device__ __forceinline__ void fp8_gemm_tile(
     else asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 2) * (NDMA + 1) + 1 + FIRST) : "memory");
     __syncthreads();
     intx8 fh[NH], fx[2];
-    float sc[TI];
+    float sc[TI], sc_hi[STRADDLE ? TI : 1];
 #pragma unroll
     for (int h = 0; h < NH; ++h) fh[h] = read_frag(HOLD_A ? lds_a[0] : lds_b[0], h0, h1, h);
     {
-        const float sb = my_bs[kb0];
+        const float sb = my_bs[kb0], sb_hi = my_bs_hi[kb0];
 #pragma unroll
-        for (int i = 0; i < TI; ++i) sc[i] = lds_s[0][s_rd + i * 16] * sb;
+        for (int i = 0; i < TI; ++i) {
+            const float sa = lds_s[0][s_rd + i * 16];
+            sc[i] = sa * sb;
+            if (STRADDLE) sc_hi[i] = sa * sb_hi;
+        }
     }
     fx[0] = read_frag(HOLD_A ? lds_b[0] : lds_a[0], x0, x1, 0);
 
@@ -290,7 +301,7 @@ __device__ __forceinline__ void fp8_gemm_tile(
         const uint8_t* lh_n = HOLD_A ? lds_a[nxt] : lds_b[nxt];          // operands and scales of the next one
         const uint8_t* lx_n = HOLD_A ? lds_b[nxt] : lds_a[nxt];
         const float* ls_n = lds_s[nxt];
-        float sc_n[TI];
+        float sc_n[TI], sc_hi_n[STRADDLE ? TI : 1];
         floatx4 p[DEPTH + 1];
 #pragma unroll
         for (int t = 0; t < NT + DEPTH; ++t) {
@@ -314,13 +325,20 @@ __device__ __forceinline__ void fp8_gemm_tile(
                     __syncthreads();
                     if (!NO_LDS) {
                         fx[0] = read_frag(lx_n, x0, x1, 0);      // queue slot 0 was last used by streamed fragment NS-2
-                        const float sb = my_bs[min(kb + 1, KB - 1)];
+                        const float sb = my_bs[min(kb + 1, KB - 1)], sb_hi = my_bs_hi[min(kb + 1, KB - 1)];
 #pragma unroll
-                        for (int i = 0; i < TI; ++i) sc_n[i] = ls_n[s_rd + i * 16] * sb;
+                        for (int i = 0; i < TI; ++i) {
+                            const float sa = ls_n[s_rd + i * 16];
+                            sc_n[i] = sa * sb;
+                            if (STRADDLE) sc_hi_n[i] = sa * sb_hi;
+                        }
                     } else {
                         asm volatile("" : "+v"(fx[0]));
 #pragma unroll
-                        for (int i = 0; i < TI; ++i) sc_n[i] = sc[i];
+                        for (int i = 0; i < TI; ++i) {
+                            sc_n[i] = sc[i];
+                            if (STRADDLE) sc_hi_n[i] = sc_hi[i];
+                        }
                     }
                 }
                 if (t >= TB) {
@@ -332,7 +350,7 @@ __device__ __forceinline__ void fp8_gemm_tile(
                 const int u = t - DEPTH, si = u / NH, h = u % NH;
                 const int i = HOLD_A ? h : si, j = HOLD_A ? si : h;
                 const floatx4 q = p[u % (DEPTH + 1)];
-                fold(acc[i][j], q, sc[i]);
+                fold(acc[i][j], q, (STRADDLE && j >= jsplit) ? sc_hi[i] : sc[i]);
             }
             if (!NO_COPY) {
 #pragma unroll
@@ -346,7 +364,10 @@ __device__ __forceinline__ void fp8_gemm_tile(
             __builtin_amdgcn_sched_barrier(0);  // keep the MFMA / FMA / ds_read / copy interleaving as written
         }
 #pragma unroll
-        for (int i = 0; i < TI; ++i) sc[i] = sc_n[i];
+        for (int i = 0; i < TI; ++i) {
+            sc[i] = sc_n[i];
+            if (STRADDLE) sc_hi[i] = sc_hi_n[i];
+        }
         cur = nxt;
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing may still be writing LDS when the wave ends

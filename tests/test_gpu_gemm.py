@@ -76,6 +76,7 @@ def test_gemm_exact_integer_cases_all_kernels(M, N, K):
 @pytest.mark.parametrize("M,N,K", [(896, 9300, 256), (880, 9344, 640),         # 128x128 tiles, 2 K blocks in LDS
                                    (2000, 2304, 256), (2048, 2200, 512),          # the same for a short K
                                    (2000, 2304, 1024), (4096, 1536, 1152), (1300, 5800, 2304),   # 128x256 tiles, ring of 3
+                                   (4096, 1100, 1024), (4000, 1530, 1280), (3000, 1700, 1152), (3072, 1536, 2048),   # 128x192 tiles (wave columns straddle weight-scale blocks)
                                    (12800, 384, 1024),                                              # 128x256 tiles although they pad more
                                    (38400, 128, 1024), (36000, 100, 1280),       # 256x128 tiles, ring of 3
                                    (1536, 2048, 128), (1500, 2000, 1280),      # 128x128 tiles, ring of 4 K blocks
