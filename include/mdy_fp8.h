@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define MDY_FP8_ABI_VERSION 5
+#define MDY_FP8_ABI_VERSION 6
 
 /* error codes (negative = argument rejected before any launch) */
 #define MDY_OK 0
@@ -247,6 +247,21 @@ int mdy_fp8_grouped_gemm_nt(const void* a, const float* a_s, int64_t as_row_stri
                             const void* b, const float* b_s, void* c, const void* bias,
                             const int64_t* m_splits, int64_t G, int64_t N, int64_t K, int out_dtype,
                             void* stream);
+
+/* Row padding (unpad = 0) / unpadding (unpad != 0) of grouped activations: the rows of the unpadded matrix are G
+ * consecutive groups of m_splits[g] rows; in the padded matrix group g owns a slot of ceil(m_splits[g] / multiple) *
+ * multiple rows whose rows beyond m_splits[g] are zero.  Replaces Fp8Padding / Fp8Unpadding
+ * (triton_kernels/megatron_patchs/dpsk_grouped_linear.py:690-902: TransformerEngine's multi_padding_fused with
+ * multiple = 256, and torch.split + torch.cat for the way back).
+ *
+ *   x         source, row-major, row_bytes bytes per row (any element type): [sum m, row_bytes] when padding,
+ *             [sum pad(m), row_bytes] when unpadding
+ *   y         destination of the other layout; every byte of it is written
+ *   m_splits  HOST pointer to G non-negative row counts (read before the call returns)
+ * 16-byte aligned pointers and row_bytes % 16 == 0 take the vector path; anything else is copied in 2- or 1-byte pieces.
+ */
+int mdy_group_pad_rows(const void* x, void* y, const int64_t* m_splits, int64_t G, int64_t row_bytes, int64_t multiple,
+                       int unpad, void* stream);
 
 /* In-place x[m, :] = bf16(fp32(x[m, :]) + fp32(b)) on bf16 x [M, N] row-major, bf16 b [N].
  * Replaces add_bias (fp8.py:297-305, kernel :283-295). */

@@ -11,5 +11,7 @@ from .fp8_kernel import (Fp8MLP, fp8_ckpt_mlp, silu_act_quant, silu_bwd, silu_fw
 from .megatron_patchs.fp8_matmul import (fp8_grouped_matmul, group_per_token_cast_to_fp8, per_block_cast_to_fp8,  # noqa: F401
                          per_token_cast_to_fp8)
 
-__all__ = ["Fp8MLP", "fp8_ckpt_mlp", "per_token_cast_to_fp8", "group_per_token_cast_to_fp8", "per_block_cast_to_fp8", "fp8_grouped_matmul", "silu_fwd", "silu_bwd", "triton_silu", "silu_act_quant", "weight_quant_block", "act_quant", "weight_dequant", "fp8_gemm", "quant_input", "quant_weight", "quant_grad_output", "fp8_matmul", "add_bias",
+from .megatron_patchs.dpsk_grouped_linear import Fp8Padding, Fp8Unpadding  # noqa: F401
+
+__all__ = ["Fp8Padding", "Fp8Unpadding", "Fp8MLP", "fp8_ckpt_mlp", "per_token_cast_to_fp8", "group_per_token_cast_to_fp8", "per_block_cast_to_fp8", "fp8_grouped_matmul", "silu_fwd", "silu_bwd", "triton_silu", "silu_act_quant", "weight_quant_block", "act_quant", "weight_dequant", "fp8_gemm", "quant_input", "quant_weight", "quant_grad_output", "fp8_matmul", "add_bias",
            "DeepLinear"]

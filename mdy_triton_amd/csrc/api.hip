@@ -267,6 +267,27 @@ int mdy_fp8_grouped_gemm_nt(const void* a, const float* a_s, int64_t as_row_stri
                     "fp8_grouped_gemm_nt");
 }
 
+int mdy_group_pad_rows(const void* x, void* y, const int64_t* m_splits, int64_t G, int64_t row_bytes, int64_t multiple,
+                       int unpad, void* stream) {
+    if (G < 0 || G > (1 << 20) || row_bytes < 0 || row_bytes > ((int64_t)1 << 32) || multiple < 1 || multiple > (1 << 20))
+        return fail(MDY_E_SHAPE, "group_pad_rows: bad G=%lld / row_bytes=%lld / multiple=%lld", (long long)G, (long long)row_bytes,
+                    (long long)multiple);
+    if (G == 0 || row_bytes == 0) return 0;
+    if (!m_splits) return fail(MDY_E_NULL, "group_pad_rows: null m_splits");
+    int64_t rows = 0, padded = 0;
+    for (int64_t g = 0; g < G; ++g) {
+        if (m_splits[g] < 0 || m_splits[g] > kMaxDim) return fail(MDY_E_SHAPE, "group_pad_rows: m_splits[%lld]=%lld", (long long)g, (long long)m_splits[g]);
+        rows += m_splits[g];
+        padded += (m_splits[g] + multiple - 1) / multiple * multiple;
+    }
+    if (padded > ((int64_t)1 << 36)) return fail(MDY_E_SHAPE, "group_pad_rows: too many rows (%lld)", (long long)padded);
+    if ((unpad ? rows : padded) == 0) return 0;
+    if (!y || (!x && (unpad ? padded : rows) > 0)) return fail(MDY_E_NULL, "group_pad_rows: null pointer");
+    if (int e = check_device()) return e;
+    return launched(mdy::launch_group_pad(x, y, m_splits, G, row_bytes, multiple, unpad, static_cast<hipStream_t>(stream)),
+                    "group_pad_rows");
+}
+
 int mdy_add_bias(void* x, const void* b, int64_t M, int64_t N, void* stream) {
     if (M < 0 || N < 0 || M > kMaxDim || N > kMaxDim) return fail(MDY_E_SHAPE, "add_bias: bad shape");
     if (M == 0 || N == 0) return 0;

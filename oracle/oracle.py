@@ -35,6 +35,9 @@ Pinning status (what fixes each function besides its own formula):
       compositions of the above (per group: fp8_gemm); checked against unquantized
       fp32 gradients within the quantization error band and for operand roles
       (swapping x and dy transposes wgrad).
+  fp8_padding / fp8_unpadding
+      pure row moves: brute-force row-by-row loops on small inputs, the round trip
+      unpad(pad(x)) == x, zero padding rows, slot starts at multiples of 256.
   fp8_matmul (DeepLinear's GEMM)
       PARITY UNPINNED at the third-party boundary: the reference calls
       `deep_gemm.gemm_fp8_fp8_bf16_nt` (dpsk_fp8linear/fp8.py:310; the grouped
@@ -418,3 +421,27 @@ def fp8_grouped_matmul(qa, sa, qb, sb, m_splits, bias: Optional[torch.Tensor] = 
                     else torch.empty(0, qb.size(1), dtype=torch.bfloat16))
         row += mg
     return torch.cat(outs, 0)
+
+
+def fp8_padding(inp: torch.Tensor, m_splits, multiple: int = 256):
+    """Fp8Padding (megatron_patchs/dpsk_grouped_linear.py:798-902): group g's m_splits[g] rows move to the start of a
+    slot of cdiv(m, 256) * 256 rows, the rest of the slot is zero (TransformerEngine's multi_padding_fused, called at
+    :817).  Returns (padded [sum pad(m), H], padded_m_splits)."""
+    x = inp.detach().cpu().reshape(-1, inp.shape[-1])
+    pads = [(int(m) + multiple - 1) // multiple * multiple for m in m_splits]
+    out = torch.zeros(sum(pads), x.size(1), dtype=x.dtype)
+    src = dst = 0
+    for m, pm in zip(m_splits, pads):
+        out[dst:dst + m] = x[src:src + m]
+        src += m
+        dst += pm
+    return out, pads
+
+
+def fp8_unpadding(inp: torch.Tensor, m_splits, multiple: int = 256) -> torch.Tensor:
+    """Fp8Unpadding (dpsk_grouped_linear.py:690-793): torch.split by the padded sizes, the first m_splits[g] rows of
+    every piece, torch.cat (:703-706)."""
+    x = inp.detach().cpu().reshape(-1, inp.shape[-1])
+    pads = [(int(m) + multiple - 1) // multiple * multiple for m in m_splits]
+    pieces = torch.split(x, pads)
+    return torch.cat([p[:m] for p, m in zip(pieces, m_splits)], 0)

@@ -245,3 +245,63 @@ def test_grouped_gemm_exact_integer_random_splits():
         N = int(rng.choice([128, 200, 256, 520, 776, 1024]))
         K = 128 * int(rng.integers(1, 6))
         exact_grouped_case(m_splits, N, K, 1000 + case, call_f32)
+
+
+# ------------------------------------------------------------------ Fp8Padding / Fp8Unpadding (dpsk_grouped_linear.py:690-902)
+@pytest.mark.parametrize("dtype,H", [(torch.bfloat16, 512), (torch.bfloat16, 7), (torch.uint8, 33), (torch.float32, 64)])
+def test_group_padding_bit_exact_and_round_trip(dtype, H):
+    """Every alignment path (16-, 2- and 1-byte pieces), empty groups, more groups than one launch takes."""
+    from mdy_triton_amd.megatron_patchs.dpsk_grouped_linear import Fp8Padding, Fp8Unpadding, pad_groups, unpad_groups
+    rng = np.random.default_rng(5)
+    for m_splits in ([3, 0, 256, 257, 1, 511], [100], [0, 0], [int(v) for v in rng.integers(0, 40, 300)]):
+        rows = sum(m_splits)
+        if dtype == torch.uint8:
+            x = torch.from_numpy(rng.integers(1, 255, (rows, H), dtype=np.uint8))
+        else:
+            x = torch.from_numpy(rng.standard_normal((rows, H)).astype(np.float32)).to(dtype)
+        want, pads = O.fp8_padding(x, m_splits)
+        with torch.no_grad():
+            got, got_pads = Fp8Padding(len(m_splits))(x.to(DEV), m_splits)
+        assert got_pads == pads and got.dtype == dtype and got.shape == want.shape
+        assert torch.equal(got.cpu().contiguous().flatten().view(torch.uint8), want.contiguous().flatten().view(torch.uint8))
+        with torch.no_grad():
+            back = Fp8Unpadding(len(m_splits))(got, m_splits)
+        assert torch.equal(back.cpu().contiguous().flatten().view(torch.uint8), x.contiguous().flatten().view(torch.uint8))
+        assert torch.equal(back.cpu().contiguous().flatten().view(torch.uint8), O.fp8_unpadding(want, m_splits).contiguous().flatten().view(torch.uint8))
+        # a destination full of garbage is overwritten everywhere (the padding rows are written, not assumed zero)
+        assert torch.equal(pad_groups(x.to(DEV), m_splits, multiple=64).cpu().contiguous().flatten().view(torch.uint8),
+                           O.fp8_padding(x, m_splits, 64)[0].contiguous().flatten().view(torch.uint8))
+        assert torch.equal(unpad_groups(pad_groups(x.to(DEV), m_splits, 64), m_splits, 64).cpu().contiguous().flatten().view(torch.uint8), x.contiguous().flatten().view(torch.uint8))
+    with pytest.raises(ValueError):
+        pad_groups(torch.zeros(5, 4, device=DEV), [2, 2])
+    with pytest.raises(AssertionError):
+        Fp8Padding(3)(torch.zeros(4, 4, device=DEV), [2, 2])
+
+
+def test_group_padding_autograd_pair_and_ragged_quantizer():
+    """Each direction is the other's gradient, and a ragged batch reaches the grouped quantizer (which wants groups
+    of multiples of 256 rows, fp8_matmul.py:227) through the padding: bytes and scales equal the oracle's on the
+    oracle's padded copy."""
+    from mdy_triton_amd.megatron_patchs.dpsk_grouped_linear import Fp8Padding, Fp8Unpadding
+    g = torch.Generator().manual_seed(8)
+    m_splits = [130, 0, 300, 17]
+    H = 512
+    x = torch.randn(sum(m_splits), H, generator=g).bfloat16()
+    xg = x.to(DEV).requires_grad_(True)
+    padded, pads = Fp8Padding(4)(xg, m_splits)
+    w = torch.randn(sum(pads), H, generator=g).bfloat16().to(DEV)
+    (padded.float() * w.float()).sum().backward()
+    assert torch.equal(xg.grad.cpu(), O.fp8_unpadding(w.cpu(), m_splits))
+    pg = padded.detach().clone().requires_grad_(True)
+    out = Fp8Unpadding(4)(pg, m_splits)
+    dy = torch.randn(sum(m_splits), H, generator=g).bfloat16().to(DEV)
+    out.backward(dy)
+    assert torch.equal(pg.grad.cpu(), O.fp8_padding(dy.cpu(), m_splits)[0])
+    # ragged batch -> padded -> grouped quantizer with transposed copies
+    y, s, yts, sts = m.group_per_token_cast_to_fp8(padded.detach(), pads)
+    ry, rs, ryts, rsts = O.group_per_token_cast_to_fp8(O.fp8_padding(x, m_splits)[0], pads)
+    assert torch.equal(y.cpu().contiguous().flatten().view(torch.uint8), ry.contiguous().flatten().view(torch.uint8)) and torch.equal(s.cpu(), rs)
+    for a, b in zip(yts, ryts):
+        assert torch.equal(a.cpu().contiguous().flatten().view(torch.uint8), b.contiguous().flatten().view(torch.uint8))
+    for a, b in zip(sts, rsts):
+        assert torch.equal(a.cpu().contiguous(), b.contiguous())

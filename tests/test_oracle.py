@@ -381,3 +381,26 @@ def test_grouped_oracle_functions_reduce_to_the_pinned_ones():
     out = O.fp8_grouped_matmul(qa, sa, qb, sb2, [300, 212])
     assert torch.equal(out[:300], O.fp8_gemm(qa[:300], sa.contiguous()[:300], qb[0], sb2[0]))
     assert torch.equal(out[300:], O.fp8_gemm(qa[300:], sa.contiguous()[300:], qb[1], sb2[1]))
+
+
+def test_fp8_padding_row_by_row():
+    """The padding pair against plain Python loops over rows (what the layout means, no tensor ops): every
+    source row lands at slot_start[g] + r, every other destination row is zero, and unpadding is the inverse."""
+    g = torch.Generator().manual_seed(31)
+    m_splits = [3, 0, 256, 257, 1, 511]
+    H = 5
+    x = torch.randn(sum(m_splits), H, generator=g).bfloat16()
+    padded, pads = O.fp8_padding(x, m_splits)
+    assert pads == [256, 0, 256, 512, 256, 512] and padded.shape == (sum(pads), H)
+    want = [[0.0] * H for _ in range(sum(pads))]
+    src = dst = 0
+    for m, pm in zip(m_splits, pads):
+        assert dst % 256 == 0
+        for r in range(m):
+            want[dst + r] = x[src + r].float().tolist()
+        src += m
+        dst += pm
+    assert padded.float().tolist() == want
+    back = O.fp8_unpadding(padded, m_splits)
+    assert torch.equal(back, x)
+    assert O.fp8_padding(x[:0], [0, 0])[0].shape == (0, H)
