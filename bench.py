@@ -74,6 +74,8 @@ def parse_args():
                     help="time the tile kernel with parts of its K loop switched off, with power and clock (no JSON)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload (skip C2, C4, C5 and the power loop)")
+    ap.add_argument("--only-decode", action="store_true",
+                    help="only the six decode shapes (C5): 200 eager calls each, then the graph replays; prints their JSON entries")
     ap.add_argument("--calib-copy", action="store_true",
                     help="first run one plain 256 MiB device-to-device copy kernel (counter calibration for rocprofv3 --pmc)")
     return ap.parse_args()
@@ -349,7 +351,7 @@ def kernel_entries(torch, m, timer, x, wq, ws, reps=12):
     }
 
 
-def decode_entries(torch, m, dev):
+def decode_entries(torch, m, dev, eager_calls=0):
     """The six decode / routed-expert shapes: per-call time inside a replayed HIP graph, against the HBM peak on the
     algorithmic bytes (weights + activations + scales + output).  The weights (14.7 MB) stay in the caches between
     the calls of a graph, so this is the kernel's speed, not a cold-memory figure."""
@@ -360,6 +362,8 @@ def decode_entries(torch, m, dev):
         w = torch.randn(N, K, generator=g).mul_(0.02).bfloat16().to(dev)
         wq, ws = quantize_weight(torch, w, dev)
         xq, xs = m.act_quant(x)
+        for _ in range(eager_calls):        # for a kernel trace: plain launches, one kernel record each
+            m.fp8_gemm(xq, xs, wq, ws, out_dtype=torch.bfloat16)
         us = graph_replay_us(torch, lambda: m.fp8_gemm(xq, xs, wq, ws, out_dtype=torch.bfloat16))
         aq_us = graph_replay_us(torch, lambda: m.act_quant(x))
         b = gemm_bytes(M, N, K)
@@ -386,6 +390,9 @@ def main():
     torch.cuda.set_device(dev)
     if args.ablation:
         ablation(torch, m, dev)
+        return
+    if args.only_decode:
+        print(json.dumps({"C5_graph_replay": decode_entries(torch, m, dev, eager_calls=200)}))
         return
     seed, kind, M, N, K, desc = WORKLOADS[args.workload]
     x, w = make_inputs(torch, kind, M, N, K, seed, dev)
