@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define MDY_FP8_ABI_VERSION 6
+#define MDY_FP8_ABI_VERSION 7
 
 /* error codes (negative = argument rejected before any launch) */
 #define MDY_OK 0
@@ -105,6 +105,36 @@ int mdy_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t, in
 int mdy_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
                         int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int64_t s_kb_stride,
                         int t_mode, void* stream);
+
+/* Official-dialect training quantizer (s = amax / 448, no clamp, no eps): the row-wise 1x128 quantization of x and
+ * the quantized transpose with one scale per column and 128 rows, one read of x.  Replaces the pair
+ * act_quant_block(x) / act_quant_block(x, transpose=True) (triton_kernels/deepseekv3/fp8_kernel.py:62-87, kernel
+ * :14-60) that the reference's Fp8Linear runs on x and on dy (:286-301).
+ *
+ *   x    bf16 [M, K], element (m, k) at x[m * x_row_stride + k * x_col_stride]
+ *   y    e4m3fn [PM, PK] row-major or NULL (then s must be NULL too: only the transposed copy is produced)
+ *   s    fp32 [PM, PK/128] row-major
+ *   y_t  e4m3fn [PK, PM] row-major: y_t[k, m] = x[m, k] / s_t[k, m / 128]
+ *   s_t  fp32 [PK, PM/128] row-major
+ * PM >= M and PK >= K are multiples of 128; padding reads as 0 (an all-zero group has scale 0 and NaN bytes, as in the
+ * reference).  y / y_t 8-byte aligned.
+ */
+int mdy_act_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
+                            int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, void* stream);
+
+/* Block-scaled FP8 GEMM, NT layout, with 1x128 scales on both operands:
+ *   c[m, n] = sum_kb (sum_{k in kb} a[m,k] * b[n,k]) * a_s[m, kb] * b_s[n, kb]
+ * Replaces fp8_matmul(..., have_w=False) (triton_kernels/deepseekv3/fp8_kernel.py:214-252, kernel branch :190-205),
+ * the weight-gradient GEMM of the reference's Fp8Linear (fp8_matmul_bwd, :254-257).
+ *
+ *   a   e4m3fn [M, K] row-major, 16-byte aligned     a_s fp32, element (m, kb) at a_s[m * as_row_stride + kb * as_col_stride]
+ *   b   e4m3fn [N, K] row-major, 16-byte aligned     b_s fp32, element (n, kb) at b_s[n * bs_row_stride + kb * bs_col_stride]
+ *   c   [M, N] row-major of out_dtype
+ * K % 128 == 0, K <= 2^20; scale strides non-negative, each scale tensor spanning less than 2^31 bytes.
+ */
+int mdy_fp8_gemm_nt_rowscaled(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
+                              const void* b, const float* b_s, int64_t bs_row_stride, int64_t bs_col_stride, void* c,
+                              int64_t M, int64_t N, int64_t K, int out_dtype, void* stream);
 
 /* SwiGLU, alone or fused with the 1x128 activation quantizer that feeds the next GEMM.
  *   act[m, n] = bf16( silu(gate[m, n]) * up[m, n] ), silu(g) = g / (1 + exp(-g)) in fp32;

@@ -10,7 +10,7 @@ import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libmdyfp8.so")
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 _lock = threading.Lock()
 _lib = None
@@ -25,6 +25,8 @@ SIGNATURES = {
     "mdy_weight_quant": [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p],
     "mdy_quant_transpose": [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p],
     "mdy_fp8_grouped_gemm_nt": [_p, _p, _i64, _i64, _p, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p],
+    "mdy_act_quant_transpose": [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p],
+    "mdy_fp8_gemm_nt_rowscaled": [_p, _p, _i64, _i64, _p, _p, _i64, _i64, _p, _i64, _i64, _i64, _int, _p],
     "mdy_swiglu": [_p, _p, _p, _p, _i64, _i64, _i64, _int, _i64, _i64, _i64, _i64, _int, _p],
     "mdy_swiglu_bwd": [_p, _p, _p, _i64, _i64, _i64, _int, _p],
     "mdy_weight_dequant": [_p, _p, _p, _i64, _i64, _int, _p],

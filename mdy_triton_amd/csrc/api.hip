@@ -106,6 +106,40 @@ int mdy_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t,
                     "quant_transpose");
 }
 
+int mdy_act_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
+                            int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, void* stream) {
+    if (M < 0 || K < 0 || PM < M || PK < K || PM > kMaxDim || PK > kMaxDim)
+        return fail(MDY_E_SHAPE, "act_quant_transpose: need 0 <= M <= PM, 0 <= K <= PK");
+    if (PM % 128 != 0 || PK % 128 != 0) return fail(MDY_E_SHAPE, "act_quant_transpose: PM=%lld, PK=%lld must be multiples of 128", (long long)PM, (long long)PK);
+    if ((y == nullptr) != (s == nullptr)) return fail(MDY_E_NULL, "act_quant_transpose: y and s must be given together");
+    if (PM == 0 || PK == 0) return 0;
+    if (!y_t || !s_t || (!x && M > 0 && K > 0)) return fail(MDY_E_NULL, "act_quant_transpose: null pointer");
+    if ((y && !aligned(y, 8)) || !aligned(y_t, 8)) return fail(MDY_E_ALIGN, "act_quant_transpose: y / y_t must be 8-byte aligned");
+    if (!aligned(x, 2) || (s && !aligned(s, 4)) || !aligned(s_t, 4)) return fail(MDY_E_ALIGN, "act_quant_transpose: x/s/s_t misaligned for their element type");
+    if (int e = check_device()) return e;
+    return launched(mdy::launch_act_quant_transpose(x, y, s, y_t, s_t, M, K, x_row_stride, x_col_stride, PM, PK,
+                                                    static_cast<hipStream_t>(stream)),
+                    "act_quant_transpose");
+}
+
+int mdy_fp8_gemm_nt_rowscaled(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,
+                              const float* b_s, int64_t bs_row_stride, int64_t bs_col_stride, void* c, int64_t M, int64_t N,
+                              int64_t K, int out_dtype, void* stream) {
+    if (out_dtype != MDY_DT_BF16 && out_dtype != MDY_DT_F32) return fail(MDY_E_DTYPE, "fp8_gemm_nt_rowscaled: unknown out_dtype %d", out_dtype);
+    if (M < 0 || N < 0 || K < 128 || K % 128 != 0 || M > kMaxDim || N > kMaxDim || K > (1 << 20))
+        return fail(MDY_E_SHAPE, "fp8_gemm_nt_rowscaled: needs K a multiple of 128 up to 2^20 (M=%lld N=%lld K=%lld)", (long long)M,
+                    (long long)N, (long long)K);
+    if (M == 0 || N == 0) return 0;
+    if (!a || !a_s || !b || !b_s || !c) return fail(MDY_E_NULL, "fp8_gemm_nt_rowscaled: null pointer");
+    if (!aligned(a, 16) || !aligned(b, 16) || !aligned(c, out_dtype == MDY_DT_BF16 ? 2 : 4) || !aligned(a_s, 4) || !aligned(b_s, 4))
+        return fail(MDY_E_ALIGN, "fp8_gemm_nt_rowscaled: a and b must be 16-byte aligned, c and the scales aligned for their type");
+    if (int e = check_device()) return e;
+    const int rc = mdy::launch_fp8_gemm_nt_rowscaled(a, a_s, as_row_stride, as_col_stride, b, b_s, bs_row_stride, bs_col_stride, c,
+                                                     M, N, K, out_dtype, static_cast<hipStream_t>(stream));
+    if (rc == -1) return fail(MDY_E_SHAPE, "fp8_gemm_nt_rowscaled: scale strides must be non-negative and span less than 2^31 bytes");
+    return launched(rc, "fp8_gemm_nt_rowscaled");
+}
+
 int mdy_swiglu(const void* x, void* act, void* y, float* s, int64_t M, int64_t N, int64_t x_row_stride, int gate_first,
                int64_t PM, int64_t PN, int64_t s_row_stride, int64_t s_col_stride, int mode, void* stream) {
     if (M < 0 || N < 0 || M > kMaxDim || 2 * N > kMaxDim) return fail(MDY_E_SHAPE, "swiglu: bad shape M=%lld N=%lld", (long long)M, (long long)N);

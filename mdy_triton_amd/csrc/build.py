@@ -9,7 +9,7 @@ import sys
 from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SOURCES = ["api.hip", "act_quant.hip", "weight_quant.hip", "quant_transpose.hip", "swiglu.hip", "weight_dequant.hip", "fp8_gemm.hip", "gemm_probe.hip", "group_pad.hip", "add_bias.hip"]
+SOURCES = ["api.hip", "act_quant.hip", "weight_quant.hip", "quant_transpose.hip", "swiglu.hip", "weight_dequant.hip", "fp8_gemm.hip", "gemm_probe.hip", "fp8_gemm_rowscaled.hip", "group_pad.hip", "add_bias.hip"]
 LIB = os.path.join(HERE, "libmdyfp8.so")
 
 # -packed-fp32-ops: keep the compiler from forming v_pk_{add,mul,fma}_f32.

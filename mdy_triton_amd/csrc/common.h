@@ -190,6 +190,11 @@ int launch_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t,
 int launch_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
                            int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int64_t s_kb_stride,
                            int t_mode, hipStream_t stream);
+int launch_act_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
+                               int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, hipStream_t stream);
+int launch_fp8_gemm_nt_rowscaled(const void* a, const float* a_s, int64_t as_rs, int64_t as_cs, const void* b,
+                                 const float* b_s, int64_t bs_rs, int64_t bs_cs, void* c, int64_t M, int64_t N, int64_t K,
+                                 int out_dtype, hipStream_t stream);
 int launch_swiglu(const void* x, void* act, void* y, float* s, int64_t M, int64_t N, int64_t x_row_stride,
                   int gate_first, int64_t PM, int64_t PN, int64_t s_row_stride, int64_t s_col_stride, int mode,
                   hipStream_t stream);

@@ -2,7 +2,9 @@
 //   (1) the row-wise 1x128 quantization y[PM,PK] with scales s[kb*s_kb_stride + m]      (as the forward quantizer), and
 //   (2) the quantized TRANSPOSE y_t[PK,PM], scaled either per 128x1 column group (t_mode 0) or per
 //       128x128 block (t_mode 1),
-// both in the DeepLinear dialect (scale = (min(amax,1e4) + 1e-8) / 448, saturating cast).
+// in the DeepLinear dialect (MODE 1: scale = (min(amax,1e4) + 1e-8) / 448, saturating cast) or, per column group only,
+// in the official dialect (MODE 0: scale = amax / 448, no clamp, no eps: act_quant_block(x) and
+// act_quant_block(x, transpose=True) of /root/reference/triton_kernels/deepseekv3/fp8_kernel.py:14-87 in one pass).
 //
 // Restates _quant_grad_output_kernel (/root/reference/triton_kernels/dpsk_fp8linear/fp8.py:13-44;
 // t_mode 0: second half at :40-44 quantizes along axis 0 and stores ST[off_n + pid_m*PN]) and the
@@ -21,20 +23,25 @@
 
 namespace mdy {
 
-// x / s in the DeepLinear dialect.  FAST (amax <= 1e4, so |x/s| <= 448 needs no clamp) uses the
-// reciprocal form; otherwise an IEEE division saturated at +-448 (NaN kept).
-template <bool FAST>
+// x / s.  FAST (the group's amax lies where the reciprocal form is proven bit-identical to IEEE division and,
+// in the DeepLinear dialect, amax <= 1e4, so |x/s| <= 448 needs no clamp) uses the reciprocal form; otherwise an
+// IEEE division, saturated at +-448 in the DeepLinear dialect (NaN kept).
+template <int MODE, bool FAST>
 __device__ __forceinline__ float qt_quot(float x, float s, float r) {
     if (FAST) return fast_quotient(x, s, r);
-    return sat_for_mode<1>(x / s);
+    return sat_for_mode<MODE>(x / s);
 }
 
-template <int TMODE, bool VEC, int RPT>
+// Scale layouts: row scale of row m, K group kb at s[kb * s_kb_stride + m * s_m_stride]; column-group scale of
+// column k, row group a at s_t[a * st_a_stride + k * st_k_stride] (TMODE 0) / block scale at s_t[kb * (PM/128) + a]
+// (TMODE 1).  y may be null (MODE 0 callers that only want the transposed copy): the row-wise outputs are skipped.
+template <int MODE, int TMODE, bool VEC, int RPT>
 __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ y,
                                                                float* __restrict__ s, uint8_t* __restrict__ y_t,
                                                                float* __restrict__ s_t, int M, int K,
                                                                int64_t x_row_stride, int64_t x_col_stride, int PM,
-                                                               int PK, int64_t s_kb_stride) {
+                                                               int PK, int64_t s_kb_stride, int64_t s_m_stride,
+                                                               int64_t st_a_stride, int64_t st_k_stride) {
     constexpr int NRG = 128 / RPT;        // row groups of RPT consecutive rows; 16 threads (8 columns each) per group
     constexpr int WAVES = NRG / 4;
     __shared__ float col_part[WAVES][128];  // per wave (4 row groups) partial column maxima
@@ -88,17 +95,17 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
 
     // ---- (1) row-wise quantization straight from registers
 #pragma unroll
-    for (int i = 0; i < RPT; ++i) {
+    for (int i = 0; i < (y != nullptr ? RPT : 0); ++i) {
         const int row = bm * 128 + rg * RPT + i;    // < PM
-        const float sc = group_scale<1>(rmax[i]);
+        const float sc = group_scale<MODE>(rmax[i]);
         const float r = 1.0f / sc;
         float q[8];
-        if (group_is_fast<1>(rmax[i])) {
+        if (group_is_fast<MODE>(rmax[i])) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) q[j] = qt_quot<true>(f[i][j], sc, r);
+            for (int j = 0; j < 8; ++j) q[j] = qt_quot<MODE, true>(f[i][j], sc, r);
         } else {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) q[j] = qt_quot<false>(f[i][j], sc, r);
+            for (int j = 0; j < 8; ++j) q[j] = qt_quot<MODE, false>(f[i][j], sc, r);
         }
         store_nt8(y + (int64_t)row * PK + c0, make_uint2(pack4_e4m3(q[0], q[1], q[2], q[3]), pack4_e4m3(q[4], q[5], q[6], q[7])));
         if ((t & 15) == 0) row_sc[rg * RPT + i] = sc;
@@ -120,13 +127,12 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
             float m = 0.0f;
 #pragma unroll
             for (int g = 0; g < WAVES; ++g) m = fmaxf(m, col_part[g][t]);
-            const float sc = group_scale<1>(m);
+            const float sc = group_scale<MODE>(m);
             col_amax[t] = m;
             col_sc[t] = sc;
             col_rc[t] = 1.0f / sc;
-            // logical s_t[k, a]: stored [A][PK]
-            s_t[(int64_t)bm * PK + bk * 128 + t] = sc;
-            s[(int64_t)bk * s_kb_stride + bm * 128 + t] = row_sc[t];
+            s_t[(int64_t)bm * st_a_stride + (int64_t)(bk * 128 + t) * st_k_stride] = sc;
+            if (y != nullptr) s[(int64_t)bk * s_kb_stride + (int64_t)(bm * 128 + t) * s_m_stride] = row_sc[t];
         }
         __syncthreads();
 #pragma unroll
@@ -146,9 +152,9 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
         float bmax = blk_part[0];
 #pragma unroll
         for (int w = 1; w < WAVES; ++w) bmax = fmaxf(bmax, blk_part[w]);
-        if (t == 0) s_t[(int64_t)bk * (PM >> 7) + bm] = group_scale<1>(bmax);
-        if (t < 128) s[(int64_t)bk * s_kb_stride + bm * 128 + t] = row_sc[t];
-        const float bsc = group_scale<1>(bmax), brc = 1.0f / bsc;
+        if (t == 0) s_t[(int64_t)bk * (PM >> 7) + bm] = group_scale<MODE>(bmax);
+        if (t < 128 && y != nullptr) s[(int64_t)bk * s_kb_stride + (int64_t)(bm * 128 + t) * s_m_stride] = row_sc[t];
+        const float bsc = group_scale<MODE>(bmax), brc = 1.0f / bsc;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             tamax[j] = bmax;
@@ -158,17 +164,17 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
     }
     bool tfast = true;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) tfast = tfast && group_is_fast<1>(tamax[j]);
+    for (int j = 0; j < 8; ++j) tfast = tfast && group_is_fast<MODE>(tamax[j]);
     uint32_t qlo[RPT], qhi[RPT];   // row i of the transposed copy's bytes: columns 0..3 | 4..7
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
         float q[8];
         if (tfast) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) q[j] = qt_quot<true>(f[i][j], tsc[j], tr[j]);
+            for (int j = 0; j < 8; ++j) q[j] = qt_quot<MODE, true>(f[i][j], tsc[j], tr[j]);
         } else {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) q[j] = qt_quot<false>(f[i][j], tsc[j], tr[j]);
+            for (int j = 0; j < 8; ++j) q[j] = qt_quot<MODE, false>(f[i][j], tsc[j], tr[j]);
         }
         qlo[i] = pack4_e4m3(q[0], q[1], q[2], q[3]);
         qhi[i] = pack4_e4m3(q[4], q[5], q[6], q[7]);
@@ -206,9 +212,11 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
     }
 }
 
-int launch_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
-                           int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int64_t s_kb_stride,
-                           int t_mode, hipStream_t stream) {
+// Shared launcher.  mode: dialect (0 official, column groups only; 1 DeepLinear); t_mode: 0 per column group, 1 per
+// 128x128 block.
+static int launch_qt(int mode, const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
+                     int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int64_t s_kb_stride,
+                     int64_t s_m_stride, int64_t st_a_stride, int64_t st_k_stride, int t_mode, hipStream_t stream) {
     if (PM == 0 || PK == 0) return 0;
     dim3 grid;
     if (!grid_rows(PK / 128, PM / 128, grid)) return kErrTooManyBlocks;
@@ -220,22 +228,39 @@ int launch_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     uint8_t* yp = static_cast<uint8_t*>(y);
     uint8_t* ytp = static_cast<uint8_t*>(y_t);
-#define MDY_QT(TM, VEC)                                                                                                 \
+#define MDY_QT(MODE, TM, VEC)                                                                                           \
     do {                                                                                                                \
         if (wide)                                                                                                       \
-            hipLaunchKernelGGL((quant_transpose_kernel<TM, VEC, 4>), grid, block, 0, stream, xp, yp, s, ytp, s_t, (int)M, \
-                               (int)K, x_row_stride, x_col_stride, (int)PM, (int)PK, s_kb_stride);                      \
+            hipLaunchKernelGGL((quant_transpose_kernel<MODE, TM, VEC, 4>), grid, block, 0, stream, xp, yp, s, ytp, s_t, \
+                               (int)M, (int)K, x_row_stride, x_col_stride, (int)PM, (int)PK, s_kb_stride, s_m_stride,   \
+                               st_a_stride, st_k_stride);                                                               \
         else                                                                                                            \
-            hipLaunchKernelGGL((quant_transpose_kernel<TM, VEC, 8>), grid, block, 0, stream, xp, yp, s, ytp, s_t, (int)M, \
-                               (int)K, x_row_stride, x_col_stride, (int)PM, (int)PK, s_kb_stride);                      \
+            hipLaunchKernelGGL((quant_transpose_kernel<MODE, TM, VEC, 8>), grid, block, 0, stream, xp, yp, s, ytp, s_t, \
+                               (int)M, (int)K, x_row_stride, x_col_stride, (int)PM, (int)PK, s_kb_stride, s_m_stride,   \
+                               st_a_stride, st_k_stride);                                                               \
     } while (0)
-    if (t_mode == 0) {
-        if (vec) MDY_QT(0, true); else MDY_QT(0, false);
+    if (mode == 0) {
+        if (vec) MDY_QT(0, 0, true); else MDY_QT(0, 0, false);
+    } else if (t_mode == 0) {
+        if (vec) MDY_QT(1, 0, true); else MDY_QT(1, 0, false);
     } else {
-        if (vec) MDY_QT(1, true); else MDY_QT(1, false);
+        if (vec) MDY_QT(1, 1, true); else MDY_QT(1, 1, false);
     }
 #undef MDY_QT
     return (int)hipGetLastError();
+}
+
+int launch_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
+                           int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int64_t s_kb_stride,
+                           int t_mode, hipStream_t stream) {
+    // DeepLinear layouts: row scales [PK/128][s_kb_stride >= PM], column-group scales [PM/128][PK]
+    return launch_qt(1, x, y, s, y_t, s_t, M, K, x_row_stride, x_col_stride, PM, PK, s_kb_stride, 1, PK, 1, t_mode, stream);
+}
+
+int launch_act_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
+                               int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, hipStream_t stream) {
+    // official layouts, both row-major: s [PM][PK/128], s_t [PK][PM/128]
+    return launch_qt(0, x, y, s, y_t, s_t, M, K, x_row_stride, x_col_stride, PM, PK, 1, PK / 128, 1, PM / 128, 0, stream);
 }
 
 }  // namespace mdy

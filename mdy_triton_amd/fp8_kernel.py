@@ -3,7 +3,9 @@
 Drop-in for the parts of /root/reference/triton_kernels/deepseekv3/fp8_kernel.py that sit
 directly before the FP8 linear path: silu_fwd / silu_bwd / triton_silu (fp8_kernel.py:384-434),
 weight_quant_block (:124-138), plus silu_act_quant, which fuses the `silu_fwd -> act_quant`
-pair of the FP8 MLP (fp8_kernel.py:447-450, 500-515) into one pass over the up/gate tensor.
+pair of the FP8 MLP (fp8_kernel.py:447-450, 500-515) into one pass over the up/gate tensor; and for
+that file's own linear layer in the official dialect (s = amax / finfo.max, no clamp, no eps):
+act_quant_block (:62-87), fp8_matmul (:214-252), fp8_matmul_bwd (:254-257), Fp8Linear (:259-313).
 Only float8_e4m3fn is implemented (the reference defaults to e5m2 but its notebook passes
 e4m3fn, deepseekv3/fp8-benchmark.ipynb line 78).
 """
@@ -139,6 +141,167 @@ def weight_quant_block(x: torch.Tensor, BLOCK_M: int = 128, BLOCK_N: int = 128,
         check(lib().mdy_weight_quant(ptr(x), ptr(y), ptr(s), None, None, M, N, x.stride(0), x.stride(1), M, N, 0,
                                      stream_ptr(dev)), "weight_quant_block")
     return y, s
+
+
+def _act_quant_transposed(x2: torch.Tensor, with_rows: bool, who: str):
+    """x2 [M, N] bf16 (any strides) -> (y, s, y_t_padded, s_t): the official-dialect row-wise quantization (None, None
+    unless with_rows) and the quantized transpose y_t [N, PM] with s_t [N, PM/128], PM = cdiv(M, 128) * 128."""
+    if x2.dtype != torch.bfloat16:
+        raise TypeError("%s expects a bfloat16 tensor, got %s" % (who, x2.dtype))
+    dev = require_gpu(x2)
+    M, N = x2.shape
+    PM = (M + 127) // 128 * 128
+    y = torch.empty(PM, N, device=dev, dtype=FP8) if with_rows else None
+    s = torch.empty(PM, N // 128, device=dev, dtype=torch.float32) if with_rows else None
+    y_t = torch.empty(N, PM, device=dev, dtype=FP8)
+    s_t = torch.empty(N, PM // 128, device=dev, dtype=torch.float32)
+    if PM * N > 0:
+        with on_device(dev):
+            check(lib().mdy_act_quant_transpose(ptr(x2), ptr(y), ptr(s), ptr(y_t), ptr(s_t), M, N, x2.stride(0), x2.stride(1),
+                                                PM, N, stream_ptr(dev)), who)
+    return y, s, y_t, s_t
+
+
+def act_quant_block(x: torch.Tensor, transpose: bool = False, dtype: torch.dtype = FP8,
+                    BLOCK_N: int = 128) -> Tuple[torch.Tensor, torch.Tensor]:
+    """1x128 quantizer with s = amax / 448 (fp8_kernel.py:62-87).
+
+    transpose=False: (y like x, s [..., N/128]), the same as offical_kernel.act_quant.  transpose=True: the
+    flattened [M, N] input is quantized along M: y [N, M], s [N, cdiv(M, 128)] (a last group shorter than 128 is
+    completed with zeros, as the reference's masked loads do).
+    """
+    assert x.size(-1) % BLOCK_N == 0
+    if BLOCK_N != 128:
+        raise ValueError("only BLOCK_N=128 is implemented (the reference default)")
+    _require_e4m3(dtype, "act_quant_block")
+    if not transpose:
+        from .offical_kernel import act_quant
+        return act_quant(x if x.is_contiguous() else x.contiguous())
+    x2 = x.reshape(-1, x.size(-1))
+    M = x2.size(0)
+    _, _, y_t, s_t = _act_quant_transposed(x2, False, "act_quant_block")
+    return (y_t if y_t.size(1) == M else y_t[:, :M].contiguous()), s_t
+
+
+def fp8_matmul(x: torch.Tensor, w: torch.Tensor, scale_x: torch.Tensor, scale_w: torch.Tensor,
+               bias: Optional[torch.Tensor] = None, have_w: bool = True) -> torch.Tensor:
+    """bf16 y = x . w^T on block-scaled FP8 operands (fp8_kernel.py:214-252).
+
+    have_w=True (forward, input gradient): x [..., K] with scale_x [..., K/128], w [N, K] with 128x128 block scales
+    scale_w [N/128, K/128], optional bias [N] added in fp32.  have_w=False (weight gradient): x [M, K] and w [N, K]
+    both carry one scale per row and 128 columns, scale_x [M, cdiv(K,128)], scale_w [N, cdiv(K,128)]; a K that is not a
+    multiple of 128 is completed with zeros.
+    """
+    if x.dtype != FP8 or w.dtype != FP8:
+        raise TypeError("fp8_matmul expects float8_e4m3fn operands")
+    if have_w:
+        assert x.size(-1) % 128 == 0, 'in forward x @ w.T'
+        from .offical_kernel import fp8_gemm
+        x2 = x.reshape(-1, x.size(-1))
+        y = fp8_gemm(x2 if x2.is_contiguous() else x2.contiguous(), scale_x.reshape(-1, scale_x.size(-1)).contiguous(),
+                     w if w.is_contiguous() else w.contiguous(), scale_w.contiguous(), out_dtype=torch.bfloat16,
+                     bias=None if bias is None else bias.to(torch.bfloat16).contiguous())
+        return y.view(*x.shape[:-1], -1)
+    assert x.size(0) % 128 == 0, 'in backward dy.T @ x or dy @ w'
+    assert bias is None
+    dev = require_gpu(x, w, scale_x, scale_w)
+    x2 = x.reshape(-1, x.size(-1))
+    M, K = x2.shape
+    N = w.size(0)
+    if w.size(1) != K or tuple(scale_x.shape[-2:]) != (M, (K + 127) // 128) or tuple(scale_w.shape) != (N, (K + 127) // 128):
+        raise ValueError("shape mismatch: x %s scale_x %s w %s scale_w %s" % (tuple(x.shape), tuple(scale_x.shape), tuple(w.shape),
+                                                                                tuple(scale_w.shape)))
+    return _matmul_rowscaled(x2, scale_x.reshape(M, -1), w, scale_w, M, N, K, dev)
+
+
+def _matmul_rowscaled(x2, sx, w, sw, M, N, K, dev):
+    """[M, K] . [N, K]^T with per-row scales on both sides; operands may be column slices of K-padded buffers."""
+    PK = (K + 127) // 128 * 128
+
+    def k_padded(t):      # a [rows, K] view whose storage already runs to a multiple of 128 columns, zero filled
+        if K == PK and t.stride(1) == 1 and t.stride(0) == K and t.data_ptr() % 16 == 0:
+            return t
+        full = torch.zeros(t.size(0), PK, device=dev, dtype=torch.uint8)
+        full[:, :K] = t.view(torch.uint8)
+        return full.view(FP8)
+    a, b = k_padded(x2), k_padded(w)
+    out = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
+    if M * N == 0:
+        return out
+    with on_device(dev):
+        check(lib().mdy_fp8_gemm_nt_rowscaled(ptr(a), ptr(sx), sx.stride(0), sx.stride(1), ptr(b), ptr(sw), sw.stride(0),
+                                              sw.stride(1), ptr(out), M, N, PK, 0, stream_ptr(dev)), "fp8_matmul")
+    return out
+
+
+def fp8_matmul_bwd(xt, w, dy, dyt, scale_xt, scale_w, scale_dy, scale_dyt):
+    """Input and weight gradient of y = x . w^T from the quantized copies (fp8_kernel.py:254-257)."""
+    dx = fp8_matmul(dy, w, scale_dy, scale_w, have_w=True)
+    dw = fp8_matmul(dyt, xt, scale_dyt, scale_xt, have_w=False)
+    return dx, dw
+
+
+class _Fp8LinearFunction(torch.autograd.Function):
+    """fp8_kernel.py:259-301.  Forward: act_quant_block(x), weight_quant_block(w), GEMM with the bias in its epilogue.
+    Backward: x and dy quantized along the tokens (transposed copies, one kernel pass over dy for both of its copies),
+    w^T block-quantized; dx = dy . w through the tile kernels, dw = dy^T . x through the GEMM with row scales on both
+    operands.  The transposed copies keep their zero padding to a multiple of 128 tokens, so any token count works."""
+
+    @staticmethod
+    def forward(ctx, x, w, bias, fp8_dtype):
+        _require_e4m3(fp8_dtype, "Fp8Linear")
+        input_shape = x.shape
+        x2 = x.reshape(-1, input_shape[-1])
+        qx, sx = act_quant_block(x2, dtype=fp8_dtype)
+        qw, sw = weight_quant_block(w, dtype=fp8_dtype)
+        y = fp8_matmul(qx, qw, sx, sw, bias, have_w=True)
+        ctx.save_for_backward(x2, w)
+        ctx.bias = bias
+        ctx.fp8_dtype = fp8_dtype
+        ctx.input_shape = input_shape
+        return y.view(*input_shape[:-1], -1)
+
+    @staticmethod
+    def backward(ctx, dy):
+        dy2 = dy.reshape(-1, dy.size(-1))
+        if dy2.dtype != torch.bfloat16:
+            dy2 = dy2.to(torch.bfloat16)
+        dbias = dy2.sum(0) if ctx.bias is not None and ctx.needs_input_grad[2] else None
+        x2, w = ctx.saved_tensors
+        M, K = x2.shape
+        N = w.size(0)
+        dev = x2.device
+        dx = dw = None
+        need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        qdy, sdy, qdyt, sdyt = _act_quant_transposed(dy2, need_dx, "Fp8Linear.backward")
+        if need_dx:
+            qwt, swt = weight_quant_block(w.t(), dtype=ctx.fp8_dtype)       # [K, N], blocks of w^T
+            dx = fp8_matmul(qdy[:M], qwt, sdy[:M], swt, have_w=True).view(ctx.input_shape)
+        if need_dw:
+            _, _, qxt, sxt = _act_quant_transposed(x2, False, "Fp8Linear.backward")
+            PM = qdyt.size(1)
+            dw = torch.empty(N, K, device=dev, dtype=torch.bfloat16)
+            with on_device(dev):
+                check(lib().mdy_fp8_gemm_nt_rowscaled(ptr(qdyt), ptr(sdyt), sdyt.stride(0), sdyt.stride(1), ptr(qxt), ptr(sxt),
+                                                      sxt.stride(0), sxt.stride(1), ptr(dw), N, K, PM, 0, stream_ptr(dev)),
+                      "Fp8Linear.backward")
+        return dx, dw, dbias, None
+
+
+fp8_linear_with_quant_ops = _Fp8LinearFunction.apply
+
+
+class Fp8Linear(torch.nn.Linear):
+    """nn.Linear on the official-dialect FP8 path (fp8_kernel.py:303-313).  Only float8_e4m3fn is implemented; the
+    reference's default, float8_e5m2, raises TypeError."""
+
+    def __init__(self, in_features, out_features, bias=True, device=None, dtype=None, fp8_dtype=FP8):
+        super().__init__(in_features, out_features, bias, device, dtype)
+        _require_e4m3(fp8_dtype, "Fp8Linear")
+        self.fp8_dtype = fp8_dtype
+
+    def forward(self, x):
+        return fp8_linear_with_quant_ops(x, self.weight, self.bias, self.fp8_dtype)
 
 
 class _Fp8MlpCkptOps(torch.autograd.Function):

@@ -35,6 +35,11 @@ Pinning status (what fixes each function besides its own formula):
       compositions of the above (per group: fp8_gemm); checked against unquantized
       fp32 gradients within the quantization error band and for operand roles
       (swapping x and dy transposes wgrad).
+  act_quant_block / fp8_matmul_official / fp8_linear_forward / fp8_linear_backward  (the reference's Fp8Linear)
+      act_quant_block(x) is act_quant; act_quant_block(x, transpose=True) must equal act_quant of the zero-padded
+      transposed matrix (checked, with a brute-force group loop on top); the GEMM with row scales on both operands
+      against a float64 evaluation of its formula, exactly-representable integer cases, and its reduction to the
+      pinned fp8_gemm when the weight-row scales are constant within each 128-row block.
   fp8_padding / fp8_unpadding
       pure row moves: brute-force row-by-row loops on small inputs, the round trip
       unpad(pad(x)) == x, zero padding rows, slot starts at multiples of 256.
@@ -445,3 +450,68 @@ def fp8_unpadding(inp: torch.Tensor, m_splits, multiple: int = 256) -> torch.Ten
     pads = [(int(m) + multiple - 1) // multiple * multiple for m in m_splits]
     pieces = torch.split(x, pads)
     return torch.cat([p[:m] for p, m in zip(pieces, m_splits)], 0)
+
+
+# ---------------------------------------------------------------------------
+# The official-dialect linear layer of deepseekv3/fp8_kernel.py (Fp8Linear)
+# ---------------------------------------------------------------------------
+def act_quant_block(x: torch.Tensor, transpose: bool = False):
+    """fp8_kernel.py:62-87 (kernel :14-60): s = max|group| / 448 over 128 consecutive elements of a row, y = x / s
+    cast to e4m3fn, no clamp, no eps.  transpose=True quantizes x^T (the flattened [M, N] input along M); a last
+    group shorter than 128 is completed with zeros (the kernel's boundary_check / padding_option='zero', :47-50).
+    Returns (y, s): y like x and s [..., N/128], or y [N, M] and s [N, cdiv(M, 128)]."""
+    x2 = x.detach().cpu().float().reshape(-1, x.shape[-1])
+    if transpose:
+        x2 = x2.t()
+    R, C = x2.shape
+    PC = _cdiv(C, BLOCK) * BLOCK
+    xp = torch.zeros(R, PC, dtype=torch.float32)
+    xp[:, :C] = x2
+    g = xp.reshape(R, PC // BLOCK, BLOCK)
+    s = g.abs().amax(-1) / FP8_MAX
+    y = (g / s[:, :, None]).to(FP8).reshape(R, PC)[:, :C].contiguous()
+    if transpose:
+        return y, s
+    return y.reshape(x.shape), s.reshape(*x.shape[:-1], PC // BLOCK)
+
+
+def fp8_matmul_official(x, w, scale_x, scale_w, bias: Optional[torch.Tensor] = None, have_w: bool = True) -> torch.Tensor:
+    """fp8_kernel.py:214-252.  have_w=True: the block-scaled GEMM of offical_kernel.py with the bias added in fp32
+    before the bf16 cast (:207-209) - the weight scale of output column n is row n // 128 of scale_w (the kernel's
+    `pid_n * stride_sw1` with 256-wide tiles addresses other rows; that indexing slip is not followed).  have_w=False:
+    both operands carry one scale per row and 128 columns (:196-203): y = dequant(x) . dequant(w)^T."""
+    if have_w:
+        x2 = x.reshape(-1, x.shape[-1])
+        return fp8_gemm(x2, scale_x.reshape(x2.size(0), -1), w, scale_w, dtype=torch.bfloat16, bias=bias).reshape(*x.shape[:-1], -1)
+    assert bias is None
+
+    def deq(q, s):
+        q = q.detach().cpu().float()
+        R, C = q.shape
+        PC = _cdiv(C, BLOCK) * BLOCK
+        qp = torch.zeros(R, PC)
+        qp[:, :C] = q
+        return (qp.reshape(R, PC // BLOCK, BLOCK) * s.detach().cpu().float().reshape(R, -1)[:, :, None]).reshape(R, PC)
+    return (deq(x, scale_x) @ deq(w, scale_w).t()).to(torch.bfloat16)
+
+
+def fp8_linear_forward(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """_Fp8LinearFunction.forward (fp8_kernel.py:261-272)."""
+    x2 = x.detach().cpu().reshape(-1, x.shape[-1])
+    qx, sx = act_quant_block(x2)
+    qw, sw = weight_quant_block(w.detach().cpu())
+    return fp8_matmul_official(qx, qw, sx, sw, bias, True).reshape(*x.shape[:-1], -1)
+
+
+def fp8_linear_backward(x: torch.Tensor, w: torch.Tensor, dy: torch.Tensor, has_bias: bool = True):
+    """_Fp8LinearFunction.backward (fp8_kernel.py:274-301): (dx, dw, dbias)."""
+    x2 = x.detach().cpu().reshape(-1, x.shape[-1])
+    dy2 = dy.detach().cpu().reshape(-1, dy.shape[-1])
+    dbias = dy2.sum(0) if has_bias else None
+    qxt, sxt = act_quant_block(x2, transpose=True)
+    qdy, sdy = act_quant_block(dy2)
+    qdyt, sdyt = act_quant_block(dy2, transpose=True)
+    qwt, swt = weight_quant_block(w.detach().cpu().t().contiguous())
+    dx = fp8_matmul_official(qdy, qwt, sdy, swt, None, True)
+    dw = fp8_matmul_official(qdyt, qxt, sdyt, sxt, None, False)
+    return dx.reshape(x.shape), dw, dbias

@@ -1,0 +1,147 @@
+"""GPU parity of the official-dialect linear layer (deepseekv3/fp8_kernel.py: act_quant_block, fp8_matmul, Fp8Linear)
+against the CPU oracle: quantizer bytes and scales bit-exact, GEMMs within rtol = atol = 1e-2, exactly
+representable cases bit for bit."""
+import numpy as np
+import pytest
+import torch
+
+import mdy_triton_amd as m
+from mdy_triton_amd import fp8_kernel as FK
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+FP8 = torch.float8_e4m3fn
+DEV = "cuda:0"
+
+
+def u8(t):
+    return t.detach().cpu().contiguous().view(torch.uint8).numpy()
+
+
+def close(got, ref):
+    return torch.allclose(got.float().cpu(), ref.float(), rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("M,N", [(256, 128), (1024, 7168), (200, 256), (5, 128), (4096, 1536), (129, 384)])
+def test_act_quant_block_both_directions_bit_exact(M, N):
+    g = torch.Generator().manual_seed(M + N)
+    x = torch.randn(M, N, generator=g).bfloat16()
+    x[min(3, M - 1), 5] = 300.0                      # an outlier sets one row group's and one column group's scale
+    y_ref, s_ref = O.act_quant_block(x)
+    yt_ref, st_ref = O.act_quant_block(x, transpose=True)
+    y, s = m.act_quant_block(x.to(DEV))
+    yt, st = m.act_quant_block(x.to(DEV), transpose=True)
+    assert y.shape == (M, N) and s.shape == (M, N // 128) and yt.shape == (N, M) and st.shape == (N, (M + 127) // 128)
+    assert yt.is_contiguous() and st.is_contiguous()
+    assert np.array_equal(u8(y), u8(y_ref)) and torch.equal(s.cpu(), s_ref)
+    assert np.array_equal(u8(yt), u8(yt_ref)) and torch.equal(st.cpu(), st_ref)
+    # one pass for both copies (what the backward uses) and a strided input (a column slice of a wider tensor)
+    y2, s2, yt2, st2 = FK._act_quant_transposed(x.to(DEV), True, "test")
+    assert np.array_equal(u8(y2[:M]), u8(y_ref)) and torch.equal(s2[:M].cpu(), s_ref)
+    assert np.array_equal(u8(yt2[:, :M]), u8(yt_ref)) and torch.equal(st2.cpu(), st_ref)
+    wide = torch.randn(M, N + 64, generator=g).bfloat16().to(DEV)
+    yt3, st3 = m.act_quant_block(wide[:, 32:32 + N], transpose=True)
+    yt3_ref, st3_ref = O.act_quant_block(wide[:, 32:32 + N].cpu(), transpose=True)
+    assert np.array_equal(u8(yt3), u8(yt3_ref)) and torch.equal(st3.cpu(), st3_ref)
+
+
+def test_act_quant_block_leading_dims_and_asserts():
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(2, 3, 64, 256, generator=g).bfloat16()
+    y, s = m.act_quant_block(x.to(DEV))
+    yr, sr = O.act_quant_block(x)
+    assert y.shape == x.shape and s.shape == (2, 3, 64, 2) and np.array_equal(u8(y), u8(yr)) and torch.equal(s.cpu(), sr)
+    yt, st = m.act_quant_block(x.to(DEV), transpose=True)
+    ytr, str_ = O.act_quant_block(x, transpose=True)
+    assert yt.shape == (256, 384) and np.array_equal(u8(yt), u8(ytr)) and torch.equal(st.cpu(), str_)
+    with pytest.raises(AssertionError):
+        m.act_quant_block(torch.zeros(4, 100, device=DEV, dtype=torch.bfloat16))
+    with pytest.raises(TypeError):
+        m.act_quant_block(x.to(DEV), dtype=torch.float8_e5m2)
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (256, 384, 512), (130, 200, 384), (1000, 260, 1024), (64, 64, 2304)])
+def test_rowscaled_gemm_exact_integer(M, N, K):
+    """Integer operands and power-of-two scales on both sides: every product and sum is exact, so the bf16 result must
+    equal the float64 computation rounded once (catches swapped scale roles, K-block order, tile edges)."""
+    g = torch.Generator().manual_seed(M + N + K)
+    ai = torch.randint(-3, 4, (M, K), generator=g)
+    bi = torch.randint(-3, 4, (N, K), generator=g)
+    KB = K // 128
+    ea = torch.randint(-2, 3, (M, KB), generator=g)
+    eb = torch.randint(-2, 3, (N, KB), generator=g)
+    exact = torch.zeros(M, N, dtype=torch.float64)
+    for kb in range(KB):
+        exact += (ai[:, kb * 128:(kb + 1) * 128].double() @ bi[:, kb * 128:(kb + 1) * 128].double().t()) * \
+            torch.exp2((ea[:, kb][:, None] + eb[:, kb][None, :]).double())
+    got = FK.fp8_matmul(ai.float().to(FP8).to(DEV), bi.float().to(FP8).to(DEV), torch.exp2(ea.float()).to(DEV),
+                        torch.exp2(eb.float()).to(DEV), have_w=False) if M % 128 == 0 else \
+        FK._matmul_rowscaled(ai.float().to(FP8).to(DEV), torch.exp2(ea.float()).to(DEV), bi.float().to(FP8).to(DEV),
+                             torch.exp2(eb.float()).to(DEV), M, N, K, torch.device(DEV))
+    assert got.dtype == torch.bfloat16 and torch.equal(got.cpu().double(), exact.to(torch.bfloat16).double())
+
+
+def test_rowscaled_gemm_random_and_ragged_k():
+    g = torch.Generator().manual_seed(9)
+    M, N, K = 256, 300, 1000                            # K not a multiple of 128: completed with zeros
+    x = torch.randn(K, M, generator=g).bfloat16()      # tokens x features: the operands are quantized transposes
+    w = torch.randn(K, N, generator=g).bfloat16()
+    a, sa = O.act_quant_block(x, transpose=True)        # [M, K], [M, 8]
+    b, sb = O.act_quant_block(w, transpose=True)
+    ref = O.fp8_matmul_official(a, b, sa, sb, None, False)
+    got = FK.fp8_matmul(a.to(DEV), b.to(DEV), sa.to(DEV), sb.to(DEV), have_w=False)
+    assert got.shape == (M, N) and close(got, ref)
+    with pytest.raises(AssertionError):
+        FK.fp8_matmul(a[:100].to(DEV), b.to(DEV), sa[:100].to(DEV), sb.to(DEV), have_w=False)
+    # the C entry point rejects what it cannot address
+    from mdy_triton_amd import _lib
+    L = _lib.load()
+    one = torch.zeros(64, dtype=torch.uint8, device=DEV)
+    p = one.data_ptr()
+    assert L.mdy_fp8_gemm_nt_rowscaled(p, p, 1, 1, p, p, 1, 1, p, 4, 4, 100, 0, None) == -2
+    assert L.mdy_fp8_gemm_nt_rowscaled(p + 1, p, 1, 1, p, p, 1, 1, p, 4, 4, 128, 0, None) == -3
+    assert L.mdy_fp8_gemm_nt_rowscaled(None, p, 1, 1, p, p, 1, 1, p, 4, 4, 128, 0, None) == -1
+    assert L.mdy_fp8_gemm_nt_rowscaled(p, p, -1, 1, p, p, 1, 1, p, 4, 4, 128, 0, None) == -2
+    assert L.mdy_act_quant_transpose(p, None, p, p, p, 4, 128, 128, 1, 128, 128, None) == -1
+
+
+@pytest.mark.parametrize("bias", [True, False])
+@pytest.mark.parametrize("shape,N", [((2, 128, 256), 256), ((512, 1024), 768), ((3, 50, 384), 128), ((1024, 7168), 1536)])
+def test_fp8_linear_forward_backward(shape, N, bias):
+    g = torch.Generator().manual_seed(sum(shape) + N)
+    K = shape[-1]
+    w = (torch.randn(N, K, generator=g) * 0.02).bfloat16()
+    b = torch.randn(N, generator=g).bfloat16() if bias else None
+    x = torch.randn(*shape, generator=g).bfloat16()
+    dy = torch.randn(*shape[:-1], N, generator=g).bfloat16()
+    ref_out = O.fp8_linear_forward(x, w, b)
+    ref_dx, ref_dw, ref_db = O.fp8_linear_backward(x, w, dy, bias)
+    lin = m.Fp8Linear(K, N, bias=bias, dtype=torch.bfloat16, fp8_dtype=torch.float8_e4m3fn)
+    with torch.no_grad():
+        lin.weight.copy_(w)
+        if bias:
+            lin.bias.copy_(b)
+    lin = lin.to(DEV)
+    xg = x.to(DEV).requires_grad_(True)
+    out = lin(xg)
+    out.backward(dy.to(DEV))
+    assert out.shape == (*shape[:-1], N) and out.dtype == torch.bfloat16
+    if bias:      # the relative part of the tolerance belongs to the GEMM result before the bias
+        mag = torch.maximum(ref_out.float().abs(), (ref_out.float() - b.float()).abs())
+        assert bool(((out.float().cpu() - ref_out.float()).abs() <= 1e-2 + 1e-2 * mag).all())
+    else:
+        assert close(out, ref_out)
+    assert xg.grad.shape == x.shape and close(xg.grad, ref_dx)
+    assert lin.weight.grad.shape == (N, K) and close(lin.weight.grad, ref_dw)
+    if bias:
+        assert torch.allclose(lin.bias.grad.float().cpu(), ref_db.float(), rtol=1e-2, atol=1e-2)
+    # only one of the two gradients wanted
+    lin.zero_grad()
+    lin(x.to(DEV)).backward(dy.to(DEV))
+    assert close(lin.weight.grad, ref_dw)
+    lin.weight.requires_grad_(False)
+    xg2 = x.to(DEV).requires_grad_(True)
+    lin(xg2).backward(dy.to(DEV))
+    assert close(xg2.grad, ref_dx)
+    with pytest.raises(TypeError, match="float8_e4m3fn"):
+        m.Fp8Linear(K, N, dtype=torch.bfloat16, fp8_dtype=torch.float8_e5m2)

@@ -404,3 +404,77 @@ def test_fp8_padding_row_by_row():
     back = O.fp8_unpadding(padded, m_splits)
     assert torch.equal(back, x)
     assert O.fp8_padding(x[:0], [0, 0])[0].shape == (0, H)
+
+
+def test_act_quant_block_transposed_reduces_to_act_quant_and_groups():
+    """act_quant_block(x, transpose=True) == act_quant of the transposed, zero-padded matrix (the pinned
+    quantizer), plus a plain loop over the groups of two columns: scale = max|.| / 448 in numpy float32 and
+    bytes through the from-definition codec."""
+    g = torch.Generator().manual_seed(41)
+    for (M, N) in ((256, 128), (200, 256), (5, 128)):
+        x = torch.randn(M, N, generator=g).bfloat16()
+        y, s = O.act_quant_block(x, transpose=True)
+        assert y.shape == (N, M) and s.shape == (N, (M + 127) // 128)
+        PM = (M + 127) // 128 * 128
+        xt = torch.zeros(N, PM).bfloat16()
+        xt[:, :M] = x.t()
+        y2, s2 = O.act_quant(xt)
+        assert np.array_equal(u8(y), u8(y2[:, :M].contiguous())) and torch.equal(s, s2)
+        xf = x.float().numpy()
+        for col in (0, N - 1):
+            for gi in range((M + 127) // 128):
+                grp = xf[gi * 128:(gi + 1) * 128, col]
+                sc = np.float32(np.abs(grp).max()) / np.float32(448.0)
+                assert s[col, gi].item() == sc
+                want = F.encode_rne((grp / sc).astype(np.float32))
+                assert np.array_equal(u8(y)[col, gi * 128:gi * 128 + len(grp)], want)
+    yy, ss = O.act_quant_block(x.reshape(1, 5, 128))
+    ya, sa = O.act_quant(x.reshape(1, 5, 128))
+    assert np.array_equal(u8(yy), u8(ya)) and torch.equal(ss, sa)
+
+
+def test_rowscaled_matmul_float64_exact_and_reduction():
+    g = torch.Generator().manual_seed(42)
+    M, N, K = 40, 256, 384
+    a = torch.randint(0, 0x78, (M, K), generator=g, dtype=torch.uint8).view(O.FP8)
+    b = torch.randint(0, 0x78, (N, K), generator=g, dtype=torch.uint8).view(O.FP8)
+    sa = torch.rand(M, 3, generator=g) + 0.5
+    sb = torch.rand(N, 3, generator=g) + 0.5
+    got = O.fp8_matmul_official(a, b, sa, sb, None, False)
+    truth = torch.zeros(M, N, dtype=torch.float64)
+    for kb in range(3):
+        part = a[:, kb * 128:(kb + 1) * 128].double() @ b[:, kb * 128:(kb + 1) * 128].double().t()
+        truth += part * sa[:, kb].double()[:, None] * sb[:, kb].double()[None, :]
+    assert (got.double() - truth).abs().max() <= 2 ** -8 * truth.abs().max()
+    # weight-row scales constant within each 128-row block: the block-scaled GEMM (pinned) gives the same result
+    sb_blk = torch.rand(2, 3, generator=g) + 0.5
+    sb_rows = sb_blk.repeat_interleave(128, 0)
+    assert torch.equal(O.fp8_matmul_official(a, b, sa, sb_rows, None, False), O.fp8_gemm(a, sa, b, sb_blk))
+    # exactly representable: small integers, power-of-two scales (transposed scale roles would show)
+    ai = torch.randint(-3, 4, (M, K), generator=g)
+    bi = torch.randint(-3, 4, (N, K), generator=g)
+    ea = torch.randint(-2, 3, (M, 3), generator=g)
+    eb = torch.randint(-2, 3, (N, 3), generator=g)
+    exact = torch.zeros(M, N, dtype=torch.float64)
+    for kb in range(3):
+        exact += (ai[:, kb * 128:(kb + 1) * 128].double() @ bi[:, kb * 128:(kb + 1) * 128].double().t()) * \
+            torch.exp2((ea[:, kb][:, None] + eb[:, kb][None, :]).double())
+    out = O.fp8_matmul_official(ai.float().to(O.FP8), bi.float().to(O.FP8), torch.exp2(ea.float()), torch.exp2(eb.float()), None, False)
+    assert torch.equal(out.double(), exact.to(torch.bfloat16).double())
+
+
+def test_fp8_linear_oracle_close_to_unquantized():
+    g = torch.Generator().manual_seed(43)
+    x = torch.randn(4, 64, 256, generator=g).bfloat16()
+    w = (torch.randn(128, 256, generator=g) * 0.05).bfloat16()
+    b = torch.randn(128, generator=g).bfloat16()
+    dy = torch.randn(4, 64, 128, generator=g).bfloat16()
+    y = O.fp8_linear_forward(x, w, b)
+    ref = torch.nn.functional.linear(x.float(), w.float(), b.float())
+    assert y.shape == ref.shape and (y.float() - ref).abs().mean() < 0.03
+    dx, dw, db = O.fp8_linear_backward(x, w, dy)
+    dxr = dy.float() @ w.float()
+    dwr = dy.float().reshape(-1, 128).t() @ x.float().reshape(-1, 256)
+    assert dx.shape == x.shape and (dx.float() - dxr).abs().mean() < 0.06 * dxr.abs().mean()
+    assert dw.shape == w.shape and (dw.float() - dwr).abs().mean() < 0.06 * dwr.abs().mean()
+    assert torch.allclose(db.float(), dy.float().reshape(-1, 128).sum(0), rtol=1e-2, atol=1e-1)
