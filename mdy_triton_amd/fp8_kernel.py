@@ -241,6 +241,30 @@ def fp8_matmul_bwd(xt, w, dy, dyt, scale_xt, scale_w, scale_dy, scale_dyt):
     return dx, dw
 
 
+def _official_linear_backward(x2, w, dy2, need_dx, need_dw, fp8_dtype=FP8):
+    """Gradients of y = x2 . w^T in the official dialect (fp8_kernel.py:274-301): dx = dy . w on the row-wise copy of dy
+    and the block-quantized w^T, dw = dy^T . x on the transposed copies of dy and x (row scales on both operands).
+    One kernel pass over dy gives both of its copies; the transposed copies keep their zero padding to a multiple of
+    128 tokens."""
+    M, K = x2.shape
+    N = w.size(0)
+    dev = x2.device
+    dx = dw = None
+    qdy, sdy, qdyt, sdyt = _act_quant_transposed(dy2, need_dx, "Fp8Linear.backward")
+    if need_dx:
+        qwt, swt = weight_quant_block(w.t(), dtype=fp8_dtype)       # [K, N]: the 128x128 blocks of w, transposed
+        dx = fp8_matmul(qdy[:M], qwt, sdy[:M], swt, have_w=True)
+    if need_dw:
+        _, _, qxt, sxt = _act_quant_transposed(x2, False, "Fp8Linear.backward")
+        dw = torch.empty(N, K, device=dev, dtype=torch.bfloat16)
+        if N * K > 0:
+            with on_device(dev):
+                check(lib().mdy_fp8_gemm_nt_rowscaled(ptr(qdyt), ptr(sdyt), sdyt.stride(0), sdyt.stride(1), ptr(qxt), ptr(sxt),
+                                                      sxt.stride(0), sxt.stride(1), ptr(dw), N, K, qdyt.size(1), 0,
+                                                      stream_ptr(dev)), "Fp8Linear.backward")
+    return dx, dw
+
+
 class _Fp8LinearFunction(torch.autograd.Function):
     """fp8_kernel.py:259-301.  Forward: act_quant_block(x), weight_quant_block(w), GEMM with the bias in its epilogue.
     Backward: x and dy quantized along the tokens (transposed copies, one kernel pass over dy for both of its copies),
@@ -268,24 +292,8 @@ class _Fp8LinearFunction(torch.autograd.Function):
             dy2 = dy2.to(torch.bfloat16)
         dbias = dy2.sum(0) if ctx.bias is not None and ctx.needs_input_grad[2] else None
         x2, w = ctx.saved_tensors
-        M, K = x2.shape
-        N = w.size(0)
-        dev = x2.device
-        dx = dw = None
-        need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
-        qdy, sdy, qdyt, sdyt = _act_quant_transposed(dy2, need_dx, "Fp8Linear.backward")
-        if need_dx:
-            qwt, swt = weight_quant_block(w.t(), dtype=ctx.fp8_dtype)       # [K, N], blocks of w^T
-            dx = fp8_matmul(qdy[:M], qwt, sdy[:M], swt, have_w=True).view(ctx.input_shape)
-        if need_dw:
-            _, _, qxt, sxt = _act_quant_transposed(x2, False, "Fp8Linear.backward")
-            PM = qdyt.size(1)
-            dw = torch.empty(N, K, device=dev, dtype=torch.bfloat16)
-            with on_device(dev):
-                check(lib().mdy_fp8_gemm_nt_rowscaled(ptr(qdyt), ptr(sdyt), sdyt.stride(0), sdyt.stride(1), ptr(qxt), ptr(sxt),
-                                                      sxt.stride(0), sxt.stride(1), ptr(dw), N, K, PM, 0, stream_ptr(dev)),
-                      "Fp8Linear.backward")
-        return dx, dw, dbias, None
+        dx, dw = _official_linear_backward(x2, w, dy2, ctx.needs_input_grad[0], ctx.needs_input_grad[1], ctx.fp8_dtype)
+        return (dx.view(ctx.input_shape) if dx is not None else None), dw, dbias, None
 
 
 fp8_linear_with_quant_ops = _Fp8LinearFunction.apply
@@ -354,32 +362,83 @@ class _Fp8MlpCkptOps(torch.autograd.Function):
         return dx, dw_up_gate, dw_down, None, None, None, None
 
 
-def fp8_ckpt_mlp(x, w_up_gate, w_down, fp8_dtype=FP8, order="up-gate"):
+class _Fp8MlpCkptOfficial(torch.autograd.Function):
+    """The same memory-saving step in the official dialect, as the reference runs it (fp8_kernel.py:436-494):
+    act_quant_block / weight_quant_block / fp8_matmul, the activation quantized by the fused SwiGLU kernel in the
+    forward (same bytes as silu_fwd + act_quant_block), x the only activation kept."""
+
+    @staticmethod
+    def forward(ctx, x, w_up_gate, w_down, fp8_dtype=FP8, order="up-gate"):
+        _require_e4m3(fp8_dtype, "fp8_ckpt_mlp")
+        shape = x.shape
+        x2 = x.reshape(-1, shape[-1])
+        qx, sx = act_quant_block(x2, dtype=fp8_dtype)
+        qwu, swu = weight_quant_block(w_up_gate, dtype=fp8_dtype)
+        qwd, swd = weight_quant_block(w_down, dtype=fp8_dtype)
+        up_gate = fp8_matmul(qx, qwu, sx, swu)
+        qact, sact = silu_act_quant(up_gate, order, dialect="official")
+        y = fp8_matmul(qact, qwd, sact, swd)
+        ctx.save_for_backward(x2, w_up_gate, w_down)
+        ctx.order, ctx.shape, ctx.fp8_dtype = order, shape, fp8_dtype
+        return y.view(*shape[:-1], w_down.size(0))
+
+    @staticmethod
+    def backward(ctx, dy):
+        x2, w_up_gate, w_down = ctx.saved_tensors
+        dy2 = dy.reshape(-1, dy.size(-1))
+        if dy2.dtype != torch.bfloat16:
+            dy2 = dy2.to(torch.bfloat16)
+        qx, sx = act_quant_block(x2, dtype=ctx.fp8_dtype)
+        qwu, swu = weight_quant_block(w_up_gate, dtype=ctx.fp8_dtype)
+        up_gate = fp8_matmul(qx, qwu, sx, swu)
+        act = silu_fwd(up_gate, ctx.order)
+        dact, dw_down = _official_linear_backward(act, w_down, dy2, True, True, ctx.fp8_dtype)
+        dup_gate = silu_bwd(dact, up_gate, ctx.order)
+        dx, dw_up_gate = _official_linear_backward(x2, w_up_gate, dup_gate, True, True, ctx.fp8_dtype)
+        return dx.view(ctx.shape), dw_up_gate, dw_down, None, None
+
+
+def fp8_ckpt_mlp(x, w_up_gate, w_down, fp8_dtype=FP8, order="up-gate", dialect="official"):
     """Memory-saving FP8 MLP step with the reference's positional order (fp8_kernel.py:436-494:
     `fp8_ckpt_mlp(h, w1, w2, self.fp8_dtype, self.order)`).  Only float8_e4m3fn is implemented: the reference's
-    default, float8_e5m2, raises TypeError here."""
+    default, float8_e5m2, raises TypeError here.  dialect "official" (the reference's: s = amax / 448) or
+    "deeplinear" (clamp 1e4 + eps 1e-8, the quantizers of dpsk_fp8linear/fp8.py)."""
+    if dialect == "official":
+        return _Fp8MlpCkptOfficial.apply(x, w_up_gate, w_down, fp8_dtype, order)
+    if dialect != "deeplinear":
+        raise ValueError("dialect must be 'official' or 'deeplinear'")
     return _Fp8MlpCkptOps.apply(x, w_up_gate, w_down, fp8_dtype, order)
 
 
 class Fp8MLP(torch.nn.Module):
     """SwiGLU MLP on the FP8 linear path (fp8_kernel.py:500-515): up/gate projection, silu(gate) * up, down
-    projection, both projections block-wise FP8 (`DeepLinear`: e4m3fn, 1x128 activation and 128x128 weight
-    scales), no biases.
+    projection, both projections block-wise FP8 (e4m3fn, 1x128 activation and 128x128 weight scales), no biases.
 
+    dialect "official" (default, what the reference's Fp8MLP computes: its projections are `Fp8Linear`s,
+    s = amax / 448) or "deeplinear" (`DeepLinear` projections: clamp 1e4 + eps 1e-8, optional weight cache).
     Without gradients the activation goes from the up/gate GEMM to the down GEMM through the fused
     SwiGLU + quantizer (one pass, the bf16 activation is never written).  With gradients the default is the
-    composition DeepLinear -> triton_silu -> DeepLinear; `low_memory` (attribute or call argument, as in the
+    composition linear -> triton_silu -> linear; `low_memory` (attribute or call argument, as in the
     reference) keeps only the input for the backward pass and recomputes up/gate and the activation there.
     """
 
     def __init__(self, hidden_size, intermediate_size, order="up-gate", fp8_dtype=FP8, low_memory=False,
-                 device=None, dtype=torch.bfloat16):
+                 device=None, dtype=torch.bfloat16, dialect="official"):
         super().__init__()
         _require_e4m3(fp8_dtype, "Fp8MLP")
         assert order in _ORDERS, "please indicate the order of input, up-gate or gate-up"
-        from .fp8 import DeepLinear
-        self.up_gate_proj = DeepLinear(hidden_size, intermediate_size * 2, bias=False, device=device, dtype=dtype)
-        self.down_proj = DeepLinear(intermediate_size, hidden_size, bias=False, device=device, dtype=dtype)
+        if dialect not in ("official", "deeplinear"):
+            raise ValueError("dialect must be 'official' or 'deeplinear'")
+        if dialect == "official":
+            self.up_gate_proj = Fp8Linear(hidden_size, intermediate_size * 2, bias=False, device=device, dtype=dtype,
+                                          fp8_dtype=fp8_dtype)
+            self.down_proj = Fp8Linear(intermediate_size, hidden_size, bias=False, device=device, dtype=dtype,
+                                       fp8_dtype=fp8_dtype)
+        else:
+            from .fp8 import DeepLinear
+            self.up_gate_proj = DeepLinear(hidden_size, intermediate_size * 2, bias=False, device=device, dtype=dtype)
+            self.down_proj = DeepLinear(intermediate_size, hidden_size, bias=False, device=device, dtype=dtype)
+        self.dialect = dialect
         self.order = order
         self.fp8_dtype = fp8_dtype
         self.low_memory = low_memory
@@ -389,7 +448,9 @@ class Fp8MLP(torch.nn.Module):
         needs_grad = torch.is_grad_enabled() and (hidden_states.requires_grad or up.weight.requires_grad or
                                                   down.weight.requires_grad)
         if not needs_grad or low_memory or self.low_memory:
-            # cached quantized weights (re-quantized when a weight changes); the forward needs no transposed copies
+            if self.dialect == "official":
+                return _Fp8MlpCkptOfficial.apply(hidden_states, up.weight, down.weight, self.fp8_dtype, self.order)
+            # cached quantized weights (when the projections cache); the forward needs no transposed copies
             return _Fp8MlpCkptOps.apply(hidden_states, up.weight, down.weight, self.fp8_dtype, self.order,
                                         up._quantized_weight(False) if up.cache_weight else None,
                                         down._quantized_weight(False) if down.cache_weight else None)

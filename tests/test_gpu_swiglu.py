@@ -136,7 +136,7 @@ def test_fp8_mlp_three_paths(shape, inter, order):
     w_d = (torch.randn(H, inter, generator=g) * 0.03).bfloat16()
     dy = torch.randn(*shape, generator=g).bfloat16()
 
-    mlp = m.Fp8MLP(H, inter, order=order, device=DEV)
+    mlp = m.Fp8MLP(H, inter, order=order, device=DEV, dialect="deeplinear")
     up, down = mlp.up_gate_proj, mlp.down_proj
     with torch.no_grad():
         up.weight.copy_(w_ug)
@@ -193,15 +193,64 @@ def test_fp8_ckpt_mlp_reference_call_order():
     x = torch.randn(32, H, generator=g).bfloat16().to(DEV)
     w_ug = (torch.randn(2 * inter, H, generator=g) * 0.03).bfloat16().to(DEV)
     w_d = (torch.randn(H, inter, generator=g) * 0.03).bfloat16().to(DEV)
-    mlp = m.Fp8MLP(H, inter, order="gate-up", device=DEV)
+    mlp = m.Fp8MLP(H, inter, order="gate-up", device=DEV, dialect="deeplinear")
     with torch.no_grad():
         mlp.up_gate_proj.weight.copy_(w_ug)
         mlp.down_proj.weight.copy_(w_d)
         want = mlp(x)
-        got = m.fp8_ckpt_mlp(x, w_ug, w_d, torch.float8_e4m3fn, "gate-up")
+        got = m.fp8_ckpt_mlp(x, w_ug, w_d, torch.float8_e4m3fn, "gate-up", dialect="deeplinear")
         assert torch.equal(got, want)
-        assert torch.equal(m.fp8_ckpt_mlp(x, w_ug, w_d, order="gate-up"), want)
+        assert torch.equal(m.fp8_ckpt_mlp(x, w_ug, w_d, order="gate-up", dialect="deeplinear"), want)
         with pytest.raises(TypeError, match="float8_e4m3fn"):
             m.fp8_ckpt_mlp(x, w_ug, w_d, torch.float8_e5m2, "gate-up")
         with pytest.raises(TypeError, match="float8_e4m3fn"):
             m.Fp8MLP(H, inter, fp8_dtype=torch.float8_e5m2, device=DEV)
+
+
+@pytest.mark.parametrize("order", ["up-gate", "gate-up"])
+def test_fp8_mlp_official_dialect_three_paths(order):
+    """The reference's own Fp8MLP (projections = Fp8Linear, s = amax / 448): composition with gradients, the
+    memory-saving op (called positionally as the reference does) and the gradient-free fused path agree bit for bit;
+    every stage is within the GEMM tolerance of the oracle fed the device's own bf16 intermediates."""
+    H, inter, shape = 512, 768, (3, 100, 512)
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(*shape, generator=g).bfloat16()
+    w_ug = (torch.randn(2 * inter, H, generator=g) * 0.03).bfloat16()
+    w_d = (torch.randn(H, inter, generator=g) * 0.03).bfloat16()
+    dy = torch.randn(*shape, generator=g).bfloat16()
+    mlp = m.Fp8MLP(H, inter, order=order, device=DEV)
+    assert mlp.dialect == "official" and isinstance(mlp.up_gate_proj, m.Fp8Linear)
+    up, down = mlp.up_gate_proj, mlp.down_proj
+    with torch.no_grad():
+        up.weight.copy_(w_ug)
+        down.weight.copy_(w_d)
+    results = []
+    for low_memory in (False, True):
+        mlp.zero_grad()
+        xg = x.to(DEV).requires_grad_(True)
+        y = mlp(xg, low_memory=low_memory)
+        y.backward(dy.to(DEV))
+        results.append((y.detach(), xg.grad, up.weight.grad.clone(), down.weight.grad.clone()))
+    for a, b in zip(*results):
+        assert a.shape == b.shape and a.dtype == torch.bfloat16 and torch.equal(a, b)
+    with torch.no_grad():
+        assert torch.equal(mlp(x.to(DEV)), results[0][0])
+        assert torch.equal(m.fp8_ckpt_mlp(x.to(DEV), up.weight, down.weight, torch.float8_e4m3fn, order), results[0][0])
+    y_d, dx_d, dwug_d, dwd_d = results[0]
+    # stage by stage against the oracle
+    mlp.zero_grad()
+    xg = x.to(DEV).requires_grad_(True)
+    ug_d = up(xg)
+    ug_d.retain_grad()
+    act_d = m.triton_silu(ug_d, order)
+    act_d.retain_grad()
+    y2 = down(act_d)
+    y2.backward(dy.to(DEV))
+    assert torch.equal(y2, y_d)
+    ug_c, act_c = ug_d.detach().cpu(), act_d.detach().cpu()
+    assert _within(ug_d, O.fp8_linear_forward(x, w_ug, None))
+    assert _within(y_d, O.fp8_linear_forward(act_c, w_d, None))
+    dact_r, dwd_r, _ = O.fp8_linear_backward(act_c, w_d, dy, False)
+    assert _within(act_d.grad, dact_r) and _within(dwd_d, dwd_r)
+    dx_r, dwug_r, _ = O.fp8_linear_backward(x, w_ug, ug_d.grad.cpu(), False)
+    assert _within(dx_d, dx_r) and _within(dwug_d, dwug_r)
