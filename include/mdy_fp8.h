@@ -55,7 +55,8 @@ const char* mdy_fp8_last_error(void);
  * (fp8.py:122-161, kernel :87-120) with mode = MDY_QUANT_DEEPLINEAR and the
  * padded sizes that launcher computes.
  *
- *   x  bf16 [M, K], element (m, k) at x[m * x_row_stride + k]   (unit column stride)
+ *   x  bf16 [M, K], element (m, k) at x[m * x_row_stride + k]   (unit column stride; x_row_stride >= K, or 0 for
+ *      a row broadcast M times)
  *   y  e4m3fn [PM, PK] row-major; PM >= M, PK >= K, PK % 128 == 0; padding reads as 0
  *   s  fp32, scale of row m, K-block kb at s[m * s_row_stride + kb * s_col_stride]
  *      for m < PM, kb < PK / 128

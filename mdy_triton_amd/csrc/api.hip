@@ -63,7 +63,9 @@ int mdy_act_quant(const void* x, void* y, float* s, int64_t M, int64_t K, int64_
     if (PK % 128 != 0) return fail(MDY_E_SHAPE, "act_quant: PK=%lld is not a multiple of 128", (long long)PK);
     if (PM == 0 || PK == 0) return 0;
     if (!y || !s || (!x && M > 0 && K > 0)) return fail(MDY_E_NULL, "act_quant: null pointer");
-    if (M > 0 && x_row_stride < K) return fail(MDY_E_SHAPE, "act_quant: x_row_stride=%lld < K=%lld", (long long)x_row_stride, (long long)K);
+    // rows may overlap only as a broadcast (stride 0, an expanded tensor); a single row has no stride to speak of
+    if (M > 1 && x_row_stride != 0 && x_row_stride < K)
+        return fail(MDY_E_SHAPE, "act_quant: x_row_stride=%lld < K=%lld (and not 0)", (long long)x_row_stride, (long long)K);
     if (!aligned(y, 8)) return fail(MDY_E_ALIGN, "act_quant: y must be 8-byte aligned");
     if (!aligned(x, 2) || !aligned(s, 4)) return fail(MDY_E_ALIGN, "act_quant: x/s misaligned for their element type");
     if (int e = check_device()) return e;

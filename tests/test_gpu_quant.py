@@ -373,3 +373,22 @@ def test_quantizers_random_shapes():
         for only_forward in (True, False):
             _same_quant([t for t in m.quant_weight(xd, only_forward) if t is not None],
                         [t for t in O.quant_weight(x, only_forward) if t is not None])
+
+
+def test_quant_input_broadcast_rows():
+    """A row expanded to M rows (row stride 0) is quantized like its materialised copy, as the training quantizer
+    already does; the C entry point still rejects overlapping rows of any other stride."""
+    g = torch.Generator().manual_seed(12)
+    row = torch.randn(1, 512, generator=g).bfloat16()
+    x = row.to(DEV).expand(12, 512)
+    assert x.stride(0) == 0
+    y, s, _, _ = m.quant_input(x, True)
+    yr, sr, _, _ = O.quant_input(row.expand(12, 512).contiguous(), True)
+    assert torch.equal(y.cpu().view(torch.uint8), yr.view(torch.uint8)) and torch.equal(s.cpu().contiguous(), sr.contiguous())
+    from mdy_triton_amd import _lib
+    L = _lib.load()
+    buf = torch.zeros(4096, dtype=torch.uint8, device=DEV)
+    p = buf.data_ptr()
+    assert L.mdy_act_quant(p, p + 1024, p + 2048, 4, 128, 64, 4, 128, 1, 1, 0, None) == -2
+    assert L.mdy_act_quant(p, p + 1024, p + 2048, 1, 128, 64, 1, 128, 1, 1, 0, None) == 0
+    torch.cuda.synchronize()
