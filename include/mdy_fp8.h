@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define MDY_FP8_ABI_VERSION 7
+#define MDY_FP8_ABI_VERSION 8
 
 /* error codes (negative = argument rejected before any launch) */
 #define MDY_OK 0
@@ -297,6 +297,11 @@ int mdy_group_pad_rows(const void* x, void* y, const int64_t* m_splits, int64_t 
 /* In-place x[m, :] = bf16(fp32(x[m, :]) + fp32(b)) on bf16 x [M, N] row-major, bf16 b [N].
  * Replaces add_bias (fp8.py:297-305, kernel :283-295). */
 int mdy_add_bias(void* x, const void* b, int64_t M, int64_t N, void* stream);
+
+/* In-place gradient accumulation over n elements: x[i] = T(fp32(x[i]) + fp32(y[i])), x of x_dtype, y of y_dtype
+ * (MDY_DT_BF16 / MDY_DT_F32 each).  Replaces add_grad (triton_kernels/megatron_patchs/add_kernel.py:55-62, kernel
+ * :41-52), the Megatron patch's accumulation of a weight gradient into main_grad. */
+int mdy_add_grad(void* x, const void* y, int64_t n, int x_dtype, int y_dtype, void* stream);
 
 /* Diagnostic: element-wise fp32 -> e4m3fn with the same device conversion the
  * quantizers use (saturate != 0 clamps finite values to +-448 first).  No

@@ -10,7 +10,7 @@ import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libmdyfp8.so")
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _lock = threading.Lock()
 _lib = None
@@ -39,6 +39,7 @@ SIGNATURES = {
     "mdy_fp8_gemm_static_workspace_bytes": [],
     "mdy_fp8_gemm_static_workspace_init": [],
     "mdy_group_pad_rows": [_p, _p, _p, _i64, _i64, _i64, _int, _p],
+    "mdy_add_grad": [_p, _p, _i64, _int, _int, _p],
     "mdy_add_bias": [_p, _p, _i64, _i64, _p],
     "mdy_cast_f32_to_e4m3": [_p, _p, _i64, _int, _p],
     "mdy_quotient_selfcheck": [_p, _int, _int, _int, _p],

@@ -54,4 +54,43 @@ int launch_add_bias(void* x, const void* b, int64_t M, int64_t N, hipStream_t st
     return (int)hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// In-place gradient accumulation x = T(fp32(x) + fp32(y)) over flat tensors of n elements, x fp32 or bf16, y fp32 or
+// bf16.  Restates _add_grad_kernel (/root/reference/triton_kernels/megatron_patchs/add_kernel.py:41-62), which the
+// Megatron patch uses to add a bf16 weight gradient into the fp32 main_grad buffer.  Streaming, 8 elements per lane.
+// ---------------------------------------------------------------------------
+template <typename T>
+__device__ __forceinline__ float grad_load(const T* p, int64_t i);
+template <>
+__device__ __forceinline__ float grad_load<float>(const float* p, int64_t i) { return p[i]; }
+template <>
+__device__ __forceinline__ float grad_load<uint16_t>(const uint16_t* p, int64_t i) { return bf16_one(p[i]); }
+__device__ __forceinline__ void grad_store(float* p, int64_t i, float v) { p[i] = v; }
+__device__ __forceinline__ void grad_store(uint16_t* p, int64_t i, float v) { p[i] = (uint16_t)(pack2_bf16(v, 0.0f) & 0xFFFFu); }
+
+template <typename TX, typename TY>
+__global__ __launch_bounds__(256) void add_grad_kernel(TX* __restrict__ x, const TY* __restrict__ y, int64_t n) {
+    const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+        if (i0 + j < n) grad_store(x, i0 + j, grad_load<TX>(x, i0 + j) + grad_load<TY>(y, i0 + j));
+}
+
+// dtype codes: 0 bf16, 1 fp32
+int launch_add_grad(void* x, const void* y, int64_t n, int x_dtype, int y_dtype, hipStream_t stream) {
+    if (n == 0) return 0;
+    const int64_t blocks = (n + 2047) / 2048;
+    if (blocks > 0x7FFFFFFF) return kErrTooManyBlocks;
+    dim3 grid((unsigned)blocks), block(256);
+    if (x_dtype == 1 && y_dtype == 0)
+        hipLaunchKernelGGL((add_grad_kernel<float, uint16_t>), grid, block, 0, stream, static_cast<float*>(x), static_cast<const uint16_t*>(y), n);
+    else if (x_dtype == 1)
+        hipLaunchKernelGGL((add_grad_kernel<float, float>), grid, block, 0, stream, static_cast<float*>(x), static_cast<const float*>(y), n);
+    else if (y_dtype == 0)
+        hipLaunchKernelGGL((add_grad_kernel<uint16_t, uint16_t>), grid, block, 0, stream, static_cast<uint16_t*>(x), static_cast<const uint16_t*>(y), n);
+    else
+        hipLaunchKernelGGL((add_grad_kernel<uint16_t, float>), grid, block, 0, stream, static_cast<uint16_t*>(x), static_cast<const float*>(y), n);
+    return (int)hipGetLastError();
+}
+
 }  // namespace mdy

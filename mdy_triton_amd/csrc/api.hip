@@ -333,6 +333,18 @@ int mdy_add_bias(void* x, const void* b, int64_t M, int64_t N, void* stream) {
     return launched(mdy::launch_add_bias(x, b, M, N, static_cast<hipStream_t>(stream)), "add_bias");
 }
 
+int mdy_add_grad(void* x, const void* y, int64_t n, int x_dtype, int y_dtype, void* stream) {
+    if ((x_dtype != MDY_DT_BF16 && x_dtype != MDY_DT_F32) || (y_dtype != MDY_DT_BF16 && y_dtype != MDY_DT_F32))
+        return fail(MDY_E_DTYPE, "add_grad: dtypes must be MDY_DT_BF16 or MDY_DT_F32");
+    if (n < 0) return fail(MDY_E_SHAPE, "add_grad: n < 0");
+    if (n == 0) return 0;
+    if (!x || !y) return fail(MDY_E_NULL, "add_grad: null pointer");
+    if (!aligned(x, x_dtype == MDY_DT_BF16 ? 2 : 4) || !aligned(y, y_dtype == MDY_DT_BF16 ? 2 : 4))
+        return fail(MDY_E_ALIGN, "add_grad: misaligned pointer");
+    if (int e = check_device()) return e;
+    return launched(mdy::launch_add_grad(x, y, n, x_dtype, y_dtype, static_cast<hipStream_t>(stream)), "add_grad");
+}
+
 int mdy_cast_f32_to_e4m3(const float* x, void* y, int64_t n, int saturate, void* stream) {
     if (n < 0) return fail(MDY_E_SHAPE, "cast_f32_to_e4m3: n < 0");
     if (n == 0) return 0;

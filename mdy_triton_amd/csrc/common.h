@@ -224,6 +224,7 @@ int launch_fp8_grouped_gemm_nt(const void* a, const float* a_s, int64_t as_row_s
                                int64_t G, int64_t M, int64_t N, int64_t K, int out_dtype, hipStream_t stream);
 int launch_group_pad(const void* x, void* y, const int64_t* m_splits, int64_t G, int64_t row_bytes, int64_t multiple,
                      int unpad, hipStream_t stream);
+int launch_add_grad(void* x, const void* y, int64_t n, int x_dtype, int y_dtype, hipStream_t stream);
 int launch_add_bias(void* x, const void* b, int64_t M, int64_t N, hipStream_t stream);
 int launch_cast_f32_to_e4m3(const float* x, void* y, int64_t n, int saturate, hipStream_t stream);
 int launch_quotient_selfcheck(uint64_t* out, int amax_lo, int amax_hi, int mode, hipStream_t stream);

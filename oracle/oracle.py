@@ -276,6 +276,11 @@ def add_bias(x: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     return (x.detach().cpu().float() + b.detach().cpu().float()).to(x.dtype)
 
 
+def add_grad(x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+    """x = (fp32(x) + fp32(y)) -> x.dtype  (megatron_patchs/add_kernel.py:41-62)."""
+    return (x.detach().cpu().float() + y.detach().cpu().float()).to(x.dtype)
+
+
 def fp8_matmul(qa, sa, qb, sb) -> torch.Tensor:
     """bf16 out[PM, PNw] of DeepLinear's GEMM call (fp8.py:307-311); sa may be
     column-major.  Third-party boundary: see the module header."""

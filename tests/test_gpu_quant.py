@@ -392,3 +392,28 @@ def test_quant_input_broadcast_rows():
     assert L.mdy_act_quant(p, p + 1024, p + 2048, 4, 128, 64, 4, 128, 1, 1, 0, None) == -2
     assert L.mdy_act_quant(p, p + 1024, p + 2048, 1, 128, 64, 1, 128, 1, 1, 0, None) == 0
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("xd,yd", [(torch.float32, torch.bfloat16), (torch.float32, torch.float32),
+                                   (torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32)])
+def test_add_grad_bit_exact(xd, yd):
+    """main_grad += wgrad (megatron_patchs/add_kernel.py:55-62): one fp32 add and one rounding, so bit-exact against the
+    oracle (and against numpy's float32 add for the fp32 accumulator); odd sizes take the masked tail."""
+    from mdy_triton_amd.megatron_patchs.add_kernel import add_grad
+    from mdy_triton_amd.megatron_patchs.manger import CustomManger
+    g = torch.Generator().manual_seed(3)
+    for shape in ((1,), (2047,), (300, 513), (4, 128, 256)):
+        x = torch.randn(*shape, generator=g).to(xd)
+        y = (torch.randn(*shape, generator=g) * 3).to(yd)
+        want = O.add_grad(x, y)
+        xg = x.to(DEV)
+        out = CustomManger.add_grad(xg, y.to(DEV))
+        assert out.data_ptr() == xg.data_ptr() and out.dtype == xd
+        assert torch.equal(out.cpu().view(torch.int32 if xd == torch.float32 else torch.int16),
+                           want.view(torch.int32 if xd == torch.float32 else torch.int16))
+        if xd == torch.float32:
+            assert np.array_equal(out.cpu().numpy(), x.numpy() + y.float().numpy())
+    with pytest.raises(AssertionError):
+        add_grad(torch.zeros(4, 4, device=DEV).t(), torch.zeros(4, 4, device=DEV))
+    with pytest.raises(TypeError):
+        add_grad(torch.zeros(4, device=DEV, dtype=torch.float16), torch.zeros(4, device=DEV))
