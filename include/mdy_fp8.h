@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define MDY_FP8_ABI_VERSION 8
+#define MDY_FP8_ABI_VERSION 9
 
 /* error codes (negative = argument rejected before any launch) */
 #define MDY_OK 0
@@ -67,6 +67,16 @@ const char* mdy_fp8_last_error(void);
 int mdy_act_quant(const void* x, void* y, float* s, int64_t M, int64_t K, int64_t x_row_stride,
                   int64_t PM, int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode,
                   void* stream);
+
+/* mdy_act_quant for inputs that are not bf16: the reference kernels load with .to(tl.float32) and so also take
+ * fp16 and fp32 tensors (offical_kernel.py:12, fp8.py:108); every type is quantized from its exact fp32 value.
+ * x_dtype = MDY_XT_BF16 is mdy_act_quant itself; for the other two the quotient is an IEEE division per element
+ * (slower than the bf16 kernel, same results as the reference's arithmetic).  Strides in elements of x_dtype. */
+#define MDY_XT_BF16 0
+#define MDY_XT_F16 1
+#define MDY_XT_F32 2
+int mdy_act_quant_typed(const void* x, int x_dtype, void* y, float* s, int64_t M, int64_t K, int64_t x_row_stride,
+                        int64_t PM, int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode, void* stream);
 
 /* 128x128 block weight quantizer.
  * Replaces quant_weight(only_forward=True/False) (fp8.py:206-247, kernel :171-203)

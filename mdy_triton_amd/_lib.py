@@ -10,7 +10,7 @@ import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libmdyfp8.so")
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 _lock = threading.Lock()
 _lib = None
@@ -22,6 +22,7 @@ _int = ctypes.c_int
 # name -> argtypes; every function returns int except the two noted below.
 SIGNATURES = {
     "mdy_act_quant": [_p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p],
+    "mdy_act_quant_typed": [_p, _int, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p],
     "mdy_weight_quant": [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p],
     "mdy_quant_transpose": [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p],
     "mdy_fp8_grouped_gemm_nt": [_p, _p, _i64, _i64, _p, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p],

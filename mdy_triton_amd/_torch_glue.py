@@ -8,6 +8,7 @@ from . import _lib
 
 FP8 = torch.float8_e4m3fn
 DT_CODE = {torch.bfloat16: 0, torch.float32: 1}
+XT_CODE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}      # input types of the activation quantizer
 
 
 def require_gpu(*tensors):
@@ -18,6 +19,13 @@ def require_gpu(*tensors):
             raise RuntimeError(
                 "mdy_triton_amd operators run on a ROCm GPU only (got a %s tensor); there is no CPU path" % t.device)
     return tensors[0].device
+
+
+def xt_code(x, who):
+    try:
+        return XT_CODE[x.dtype]
+    except KeyError:
+        raise TypeError("%s expects a bfloat16, float16 or float32 tensor, got %s" % (who, x.dtype)) from None
 
 
 def ptr(t):

@@ -44,6 +44,51 @@ __device__ __forceinline__ uint4 load8(const uint16_t* __restrict__ x, int row, 
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
+// The same 8 values as fp32 for an input of type XT (0 bf16, 1 fp16, 2 fp32), zeros outside the M x K matrix.
+// The reference kernels load with .to(tl.float32), so every input type is quantized from its exact fp32 value.
+template <int XT, bool VEC>
+__device__ __forceinline__ void load8_f32(const void* __restrict__ x, int row, int col, int M, int K, int64_t x_row_stride,
+                                          float (&f)[8]) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = 0.0f;
+    if (row >= M || col >= K) return;
+    if (XT == 1) {
+        const _Float16* p = static_cast<const _Float16*>(x) + (int64_t)row * x_row_stride + col;
+        if (VEC) {
+            const uint4 v = load_nt16(p);
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                f[2 * i] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[i] & 0xFFFFu));
+                f[2 * i + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[i] >> 16));
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (col + i < K) f[i] = (float)p[i];
+        }
+    } else {
+        const float* p = static_cast<const float*>(x) + (int64_t)row * x_row_stride + col;
+        if (VEC) {
+            const uint4 a = load_nt16(p), b = load_nt16(p + 4);
+            f[0] = __uint_as_float(a.x); f[1] = __uint_as_float(a.y); f[2] = __uint_as_float(a.z); f[3] = __uint_as_float(a.w);
+            f[4] = __uint_as_float(b.x); f[5] = __uint_as_float(b.y); f[6] = __uint_as_float(b.z); f[7] = __uint_as_float(b.w);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (col + i < K) f[i] = p[i];
+        }
+    }
+}
+__device__ __forceinline__ float group_max8(const float (&f)[8]) {
+    float m = 0.0f;
+    m = fmaxf(fmaxf(fabsf(f[0]), fabsf(f[1])), m);
+    m = fmaxf(fmaxf(fabsf(f[2]), fabsf(f[3])), m);
+    m = fmaxf(fmaxf(fabsf(f[4]), fabsf(f[5])), m);
+    m = fmaxf(fmaxf(fabsf(f[6]), fabsf(f[7])), m);
+    return row16_max(m);
+}
+
 // the lane's 8 values as fp32 and the absmax of its 128-element group (16 lanes)
 __device__ __forceinline__ float unpack8_group_max(const uint4& raw, float (&f)[8]) {
     f[0] = bf16_lo(raw.x); f[1] = bf16_hi(raw.x);
@@ -137,6 +182,52 @@ __global__ __launch_bounds__(512) void act_quant_cm_kernel(const uint16_t* __res
         const int row = rb0 + rr, c = blockIdx.x * 512 + g * 128;
         if (row < PM && c < PK) s[(int64_t)(c >> 7) * s_col_stride + row] = lds_sc[g][rr];
     }
+}
+
+// fp16 / fp32 inputs: the same block shape as act_quant_kernel (8 rows x 512 columns, plain arrangement), the
+// quotient by IEEE division (the reciprocal form is proven for bf16 inputs only).
+template <int MODE, int XT, bool VEC>
+__global__ __launch_bounds__(256) void act_quant_typed_kernel(const void* __restrict__ x, uint8_t* __restrict__ y,
+                                                               float* __restrict__ s, int M, int K, int64_t x_row_stride,
+                                                               int PM, int PK, int64_t s_row_stride, int64_t s_col_stride) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int col = blockIdx.x * 512 + lane * 8;
+    const int row0 = block_row() * kAqRowsPerBlock + wave * kAqRowsPerWave;
+    float f[kAqRowsPerWave][8];
+#pragma unroll
+    for (int r = 0; r < kAqRowsPerWave; ++r) load8_f32<XT, VEC>(x, row0 + r, col, M, K, x_row_stride, f[r]);
+#pragma unroll
+    for (int r = 0; r < kAqRowsPerWave; ++r) {
+        const int row = row0 + r;
+        const float amax = group_max8(f[r]);
+        const float sc = group_scale<MODE>(amax);
+        const uint2 packed = quantize8_scaled<MODE>(f[r], sc, 0.0f, false);
+        if (row < PM && col < PK) {
+            store_nt8(y + (int64_t)row * PK + col, packed);
+            if ((lane & 15) == 0) s[(int64_t)row * s_row_stride + (int64_t)(col >> 7) * s_col_stride] = sc;
+        }
+    }
+}
+
+// x_dtype: 0 bf16 (launch_act_quant), 1 fp16, 2 fp32
+int launch_act_quant_typed(const void* x, int x_dtype, void* y, float* s, int64_t M, int64_t K, int64_t x_row_stride,
+                           int64_t PM, int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode, hipStream_t stream) {
+    if (x_dtype == 0) return launch_act_quant(x, y, s, M, K, x_row_stride, PM, PK, s_row_stride, s_col_stride, mode, stream);
+    if (PM == 0 || PK == 0) return 0;
+    const int esz = x_dtype == 1 ? 2 : 4;
+    const bool vec = (K % 8 == 0) && ((x_row_stride * esz) % 16 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+    dim3 grid;
+    if (!grid_rows((PK + 511) / 512, (PM + kAqRowsPerBlock - 1) / kAqRowsPerBlock, grid)) return kErrTooManyBlocks;
+    uint8_t* yp = static_cast<uint8_t*>(y);
+#define MDY_AQT(MODE, XT, VEC)                                                                                         \
+    hipLaunchKernelGGL((act_quant_typed_kernel<MODE, XT, VEC>), grid, dim3(256), 0, stream, x, yp, s, (int)M, (int)K, \
+                       x_row_stride, (int)PM, (int)PK, s_row_stride, s_col_stride)
+#define MDY_AQT_V(MODE, XT) do { if (vec) MDY_AQT(MODE, XT, true); else MDY_AQT(MODE, XT, false); } while (0)
+    if (mode == 0) { if (x_dtype == 1) MDY_AQT_V(0, 1); else MDY_AQT_V(0, 2); }
+    else { if (x_dtype == 1) MDY_AQT_V(1, 1); else MDY_AQT_V(1, 2); }
+#undef MDY_AQT_V
+#undef MDY_AQT
+    return (int)hipGetLastError();
 }
 
 int launch_act_quant(const void* x, void* y, float* s, int64_t M, int64_t K, int64_t x_row_stride, int64_t PM,

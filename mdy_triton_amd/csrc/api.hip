@@ -74,6 +74,26 @@ int mdy_act_quant(const void* x, void* y, float* s, int64_t M, int64_t K, int64_
                     "act_quant");
 }
 
+int mdy_act_quant_typed(const void* x, int x_dtype, void* y, float* s, int64_t M, int64_t K, int64_t x_row_stride, int64_t PM,
+                        int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode, void* stream) {
+    if (x_dtype == MDY_XT_BF16)
+        return mdy_act_quant(x, y, s, M, K, x_row_stride, PM, PK, s_row_stride, s_col_stride, mode, stream);
+    if (x_dtype != MDY_XT_F16 && x_dtype != MDY_XT_F32) return fail(MDY_E_DTYPE, "act_quant_typed: unknown x_dtype %d", x_dtype);
+    if (mode != MDY_QUANT_OFFICIAL && mode != MDY_QUANT_DEEPLINEAR) return fail(MDY_E_DTYPE, "act_quant_typed: unknown mode %d", mode);
+    if (M < 0 || K < 0 || PM < M || PK < K || PM > kMaxDim || PK > kMaxDim)
+        return fail(MDY_E_SHAPE, "act_quant_typed: need 0 <= M <= PM, 0 <= K <= PK");
+    if (PK % 128 != 0) return fail(MDY_E_SHAPE, "act_quant_typed: PK=%lld is not a multiple of 128", (long long)PK);
+    if (PM == 0 || PK == 0) return 0;
+    if (!y || !s || (!x && M > 0 && K > 0)) return fail(MDY_E_NULL, "act_quant_typed: null pointer");
+    if (M > 1 && x_row_stride != 0 && x_row_stride < K) return fail(MDY_E_SHAPE, "act_quant_typed: x_row_stride < K (and not 0)");
+    if (!aligned(y, 8) || !aligned(s, 4) || !aligned(x, x_dtype == MDY_XT_F16 ? 2 : 4))
+        return fail(MDY_E_ALIGN, "act_quant_typed: y must be 8-byte aligned, x and s aligned for their element type");
+    if (int e = check_device()) return e;
+    return launched(mdy::launch_act_quant_typed(x, x_dtype, y, s, M, K, x_row_stride, PM, PK, s_row_stride, s_col_stride, mode,
+                                                static_cast<hipStream_t>(stream)),
+                    "act_quant_typed");
+}
+
 int mdy_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t, int64_t N, int64_t K,
                      int64_t w_row_stride, int64_t w_col_stride, int64_t PN, int64_t PK, int mode, void* stream) {
     if (mode != MDY_QUANT_OFFICIAL && mode != MDY_QUANT_DEEPLINEAR) return fail(MDY_E_DTYPE, "weight_quant: unknown mode %d", mode);

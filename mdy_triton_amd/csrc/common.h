@@ -184,6 +184,8 @@ constexpr int kErrTooManyBlocks = 9;   // hipErrorInvalidConfiguration
 int launch_act_quant(const void* x, void* y, float* s, int64_t M, int64_t K, int64_t x_row_stride,
                      int64_t PM, int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode,
                      hipStream_t stream);
+int launch_act_quant_typed(const void* x, int x_dtype, void* y, float* s, int64_t M, int64_t K, int64_t x_row_stride,
+                           int64_t PM, int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode, hipStream_t stream);
 int launch_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t, int64_t N, int64_t K,
                         int64_t w_row_stride, int64_t w_col_stride, int64_t PN, int64_t PK, int mode,
                         hipStream_t stream);

@@ -10,7 +10,7 @@ from typing import Optional, Tuple
 
 import torch
 
-from ._torch_glue import FP8, check, gemm_workspace, lib, on_device, ptr, require_gpu, stream_ptr, warn_if_scalar_gemm
+from ._torch_glue import FP8, check, gemm_workspace, lib, on_device, ptr, require_gpu, stream_ptr, warn_if_scalar_gemm, xt_code
 
 
 def _cdiv(a: int, b: int) -> int:
@@ -64,8 +64,7 @@ def quant_input(x: torch.Tensor, only_forward: bool = True):
         return _quant_transpose(x, 1, "quant_input")
     if x.dim() != 2:
         raise ValueError("quant_input expects a 2-D tensor")
-    if x.dtype != torch.bfloat16:
-        raise TypeError("quant_input expects bfloat16, got %s" % x.dtype)
+    xt = xt_code(x, "quant_input")
     dev = require_gpu(x)
     M, K = x.shape
     if K > 0 and x.stride(1) != 1:
@@ -76,8 +75,8 @@ def quant_input(x: torch.Tensor, only_forward: bool = True):
     y = torch.empty(PM, PN, device=dev, dtype=FP8)
     s = torch.empty(B, PM, device=dev, dtype=torch.float32)
     with on_device(dev):
-        check(lib().mdy_act_quant(ptr(x), ptr(y), ptr(s), M, K, x.stride(0) if M > 0 else K, PM, PN, 1, PM, 1,
-                                  stream_ptr(dev)), "quant_input")
+        check(lib().mdy_act_quant_typed(ptr(x), xt, ptr(y), ptr(s), M, K, x.stride(0) if M > 0 else K, PM, PN, 1, PM, 1,
+                                        stream_ptr(dev)), "quant_input")
     return y, s.transpose(0, 1), None, None
 
 

@@ -8,7 +8,7 @@ from typing import Optional, Tuple
 
 import torch
 
-from ._torch_glue import FP8, check, gemm_workspace, lib, on_device, out_code, ptr, require_gpu, stream_ptr, warn_if_scalar_gemm
+from ._torch_glue import FP8, check, gemm_workspace, lib, on_device, out_code, ptr, require_gpu, stream_ptr, warn_if_scalar_gemm, xt_code
 
 
 def act_quant(x: torch.Tensor, block_size: int = 128) -> Tuple[torch.Tensor, torch.Tensor]:
@@ -21,15 +21,14 @@ def act_quant(x: torch.Tensor, block_size: int = 128) -> Tuple[torch.Tensor, tor
     assert x.size(-1) % block_size == 0
     if block_size != 128:
         raise ValueError("only block_size=128 is implemented (the reference default)")
-    if x.dtype != torch.bfloat16:
-        raise TypeError("act_quant expects a bfloat16 tensor, got %s" % x.dtype)
+    xt = xt_code(x, "act_quant")      # bf16 runs the tuned kernel; fp16 / fp32 are quantized from their exact fp32 values
     dev = require_gpu(x)
     K = x.size(-1)
     M = x.numel() // K if K else 0
     y = torch.empty_like(x, dtype=FP8)
     s = x.new_empty(*x.size()[:-1], K // block_size, dtype=torch.float32)
     with on_device(dev):
-        check(lib().mdy_act_quant(ptr(x), ptr(y), ptr(s), M, K, K, M, K, K // 128, 1, 0, stream_ptr(dev)), "act_quant")
+        check(lib().mdy_act_quant_typed(ptr(x), xt, ptr(y), ptr(s), M, K, K, M, K, K // 128, 1, 0, stream_ptr(dev)), "act_quant")
     return y, s
 
 

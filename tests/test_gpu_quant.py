@@ -417,3 +417,29 @@ def test_add_grad_bit_exact(xd, yd):
         add_grad(torch.zeros(4, 4, device=DEV).t(), torch.zeros(4, 4, device=DEV))
     with pytest.raises(TypeError):
         add_grad(torch.zeros(4, device=DEV, dtype=torch.float16), torch.zeros(4, device=DEV))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("M,K", [(128, 1024), (37, 384), (1, 7168), (300, 2048)])
+def test_act_quant_and_quant_input_fp16_fp32_inputs(dtype, M, K):
+    """The reference kernels load with .to(tl.float32), so fp16 and fp32 tensors are quantized from their exact
+    fp32 values (offical_kernel.py:12, fp8.py:108): bytes and scales bit-exact against the oracle, whose arithmetic
+    is dtype-agnostic.  fp32 values are not bf16-representable in general, so this also exercises group maxima and
+    quotients that the bf16 kernel never sees."""
+    g = torch.Generator().manual_seed(M + K)
+    x = (torch.randn(M, K, generator=g) * torch.rand(M, 1, generator=g) * 8).to(dtype)
+    x[0, :3] = torch.tensor([0.0, -0.0, 1e-6]).to(dtype)
+    y_ref, s_ref = O.act_quant(x)
+    y, s = m.act_quant(x.to(DEV))
+    assert y.dtype == FP8 and y.shape == x.shape and s.shape == (M, K // 128)
+    assert torch.equal(y.cpu().view(torch.uint8), y_ref.view(torch.uint8)) and torch.equal(s.cpu(), s_ref)
+    q, qs, _, _ = m.quant_input(x.to(DEV), True)
+    rq, rqs, _, _ = O.quant_input(x, True)
+    assert torch.equal(q.cpu().view(torch.uint8), rq.view(torch.uint8)) and torch.equal(qs.cpu().contiguous(), rqs.contiguous())
+    # a row-strided view (column slice of a wider tensor) takes the element-wise loads
+    wide = torch.randn(M, K + 24, generator=g).to(dtype)
+    q2, qs2, _, _ = m.quant_input(wide.to(DEV)[:, 8:8 + K], True)
+    rq2, rqs2, _, _ = O.quant_input(wide[:, 8:8 + K], True)
+    assert torch.equal(q2.cpu().view(torch.uint8), rq2.view(torch.uint8)) and torch.equal(qs2.cpu().contiguous(), rqs2.contiguous())
+    with pytest.raises(TypeError):
+        m.act_quant(torch.zeros(4, 128, device=DEV, dtype=torch.float64))
