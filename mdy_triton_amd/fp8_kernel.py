@@ -201,7 +201,7 @@ def fp8_matmul(x: torch.Tensor, w: torch.Tensor, scale_x: torch.Tensor, scale_w:
         y = fp8_gemm(x2 if x2.is_contiguous() else x2.contiguous(), scale_x.reshape(-1, scale_x.size(-1)).contiguous(),
                      w if w.is_contiguous() else w.contiguous(), scale_w.contiguous(), out_dtype=torch.bfloat16,
                      bias=None if bias is None else bias.to(torch.bfloat16).contiguous())
-        return y.view(*x.shape[:-1], -1)
+        return y.view(*x.shape[:-1], w.size(0))
     assert x.size(0) % 128 == 0, 'in backward dy.T @ x or dy @ w'
     assert bias is None
     dev = require_gpu(x, w, scale_x, scale_w)
@@ -257,7 +257,9 @@ def _official_linear_backward(x2, w, dy2, need_dx, need_dw, fp8_dtype=FP8):
     if need_dw:
         _, _, qxt, sxt = _act_quant_transposed(x2, False, "Fp8Linear.backward")
         dw = torch.empty(N, K, device=dev, dtype=torch.bfloat16)
-        if N * K > 0:
+        if qdyt.size(1) == 0:
+            dw.zero_()                                   # no tokens: an empty sum
+        elif N * K > 0:
             with on_device(dev):
                 check(lib().mdy_fp8_gemm_nt_rowscaled(ptr(qdyt), ptr(sdyt), sdyt.stride(0), sdyt.stride(1), ptr(qxt), ptr(sxt),
                                                       sxt.stride(0), sxt.stride(1), ptr(dw), N, K, qdyt.size(1), 0,
@@ -283,7 +285,7 @@ class _Fp8LinearFunction(torch.autograd.Function):
         ctx.bias = bias
         ctx.fp8_dtype = fp8_dtype
         ctx.input_shape = input_shape
-        return y.view(*input_shape[:-1], -1)
+        return y.view(*input_shape[:-1], w.size(0))
 
     @staticmethod
     def backward(ctx, dy):

@@ -145,3 +145,15 @@ def test_fp8_linear_forward_backward(shape, N, bias):
     assert close(xg2.grad, ref_dx)
     with pytest.raises(TypeError, match="float8_e4m3fn"):
         m.Fp8Linear(K, N, dtype=torch.bfloat16, fp8_dtype=torch.float8_e5m2)
+
+
+def test_fp8_linear_without_tokens():
+    """An empty batch: empty output, zero weight gradient, empty input gradient (no kernel is given a zero extent)."""
+    lin = m.Fp8Linear(256, 128, bias=True, dtype=torch.bfloat16, device=DEV)
+    x = torch.zeros(0, 256, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    out = lin(x)
+    assert out.shape == (0, 128)
+    out.sum().backward()
+    assert x.grad.shape == (0, 256) and torch.count_nonzero(lin.weight.grad) == 0 and torch.count_nonzero(lin.bias.grad) == 0
+    yt, st = m.act_quant_block(x.detach(), transpose=True)
+    assert yt.shape == (256, 0) and st.shape == (256, 0)
