@@ -275,7 +275,7 @@ def sustained(torch, fn, seconds=2.0, batch=10):
     return us, sampler.summary(half)
 
 
-def cpu_baseline(torch, kind, M, N, K, xq, xs, wq, ws):
+def cpu_baseline(torch, kind, M, N, K, xq, xs, wq, ws, x=None):
     """The CPU oracle (dequantize activations + dequantize weights + fp32 matmul -> bf16) on a
     bounded sample: `rows` activation rows (all of them up to 4096) against the full weight,
     one pass.  If rows < M the row-proportional parts are extrapolated linearly."""
@@ -296,6 +296,19 @@ def cpu_baseline(torch, kind, M, N, K, xq, xs, wq, ws):
     t3 = time.perf_counter()
     t_w, t_a, t_mm = t1 - t0, t2 - t1, t3 - t2
     full = t_w + (t_a + t_mm) * (M / rows)
+    # the two HBM-bound operators on the same host cores, each alone: the oracle's act_quant on the workload's
+    # activations, and its weight_dequant to bf16 (what the GPU kernel writes)
+    extra = {}
+    if x is not None:
+        xc = x[:rows].cpu()
+        t4 = time.perf_counter()
+        O.act_quant(xc)
+        t5 = time.perf_counter()
+        extra["act_quant"] = {"GB/s": round(3.03125 * rows * K / (t5 - t4) / 1e9, 2), "s": round(t5 - t4, 3), "rows": rows}
+    t6 = time.perf_counter()
+    O.weight_dequant(b, b_s, dtype=torch.bfloat16)
+    t7 = time.perf_counter()
+    extra["weight_dequant"] = {"GB/s": round((3.0 * N * K + 4.0 * b_s.numel()) / (t7 - t6) / 1e9, 2), "s": round(t7 - t6, 3)}
     model = ""
     try:
         for line in open("/proc/cpuinfo"):
@@ -313,6 +326,7 @@ def cpu_baseline(torch, kind, M, N, K, xq, xs, wq, ws):
                    "fp32 matmul %.2f s; row-proportional parts extrapolated to %d rows -> %.1f s per step; cpu: %s"
                    % (rows, M, N, K, t_w, t_a, t_mm, M, full, model)),
         "checksum": float(c.float().abs().mean()),
+        "kernels": extra,
     }, c
 
 
@@ -508,7 +522,7 @@ def main():
     parity_ok = bool(torch.equal(xq[rows.to(dev)].cpu().view(torch.uint8), yq_ref.view(torch.uint8))) \
         and bool(torch.equal(xs[rows.to(dev)].cpu(), s_ref))
     if not args.no_cpu:
-        result["cpu_baseline"], c_ref = cpu_baseline(torch, kind, M, N, K, xq, xs, wq, ws)
+        result["cpu_baseline"], c_ref = cpu_baseline(torch, kind, M, N, K, xq, xs, wq, ws, x)
         got = out[:c_ref.size(0)].float().cpu()
         parity_ok = parity_ok and bool(torch.allclose(got, c_ref.float(), rtol=1e-2, atol=1e-2))
         result["parity_rows_checked"] = int(c_ref.size(0))
@@ -612,6 +626,21 @@ def table(torch, m, timer, dev):
             lin(xg).backward(dy)
         line("ref DeepLinear fwd+bwd %dx%dx%d (test_fp8.ipynb:172)" % (Mr, Nr, Kr), timer.run(fwd_bwd, 6)[0],
              6.0 * Mr * Nr * Kr, "TFLOP/s", PEAK_FP8_TFLOPS)
+        del lin, xg, dy
+    for d in (4096, 7168, 8192):          # fp8-benchmark.ipynb:351-359 (fwd), :456-464 (bwd): x = [8192, d], W = [d, d]
+        lin = m.Fp8Linear(d, d, bias=False, dtype=torch.bfloat16, device=dev)
+        xg = torch.randn(8192, d, device=dev).bfloat16().requires_grad_(True)
+        dy = torch.randn(8192, d, device=dev).bfloat16()
+        with torch.no_grad():
+            fwd_us = timer.run(lambda: lin(xg), 8)[0]
+        line("ref Fp8Linear fwd 8192x%dx%d (fp8-benchmark.ipynb:351)" % (d, d), fwd_us, 2.0 * 8192 * d * d, "TFLOP/s", PEAK_FP8_TFLOPS)
+
+        def fwd_bwd():
+            lin.zero_grad(set_to_none=True)
+            xg.grad = None
+            lin(xg).backward(dy)
+        both_us = timer.run(fwd_bwd, 6)[0]
+        line("ref Fp8Linear bwd 8192x%dx%d = fwd+bwd - fwd (:456)" % (d, d), both_us - fwd_us, 4.0 * 8192 * d * d, "TFLOP/s", PEAK_FP8_TFLOPS)
         del lin, xg, dy
     # training-time operators at the C3 shapes (DeepLinear dialect): bytes = 2 in + 1 out + 1 transposed out per element
     seed, kind, M, N, K, _ = WORKLOADS["C3"]
