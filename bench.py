@@ -611,7 +611,7 @@ def table(torch, m, timer, dev):
     xr = torch.randn(16384, 4096, device=dev).bfloat16()
     line("ref act_quant 16384x4096 (fp8-benchmark.ipynb:141)", timer.run(lambda: m.act_quant(xr), 20)[0], 3.03125 * 16384 * 4096, "GB/s", PEAK_HBM_GBS)
     del xr
-    for (Mr, Nr, Kr) in ((8192, 8192, 8192), (16384, 4096, 4096), (16384, 4096, 7168), (16384, 4096, 16384)):
+    for (Mr, Nr, Kr) in ((8192, 8192, 8192), (16384, 4096, 1024), (16384, 16384, 4096), (16384, 28672, 7168), (16384, 32768, 8192)):   # test_fp8.ipynb:212-221: M = 16384, N = 4 K
         lin = m.DeepLinear(Kr, Nr, bias=False, dtype=torch.bfloat16, device=dev)
         lin.cache_weight = True
         xg = torch.randn(Mr, Kr, device=dev).bfloat16().requires_grad_(True)
