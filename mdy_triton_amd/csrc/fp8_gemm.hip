@@ -284,7 +284,7 @@ template <int MT, typename OUT>
 __global__ __launch_bounds__(512) void fp8_gemm_strip_kernel(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
-    const uint16_t* __restrict__ bias, int N, int K, int kb_per, const GroupTable tbl) {
+    const uint16_t* __restrict__ bias, int N, int K, const GroupTable tbl) {
     constexpr int ROWS = MT * 16, KC = kStripKC;
     __shared__ __attribute__((aligned(1024))) uint8_t lds_a[2][KC][ROWS * 128];
     __shared__ __attribute__((aligned(256))) float lds_sa[2][KC][64];
@@ -301,12 +301,7 @@ __global__ __launch_bounds__(512) void fp8_gemm_strip_kernel(
     if (rows <= 0) return;
     const int n0 = blockIdx.x * 128;
     const int KB = K >> 7, NB = (N + 127) >> 7;
-    // K slice of this workgroup: blockIdx.z takes K blocks z * kb_per .. (all of them when the grid has one z layer)
-    // and writes its sums into layer z of c ([gridDim.z][rows][N]: the fp32 slabs that splitk_reduce_kernel adds up)
-    const int kb0 = blockIdx.z * kb_per, kb_end = min(KB, kb0 + kb_per);
-    if (kb0 >= kb_end) return;
-    const int steps = (kb_end - kb0 + KC - 1) / KC;
-    c += (size_t)blockIdx.z * (size_t)m_total * N;
+    const int steps = (KB + KC - 1) / KC;
     const uint8_t* bg = b + (size_t)g * N * K;
 
     // ---- copies: activation rows (8 rows x 128 bytes per instruction) and their scales (one row per lane)
@@ -325,9 +320,9 @@ __global__ __launch_bounds__(512) void fp8_gemm_strip_kernel(
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
             const int j = wave + 8 * t, kc = j % KC, rg = j / KC;
-            dma16(ra, voff, rg * 8 * K + (kb0 + step * KC + kc) * 128, la0 + (buf * KC + kc) * (ROWS * 128) + rg * 1024);
+            dma16(ra, voff, rg * 8 * K + (step * KC + kc) * 128, la0 + (buf * KC + kc) * (ROWS * 128) + rg * 1024);
         }
-        dma4(rs, s_voff, min(kb0 + step * KC + wave, KB - 1) * as_cs * 4, ls0 + buf * ls_buf);
+        dma4(rs, s_voff, min(step * KC + wave, KB - 1) * as_cs * 4, ls0 + buf * ls_buf);
     };
 
     // ---- weight fragments straight from global memory: lane -> row lane%16, 32-byte K slice lane/16
@@ -337,7 +332,7 @@ __global__ __launch_bounds__(512) void fp8_gemm_strip_kernel(
     auto load_b = [&](int step) {
 #pragma unroll
         for (int kc = 0; kc < KC; ++kc) {
-            const int kb = min(kb0 + step * KC + kc, KB - 1);      // the clamped duplicates are never used
+            const int kb = min(step * KC + kc, KB - 1);      // the clamped duplicates are never used
             blo[kc] = load_nt16(bp + (size_t)kb * 128);
             bhi[kc] = load_nt16(bp + (size_t)kb * 128 + 16);
         }
@@ -362,8 +357,8 @@ __global__ __launch_bounds__(512) void fp8_gemm_strip_kernel(
         if (step + 1 < steps) copy_step(step + 1, buf ^ 1);
 #pragma unroll
         for (int kc = 0; kc < KC; ++kc) {
-            const int kb = kb0 + step * KC + kc;
-            if (kb < kb_end) {
+            const int kb = step * KC + kc;
+            if (kb < KB) {
                 const float sb = lds_bs[kb];
                 const intx8 fb = intx8{(int)blo[kc].x, (int)blo[kc].y, (int)blo[kc].z, (int)blo[kc].w,
                                        (int)bhi[kc].x, (int)bhi[kc].y, (int)bhi[kc].z, (int)bhi[kc].w};
@@ -546,7 +541,7 @@ static int launch_strip(const uint8_t* a, const float* a_s, int64_t as_rs, int64
     dim3 grid((unsigned)((N + 127) / 128), (unsigned)G), block(512);
 #define MDY_STRIP(MT)                                                                                              \
     hipLaunchKernelGGL((fp8_gemm_strip_kernel<MT, OUT>), grid, block, 0, stream, a, a_s, (int)as_rs, (int)as_cs, as_bytes, b, \
-                       b_s, c, bias, N, K, K >> 7, tbl)
+                       b_s, c, bias, N, K, tbl)
     if (max_rows <= 16) MDY_STRIP(1);
     else if (max_rows <= 32) MDY_STRIP(2);
     else if (max_rows <= 48) MDY_STRIP(3);
