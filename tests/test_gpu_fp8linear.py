@@ -1,6 +1,8 @@
 """GPU parity of the official-dialect linear layer (deepseekv3/fp8_kernel.py: act_quant_block, fp8_matmul, Fp8Linear)
 against the CPU oracle: quantizer bytes and scales bit-exact, GEMMs within rtol = atol = 1e-2, exactly
 representable cases bit for bit."""
+import math
+
 import numpy as np
 import pytest
 import torch
@@ -157,3 +159,65 @@ def test_fp8_linear_without_tokens():
     assert x.grad.shape == (0, 256) and torch.count_nonzero(lin.weight.grad) == 0 and torch.count_nonzero(lin.bias.grad) == 0
     yt, st = m.act_quant_block(x.detach(), transpose=True)
     assert yt.shape == (256, 0) and st.shape == (256, 0)
+
+
+def test_act_quant_block_non_finite_and_zero_groups():
+    """The official dialect has no eps and no clamp (fp8_kernel.py:52-54): an all-zero group has scale 0 and NaN bytes
+    (0 / 0), an infinite element makes its group's scale infinite (finite / inf = 0, inf / inf = NaN), and a NaN
+    element is ignored by the group maximum (tl.max / v_max_f32) and stays NaN.  Both copies, compared with the oracle
+    on the input whose NaNs are zeroed for the maximum only - the same convention as the forward quantizer's test."""
+    g = torch.Generator().manual_seed(6)
+    M, N = 256, 256
+    x = torch.randn(M, N, generator=g).bfloat16()
+    x[:128, 5] = 0.0                      # column group (0, 5) all zero
+    x[7, 128:256] = 0.0                   # row group (7, 1) all zero
+    x[200, 17] = float("inf")
+    x[130, 140] = float("nan")
+    y, s = m.act_quant_block(x.to(DEV))
+    yt, st = m.act_quant_block(x.to(DEV), transpose=True)
+    xz = torch.where(torch.isnan(x), torch.zeros_like(x), x)
+    yr, sr = O.act_quant_block(xz)
+    ytr, str_ = O.act_quant_block(xz, transpose=True)
+    assert torch.equal(s.cpu(), sr) and torch.equal(st.cpu(), str_)
+    assert s[7, 1].item() == 0.0 and st[5, 0].item() == 0.0 and math.isinf(s[200, 0].item()) and math.isinf(st[17, 1].item())
+    def same(got, ref, nan_at):
+        got = got.cpu().float()
+        ref = ref.float().clone()
+        ref[nan_at] = float("nan")
+        return torch.equal(torch.isnan(got), torch.isnan(ref)) and torch.equal(got[~torch.isnan(ref)], ref[~torch.isnan(ref)])
+    assert same(y, yr, (130, 140)) and same(yt, ytr, (140, 130))
+    assert torch.isnan(y.cpu().float()[7, 128:256]).all() and torch.isnan(yt.cpu().float()[5, :128]).all()
+    assert torch.isnan(y.cpu().float()[200, 17]) and (y.cpu().float()[200, :17] == 0).all()
+
+
+def test_rowscaled_gemm_non_finite_values():
+    """A NaN operand byte poisons exactly its output row / column; an infinite scale makes its row (or column) infinite
+    with the sign of the block's partial sum, NaN where that sum is zero; a zero scale drops the block: the pattern of
+    the reference's accumulation (fp8_kernel.py:196-203) evaluated block by block."""
+    g = torch.Generator().manual_seed(13)
+    M, N, K = 128, 200, 384
+    a = torch.randint(-6, 7, (M, K), generator=g).float().to(FP8)
+    b = torch.randint(-6, 7, (N, K), generator=g).float().to(FP8)
+    sa = torch.rand(M, 3, generator=g) + 0.5
+    sb = torch.rand(N, 3, generator=g) + 0.5
+    a.view(torch.uint8)[1, 3] = 0x7F
+    b.view(torch.uint8)[5, K - 1] = 0xFF
+    sa[2, 2] = float("inf")
+    sb[9, 0] = float("inf")
+    sa[3, 0] = 0.0
+    ref = torch.zeros(M, N)
+    for kb in range(3):
+        part = a[:, kb * 128:(kb + 1) * 128].float() @ b[:, kb * 128:(kb + 1) * 128].float().t()
+        ref = ref + part * (sa[:, kb][:, None] * sb[:, kb][None, :])
+    out = torch.empty(M, N, device=DEV, dtype=torch.float32)
+    from mdy_triton_amd import _lib
+    ad, bd, sad, sbd = a.to(DEV), b.to(DEV), sa.to(DEV), sb.to(DEV)
+    rc = _lib.load().mdy_fp8_gemm_nt_rowscaled(ad.data_ptr(), sad.data_ptr(), 3, 1, bd.data_ptr(), sbd.data_ptr(), 3, 1,
+                                                out.data_ptr(), M, N, K, 1, None)
+    torch.cuda.synchronize()
+    assert rc == 0
+    got = out.cpu()
+    assert torch.equal(torch.isnan(got), torch.isnan(ref)) and torch.isnan(got[1]).all() and torch.isnan(got[:, 5]).all()
+    assert torch.equal(torch.isinf(got), torch.isinf(ref)) and torch.equal(got[torch.isinf(ref)], ref[torch.isinf(ref)])
+    fin = torch.isfinite(ref)
+    assert fin[4:].any() and torch.allclose(got[fin], ref[fin], rtol=1e-4, atol=1e-2)
