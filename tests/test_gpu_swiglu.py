@@ -254,3 +254,20 @@ def test_fp8_mlp_official_dialect_three_paths(order):
     assert _within(act_d.grad, dact_r) and _within(dwd_d, dwd_r)
     dx_r, dwug_r, _ = O.fp8_linear_backward(x, w_ug, ug_d.grad.cpu(), False)
     assert _within(dx_d, dx_r) and _within(dwug_d, dwug_r)
+
+
+def test_megatron_swiglu_impl():
+    """megatron_patchs/swiglu.py: swiglu_impl(x, bias, fp8_input_store) = silu(first half) * second half, with the
+    matching gradient."""
+    from mdy_triton_amd.megatron_patchs.swiglu import fused_up_gate_silu_no_split, swiglu_impl
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(3, 40, 512, generator=g).bfloat16()
+    dy = torch.randn(3, 40, 256, generator=g).bfloat16()
+    xg = x.to(DEV).requires_grad_(True)
+    y = swiglu_impl(xg, None)
+    y.backward(dy.to(DEV))
+    ref = O.silu_fwd(x, "gate-up")
+    assert y.shape == (3, 40, 256) and torch.allclose(y.float().cpu(), ref.float(), rtol=2 ** -7, atol=1e-6)
+    dref = O.silu_bwd(dy, x, "gate-up")
+    assert torch.allclose(xg.grad.float().cpu(), dref.float(), rtol=2 ** -6, atol=1e-3)
+    assert torch.equal(fused_up_gate_silu_no_split(x.to(DEV), "gate-up"), y.detach())
