@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define MDY_FP8_ABI_VERSION 9
+#define MDY_FP8_ABI_VERSION 10
 
 /* error codes (negative = argument rejected before any launch) */
 #define MDY_OK 0
@@ -68,15 +68,19 @@ int mdy_act_quant(const void* x, void* y, float* s, int64_t M, int64_t K, int64_
                   int64_t PM, int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode,
                   void* stream);
 
-/* mdy_act_quant for inputs that are not bf16: the reference kernels load with .to(tl.float32) and so also take
- * fp16 and fp32 tensors (offical_kernel.py:12, fp8.py:108); every type is quantized from its exact fp32 value.
- * x_dtype = MDY_XT_BF16 is mdy_act_quant itself; for the other two the quotient is an IEEE division per element
- * (slower than the bf16 kernel, same results as the reference's arithmetic).  Strides in elements of x_dtype. */
+/* The general form of mdy_act_quant: inputs that are not bf16 and group widths other than 128.  The reference kernels
+ * load with .to(tl.float32) and so also take fp16 and fp32 tensors (offical_kernel.py:12, fp8.py:108), and act_quant
+ * takes any block_size (offical_kernel.py:21-27); every input type is quantized from its exact fp32 value.
+ * x_dtype = MDY_XT_BF16 with block_size = 128 is mdy_act_quant itself (the tuned kernel); everything else runs a kernel
+ * whose quotient is an IEEE division per element (same results as the reference's arithmetic, slower).
+ * block_size: a power of two from 8 to 512; PK % block_size == 0; the scale of row m, group g is at
+ * s[m * s_row_stride + g * s_col_stride].  Strides of x in elements of x_dtype. */
 #define MDY_XT_BF16 0
 #define MDY_XT_F16 1
 #define MDY_XT_F32 2
-int mdy_act_quant_typed(const void* x, int x_dtype, void* y, float* s, int64_t M, int64_t K, int64_t x_row_stride,
-                        int64_t PM, int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode, void* stream);
+int mdy_act_quant_typed(const void* x, int x_dtype, int block_size, void* y, float* s, int64_t M, int64_t K,
+                        int64_t x_row_stride, int64_t PM, int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode,
+                        void* stream);
 
 /* 128x128 block weight quantizer.
  * Replaces quant_weight(only_forward=True/False) (fp8.py:206-247, kernel :171-203)
@@ -181,6 +185,10 @@ int mdy_swiglu_bwd(const void* x, const void* dy, void* dx, int64_t M, int64_t N
  */
 int mdy_weight_dequant(const void* x, const float* s, void* y, int64_t N, int64_t K, int out_dtype,
                        void* stream);
+/* The same with square scale blocks of block_size x block_size (a power of two >= 8; s is
+ * [ceil(N/block_size), ceil(K/block_size)]): the reference's weight_dequant takes any block_size (offical_kernel.py:46). */
+int mdy_weight_dequant_block(const void* x, const float* s, void* y, int64_t N, int64_t K, int block_size, int out_dtype,
+                             void* stream);
 
 /* Block-scaled FP8 GEMM, NT layout:
  *   c[m,n] = sum_kb (sum_{k in kb} a[m,k] * b[n,k]) * a_s[m,kb] * b_s[n/128,kb]  (+ bias[n])

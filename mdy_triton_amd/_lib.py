@@ -10,7 +10,7 @@ import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libmdyfp8.so")
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 _lock = threading.Lock()
 _lib = None
@@ -22,7 +22,7 @@ _int = ctypes.c_int
 # name -> argtypes; every function returns int except the two noted below.
 SIGNATURES = {
     "mdy_act_quant": [_p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p],
-    "mdy_act_quant_typed": [_p, _int, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p],
+    "mdy_act_quant_typed": [_p, _int, _int, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p],
     "mdy_weight_quant": [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p],
     "mdy_quant_transpose": [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p],
     "mdy_fp8_grouped_gemm_nt": [_p, _p, _i64, _i64, _p, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p],
@@ -31,6 +31,7 @@ SIGNATURES = {
     "mdy_swiglu": [_p, _p, _p, _p, _i64, _i64, _i64, _int, _i64, _i64, _i64, _i64, _int, _p],
     "mdy_swiglu_bwd": [_p, _p, _p, _i64, _i64, _i64, _int, _p],
     "mdy_weight_dequant": [_p, _p, _p, _i64, _i64, _int, _p],
+    "mdy_weight_dequant_block": [_p, _p, _p, _i64, _i64, _int, _int, _p],
     "mdy_fp8_gemm_nt": [_p, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p],
     "mdy_fp8_gemm_nt_ws": [_p, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p, _i64, _p],
     "mdy_fp8_gemm_workspace_bytes": [_i64, _i64, _i64],

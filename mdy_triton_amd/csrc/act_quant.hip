@@ -52,7 +52,11 @@ __device__ __forceinline__ void load8_f32(const void* __restrict__ x, int row, i
 #pragma unroll
     for (int i = 0; i < 8; ++i) f[i] = 0.0f;
     if (row >= M || col >= K) return;
-    if (XT == 1) {
+    if (XT == 0) {
+        const uint4 v = load8<VEC>(static_cast<const uint16_t*>(x), row, col, M, K, x_row_stride);
+        f[0] = bf16_lo(v.x); f[1] = bf16_hi(v.x); f[2] = bf16_lo(v.y); f[3] = bf16_hi(v.y);
+        f[4] = bf16_lo(v.z); f[5] = bf16_hi(v.z); f[6] = bf16_lo(v.w); f[7] = bf16_hi(v.w);
+    } else if (XT == 1) {
         const _Float16* p = static_cast<const _Float16*>(x) + (int64_t)row * x_row_stride + col;
         if (VEC) {
             const uint4 v = load_nt16(p);
@@ -80,13 +84,16 @@ __device__ __forceinline__ void load8_f32(const void* __restrict__ x, int row, i
         }
     }
 }
-__device__ __forceinline__ float group_max8(const float (&f)[8]) {
+// absmax of a quantization group of `lanes` consecutive lanes x 8 values (lanes a power of two, 1..64)
+__device__ __forceinline__ float group_max8(const float (&f)[8], int lanes) {
     float m = 0.0f;
     m = fmaxf(fmaxf(fabsf(f[0]), fabsf(f[1])), m);
     m = fmaxf(fmaxf(fabsf(f[2]), fabsf(f[3])), m);
     m = fmaxf(fmaxf(fabsf(f[4]), fabsf(f[5])), m);
     m = fmaxf(fmaxf(fabsf(f[6]), fabsf(f[7])), m);
-    return row16_max(m);
+    if (lanes == 16) return row16_max(m);
+    for (int off = 1; off < lanes; off <<= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+    return m;
 }
 
 // the lane's 8 values as fp32 and the absmax of its 128-element group (16 lanes)
@@ -184,12 +191,15 @@ __global__ __launch_bounds__(512) void act_quant_cm_kernel(const uint16_t* __res
     }
 }
 
-// fp16 / fp32 inputs: the same block shape as act_quant_kernel (8 rows x 512 columns, plain arrangement), the
-// quotient by IEEE division (the reciprocal form is proven for bf16 inputs only).
+// The general form of the quantizer: fp16 / fp32 inputs, and group widths other than 128 (8 x a power of two lanes, up
+// to 512 elements: the reference's act_quant takes any block_size, offical_kernel.py:21-27).  The same block shape as
+// act_quant_kernel (8 rows x 512 columns, plain arrangement), the quotient by IEEE division (the reciprocal form is
+// proven for bf16 inputs only, and only the 128-wide bf16 case is tuned).
 template <int MODE, int XT, bool VEC>
 __global__ __launch_bounds__(256) void act_quant_typed_kernel(const void* __restrict__ x, uint8_t* __restrict__ y,
                                                                float* __restrict__ s, int M, int K, int64_t x_row_stride,
-                                                               int PM, int PK, int64_t s_row_stride, int64_t s_col_stride) {
+                                                               int PM, int PK, int64_t s_row_stride, int64_t s_col_stride,
+                                                               int group_lanes, int group_shift) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = blockIdx.x * 512 + lane * 8;
     const int row0 = block_row() * kAqRowsPerBlock + wave * kAqRowsPerWave;
@@ -199,32 +209,38 @@ __global__ __launch_bounds__(256) void act_quant_typed_kernel(const void* __rest
 #pragma unroll
     for (int r = 0; r < kAqRowsPerWave; ++r) {
         const int row = row0 + r;
-        const float amax = group_max8(f[r]);
+        const float amax = group_max8(f[r], group_lanes);
         const float sc = group_scale<MODE>(amax);
         const uint2 packed = quantize8_scaled<MODE>(f[r], sc, 0.0f, false);
         if (row < PM && col < PK) {
             store_nt8(y + (int64_t)row * PK + col, packed);
-            if ((lane & 15) == 0) s[(int64_t)row * s_row_stride + (int64_t)(col >> 7) * s_col_stride] = sc;
+            if ((lane & (group_lanes - 1)) == 0) s[(int64_t)row * s_row_stride + (int64_t)(col >> group_shift) * s_col_stride] = sc;
         }
     }
 }
 
-// x_dtype: 0 bf16 (launch_act_quant), 1 fp16, 2 fp32
-int launch_act_quant_typed(const void* x, int x_dtype, void* y, float* s, int64_t M, int64_t K, int64_t x_row_stride,
-                           int64_t PM, int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode, hipStream_t stream) {
-    if (x_dtype == 0) return launch_act_quant(x, y, s, M, K, x_row_stride, PM, PK, s_row_stride, s_col_stride, mode, stream);
+// x_dtype: 0 bf16, 1 fp16, 2 fp32; block_size: 8 x a power of two, 8..512.  bf16 with block_size 128 is launch_act_quant.
+int launch_act_quant_typed(const void* x, int x_dtype, int block_size, void* y, float* s, int64_t M, int64_t K,
+                           int64_t x_row_stride, int64_t PM, int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode,
+                           hipStream_t stream) {
+    if (x_dtype == 0 && block_size == 128)
+        return launch_act_quant(x, y, s, M, K, x_row_stride, PM, PK, s_row_stride, s_col_stride, mode, stream);
     if (PM == 0 || PK == 0) return 0;
-    const int esz = x_dtype == 1 ? 2 : 4;
+    const int esz = x_dtype == 2 ? 4 : 2;
     const bool vec = (K % 8 == 0) && ((x_row_stride * esz) % 16 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+    const int lanes = block_size / 8;
+    int shift = 0;
+    while ((1 << shift) < block_size) ++shift;
     dim3 grid;
     if (!grid_rows((PK + 511) / 512, (PM + kAqRowsPerBlock - 1) / kAqRowsPerBlock, grid)) return kErrTooManyBlocks;
     uint8_t* yp = static_cast<uint8_t*>(y);
 #define MDY_AQT(MODE, XT, VEC)                                                                                         \
     hipLaunchKernelGGL((act_quant_typed_kernel<MODE, XT, VEC>), grid, dim3(256), 0, stream, x, yp, s, (int)M, (int)K, \
-                       x_row_stride, (int)PM, (int)PK, s_row_stride, s_col_stride)
+                       x_row_stride, (int)PM, (int)PK, s_row_stride, s_col_stride, lanes, shift)
 #define MDY_AQT_V(MODE, XT) do { if (vec) MDY_AQT(MODE, XT, true); else MDY_AQT(MODE, XT, false); } while (0)
-    if (mode == 0) { if (x_dtype == 1) MDY_AQT_V(0, 1); else MDY_AQT_V(0, 2); }
-    else { if (x_dtype == 1) MDY_AQT_V(1, 1); else MDY_AQT_V(1, 2); }
+#define MDY_AQT_X(MODE) do { if (x_dtype == 0) MDY_AQT_V(MODE, 0); else if (x_dtype == 1) MDY_AQT_V(MODE, 1); else MDY_AQT_V(MODE, 2); } while (0)
+    if (mode == 0) MDY_AQT_X(0); else MDY_AQT_X(1);
+#undef MDY_AQT_X
 #undef MDY_AQT_V
 #undef MDY_AQT
     return (int)hipGetLastError();

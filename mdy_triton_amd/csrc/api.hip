@@ -74,23 +74,26 @@ int mdy_act_quant(const void* x, void* y, float* s, int64_t M, int64_t K, int64_
                     "act_quant");
 }
 
-int mdy_act_quant_typed(const void* x, int x_dtype, void* y, float* s, int64_t M, int64_t K, int64_t x_row_stride, int64_t PM,
-                        int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode, void* stream) {
-    if (x_dtype == MDY_XT_BF16)
+static bool block_size_ok(int64_t bs, int64_t lo, int64_t hi) { return bs >= lo && bs <= hi && (bs & (bs - 1)) == 0; }
+
+int mdy_act_quant_typed(const void* x, int x_dtype, int block_size, void* y, float* s, int64_t M, int64_t K, int64_t x_row_stride,
+                        int64_t PM, int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode, void* stream) {
+    if (x_dtype == MDY_XT_BF16 && block_size == 128)
         return mdy_act_quant(x, y, s, M, K, x_row_stride, PM, PK, s_row_stride, s_col_stride, mode, stream);
-    if (x_dtype != MDY_XT_F16 && x_dtype != MDY_XT_F32) return fail(MDY_E_DTYPE, "act_quant_typed: unknown x_dtype %d", x_dtype);
+    if (x_dtype != MDY_XT_BF16 && x_dtype != MDY_XT_F16 && x_dtype != MDY_XT_F32) return fail(MDY_E_DTYPE, "act_quant_typed: unknown x_dtype %d", x_dtype);
     if (mode != MDY_QUANT_OFFICIAL && mode != MDY_QUANT_DEEPLINEAR) return fail(MDY_E_DTYPE, "act_quant_typed: unknown mode %d", mode);
+    if (!block_size_ok(block_size, 8, 512)) return fail(MDY_E_SHAPE, "act_quant_typed: block_size=%d must be a power of two from 8 to 512", block_size);
     if (M < 0 || K < 0 || PM < M || PK < K || PM > kMaxDim || PK > kMaxDim)
         return fail(MDY_E_SHAPE, "act_quant_typed: need 0 <= M <= PM, 0 <= K <= PK");
-    if (PK % 128 != 0) return fail(MDY_E_SHAPE, "act_quant_typed: PK=%lld is not a multiple of 128", (long long)PK);
+    if (PK % block_size != 0) return fail(MDY_E_SHAPE, "act_quant_typed: PK=%lld is not a multiple of block_size=%d", (long long)PK, block_size);
     if (PM == 0 || PK == 0) return 0;
     if (!y || !s || (!x && M > 0 && K > 0)) return fail(MDY_E_NULL, "act_quant_typed: null pointer");
     if (M > 1 && x_row_stride != 0 && x_row_stride < K) return fail(MDY_E_SHAPE, "act_quant_typed: x_row_stride < K (and not 0)");
-    if (!aligned(y, 8) || !aligned(s, 4) || !aligned(x, x_dtype == MDY_XT_F16 ? 2 : 4))
+    if (!aligned(y, 8) || !aligned(s, 4) || !aligned(x, x_dtype == MDY_XT_F32 ? 4 : 2))
         return fail(MDY_E_ALIGN, "act_quant_typed: y must be 8-byte aligned, x and s aligned for their element type");
     if (int e = check_device()) return e;
-    return launched(mdy::launch_act_quant_typed(x, x_dtype, y, s, M, K, x_row_stride, PM, PK, s_row_stride, s_col_stride, mode,
-                                                static_cast<hipStream_t>(stream)),
+    return launched(mdy::launch_act_quant_typed(x, x_dtype, block_size, y, s, M, K, x_row_stride, PM, PK, s_row_stride, s_col_stride,
+                                                mode, static_cast<hipStream_t>(stream)),
                     "act_quant_typed");
 }
 
@@ -197,14 +200,20 @@ int mdy_swiglu_bwd(const void* x, const void* dy, void* dx, int64_t M, int64_t N
                     "swiglu_bwd");
 }
 
-int mdy_weight_dequant(const void* x, const float* s, void* y, int64_t N, int64_t K, int out_dtype, void* stream) {
+int mdy_weight_dequant_block(const void* x, const float* s, void* y, int64_t N, int64_t K, int block_size, int out_dtype,
+                             void* stream) {
     if (out_dtype != MDY_DT_BF16 && out_dtype != MDY_DT_F32) return fail(MDY_E_DTYPE, "weight_dequant: unknown out_dtype %d", out_dtype);
+    if (!block_size_ok(block_size, 8, 1 << 20)) return fail(MDY_E_SHAPE, "weight_dequant: block_size=%d must be a power of two >= 8", block_size);
     if (N < 0 || K < 0 || N > kMaxDim || K > kMaxDim) return fail(MDY_E_SHAPE, "weight_dequant: bad shape");
     if (N == 0 || K == 0) return 0;
     if (!x || !s || !y) return fail(MDY_E_NULL, "weight_dequant: null pointer");
     if (!aligned(y, out_dtype == MDY_DT_BF16 ? 2 : 4) || !aligned(s, 4)) return fail(MDY_E_ALIGN, "weight_dequant: misaligned pointer");
     if (int e = check_device()) return e;
-    return launched(mdy::launch_weight_dequant(x, s, y, N, K, out_dtype, static_cast<hipStream_t>(stream)), "weight_dequant");
+    return launched(mdy::launch_weight_dequant(x, s, y, N, K, block_size, out_dtype, static_cast<hipStream_t>(stream)), "weight_dequant");
+}
+
+int mdy_weight_dequant(const void* x, const float* s, void* y, int64_t N, int64_t K, int out_dtype, void* stream) {
+    return mdy_weight_dequant_block(x, s, y, N, K, 128, out_dtype, stream);
 }
 
 int mdy_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,

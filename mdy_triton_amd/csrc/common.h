@@ -184,8 +184,9 @@ constexpr int kErrTooManyBlocks = 9;   // hipErrorInvalidConfiguration
 int launch_act_quant(const void* x, void* y, float* s, int64_t M, int64_t K, int64_t x_row_stride,
                      int64_t PM, int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode,
                      hipStream_t stream);
-int launch_act_quant_typed(const void* x, int x_dtype, void* y, float* s, int64_t M, int64_t K, int64_t x_row_stride,
-                           int64_t PM, int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode, hipStream_t stream);
+int launch_act_quant_typed(const void* x, int x_dtype, int block_size, void* y, float* s, int64_t M, int64_t K,
+                           int64_t x_row_stride, int64_t PM, int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode,
+                           hipStream_t stream);
 int launch_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t, int64_t N, int64_t K,
                         int64_t w_row_stride, int64_t w_col_stride, int64_t PN, int64_t PK, int mode,
                         hipStream_t stream);
@@ -202,7 +203,7 @@ int launch_swiglu(const void* x, void* act, void* y, float* s, int64_t M, int64_
                   hipStream_t stream);
 int launch_swiglu_bwd(const void* x, const void* dy, void* dx, int64_t M, int64_t N, int64_t x_row_stride,
                       int gate_first, hipStream_t stream);
-int launch_weight_dequant(const void* x, const float* s, void* y, int64_t N, int64_t K, int out_dtype,
+int launch_weight_dequant(const void* x, const float* s, void* y, int64_t N, int64_t K, int block_size, int out_dtype,
                           hipStream_t stream);
 int launch_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
                        const void* b, const float* b_s, void* c, const void* bias, int64_t M, int64_t N,

@@ -23,7 +23,7 @@ constexpr int kWdCols = 64 * 8;      // columns per wave pass
 
 template <typename OUT, bool VEC>
 __global__ __launch_bounds__(256) void weight_dequant_kernel(const uint8_t* __restrict__ x, const float* __restrict__ s,
-                                                              OUT* __restrict__ y, int N, int K, int sK) {
+                                                              OUT* __restrict__ y, int N, int K, int sK, int bshift) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int col = blockIdx.x * kWdCols + lane * 8;
@@ -48,7 +48,7 @@ __global__ __launch_bounds__(256) void weight_dequant_kernel(const uint8_t* __re
                     if (col + i < K) w[i >> 2] |= (uint32_t)p[i] << ((i & 3) * 8);
                 raw[r] = make_uint2(w[0], w[1]);
             }
-            sc[r] = s[(int64_t)(row >> 7) * sK + (col >> 7)];
+            sc[r] = s[(int64_t)(row >> bshift) * sK + (col >> bshift)];      // bshift = log2(block size), 7 for 128x128 blocks
         }
     }
 #pragma unroll
@@ -85,27 +85,31 @@ __global__ __launch_bounds__(256) void weight_dequant_kernel(const uint8_t* __re
     }
 }
 
-int launch_weight_dequant(const void* x, const float* s, void* y, int64_t N, int64_t K, int out_dtype,
+// block_size: the edge of the square scale blocks, a power of two from 8 up (128 in the DeepSeek-V3 format; the
+// reference's weight_dequant takes any block_size, offical_kernel.py:46-53)
+int launch_weight_dequant(const void* x, const float* s, void* y, int64_t N, int64_t K, int block_size, int out_dtype,
                           hipStream_t stream) {
     if (N == 0 || K == 0) return 0;
     dim3 grid, block(256);
     if (!grid_rows((K + kWdCols - 1) / kWdCols, (N + kWdRows * kWdWaves - 1) / (kWdRows * kWdWaves), grid)) return kErrTooManyBlocks;
-    const int sK = (int)((K + kGroup - 1) / kGroup);
+    int bshift = 0;
+    while ((1 << bshift) < block_size) ++bshift;
+    const int sK = (int)((K + block_size - 1) / block_size);
     const bool vec = (K % 8 == 0) && ((reinterpret_cast<uintptr_t>(x) & 7) == 0) &&
                      ((reinterpret_cast<uintptr_t>(y) & 15) == 0);
     const uint8_t* xp = static_cast<const uint8_t*>(x);
     if (out_dtype == 0) {
         uint16_t* yp = static_cast<uint16_t*>(y);
         if (vec)
-            hipLaunchKernelGGL((weight_dequant_kernel<uint16_t, true>), grid, block, 0, stream, xp, s, yp, (int)N, (int)K, sK);
+            hipLaunchKernelGGL((weight_dequant_kernel<uint16_t, true>), grid, block, 0, stream, xp, s, yp, (int)N, (int)K, sK, bshift);
         else
-            hipLaunchKernelGGL((weight_dequant_kernel<uint16_t, false>), grid, block, 0, stream, xp, s, yp, (int)N, (int)K, sK);
+            hipLaunchKernelGGL((weight_dequant_kernel<uint16_t, false>), grid, block, 0, stream, xp, s, yp, (int)N, (int)K, sK, bshift);
     } else {
         float* yp = static_cast<float*>(y);
         if (vec)
-            hipLaunchKernelGGL((weight_dequant_kernel<float, true>), grid, block, 0, stream, xp, s, yp, (int)N, (int)K, sK);
+            hipLaunchKernelGGL((weight_dequant_kernel<float, true>), grid, block, 0, stream, xp, s, yp, (int)N, (int)K, sK, bshift);
         else
-            hipLaunchKernelGGL((weight_dequant_kernel<float, false>), grid, block, 0, stream, xp, s, yp, (int)N, (int)K, sK);
+            hipLaunchKernelGGL((weight_dequant_kernel<float, false>), grid, block, 0, stream, xp, s, yp, (int)N, (int)K, sK, bshift);
     }
     return (int)hipGetLastError();
 }

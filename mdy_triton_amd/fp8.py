@@ -75,7 +75,7 @@ def quant_input(x: torch.Tensor, only_forward: bool = True):
     y = torch.empty(PM, PN, device=dev, dtype=FP8)
     s = torch.empty(B, PM, device=dev, dtype=torch.float32)
     with on_device(dev):
-        check(lib().mdy_act_quant_typed(ptr(x), xt, ptr(y), ptr(s), M, K, x.stride(0) if M > 0 else K, PM, PN, 1, PM, 1,
+        check(lib().mdy_act_quant_typed(ptr(x), xt, 128, ptr(y), ptr(s), M, K, x.stride(0) if M > 0 else K, PM, PN, 1, PM, 1,
                                         stream_ptr(dev)), "quant_input")
     return y, s.transpose(0, 1), None, None
 

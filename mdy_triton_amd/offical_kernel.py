@@ -19,16 +19,17 @@ def act_quant(x: torch.Tensor, block_size: int = 128) -> Tuple[torch.Tensor, tor
     """
     assert x.is_contiguous()
     assert x.size(-1) % block_size == 0
-    if block_size != 128:
-        raise ValueError("only block_size=128 is implemented (the reference default)")
-    xt = xt_code(x, "act_quant")      # bf16 runs the tuned kernel; fp16 / fp32 are quantized from their exact fp32 values
+    if block_size < 8 or block_size > 512 or block_size & (block_size - 1):
+        raise ValueError("block_size must be a power of two from 8 to 512 (128 is the tuned case), got %d" % block_size)
+    xt = xt_code(x, "act_quant")      # bf16 with block_size 128 runs the tuned kernel; everything else the general one
     dev = require_gpu(x)
     K = x.size(-1)
     M = x.numel() // K if K else 0
     y = torch.empty_like(x, dtype=FP8)
     s = x.new_empty(*x.size()[:-1], K // block_size, dtype=torch.float32)
     with on_device(dev):
-        check(lib().mdy_act_quant_typed(ptr(x), xt, ptr(y), ptr(s), M, K, K, M, K, K // 128, 1, 0, stream_ptr(dev)), "act_quant")
+        check(lib().mdy_act_quant_typed(ptr(x), xt, block_size, ptr(y), ptr(s), M, K, K, M, K, K // block_size, 1, 0,
+                                        stream_ptr(dev)), "act_quant")
     return y, s
 
 
@@ -41,18 +42,19 @@ def weight_dequant(x: torch.Tensor, s: torch.Tensor, block_size: int = 128,
     """
     assert x.is_contiguous() and s.is_contiguous()
     assert x.dim() == 2 and s.dim() == 2
-    if block_size != 128:
-        raise ValueError("only block_size=128 is implemented (the reference default)")
+    if block_size < 8 or block_size & (block_size - 1):
+        raise ValueError("block_size must be a power of two >= 8, got %d" % block_size)
     if x.dtype != FP8 or s.dtype != torch.float32:
         raise TypeError("weight_dequant expects float8_e4m3fn weights and float32 scales")
     dev = require_gpu(x, s)
     N, K = x.size()
-    if tuple(s.shape) != ((N + 127) // 128, (K + 127) // 128):
+    if tuple(s.shape) != ((N + block_size - 1) // block_size, (K + block_size - 1) // block_size):
         raise ValueError("scale shape %s does not match weight %s" % (tuple(s.shape), tuple(x.shape)))
     dtype = out_dtype or torch.get_default_dtype()
     y = torch.empty_like(x, dtype=dtype)
     with on_device(dev):
-        check(lib().mdy_weight_dequant(ptr(x), ptr(s), ptr(y), N, K, out_code(dtype), stream_ptr(dev)), "weight_dequant")
+        check(lib().mdy_weight_dequant_block(ptr(x), ptr(s), ptr(y), N, K, block_size, out_code(dtype), stream_ptr(dev)),
+              "weight_dequant")
     return y
 
 

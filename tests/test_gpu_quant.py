@@ -443,3 +443,30 @@ def test_act_quant_and_quant_input_fp16_fp32_inputs(dtype, M, K):
     assert torch.equal(q2.cpu().view(torch.uint8), rq2.view(torch.uint8)) and torch.equal(qs2.cpu().contiguous(), rqs2.contiguous())
     with pytest.raises(TypeError):
         m.act_quant(torch.zeros(4, 128, device=DEV, dtype=torch.float64))
+
+
+@pytest.mark.parametrize("bs", [8, 32, 64, 256, 512])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_act_quant_and_weight_dequant_other_block_sizes(bs, dtype):
+    """act_quant(x, block_size) and weight_dequant(x, s, block_size) take any block size in the reference
+    (offical_kernel.py:21-27, 46-53); here every power of two from 8 (to 512 for the quantizer): bit-exact
+    against the oracle, including a ragged weight whose edge blocks are partial."""
+    g = torch.Generator().manual_seed(bs)
+    M, K = 37, 1024
+    x = (torch.randn(M, K, generator=g) * torch.rand(M, 1, generator=g) * 4).to(dtype)
+    y_ref, s_ref = O.act_quant(x, bs)
+    y, s = m.act_quant(x.to(DEV), bs)
+    assert s.shape == (M, K // bs)
+    assert torch.equal(y.cpu().view(torch.uint8), y_ref.view(torch.uint8)) and torch.equal(s.cpu(), s_ref)
+    N2, K2 = 300, 776
+    wq = torch.randint(0, 0x7F, (N2, K2), generator=g, dtype=torch.uint8).view(FP8)
+    ws = torch.rand((N2 + bs - 1) // bs, (K2 + bs - 1) // bs, generator=g) + 0.25
+    for od in (torch.bfloat16, torch.float32):
+        got = m.weight_dequant(wq.to(DEV), ws.to(DEV), bs, out_dtype=od)
+        ref = O.weight_dequant(wq, ws, bs, dtype=od)
+        assert torch.equal(got.cpu().view(torch.int16 if od == torch.bfloat16 else torch.int32),
+                           ref.view(torch.int16 if od == torch.bfloat16 else torch.int32))
+    with pytest.raises(ValueError):
+        m.act_quant(x.to(DEV)[:, :960].contiguous(), 96)
+    with pytest.raises(ValueError):
+        m.weight_dequant(wq.to(DEV), ws.to(DEV), 100)
