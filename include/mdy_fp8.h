@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define MDY_FP8_ABI_VERSION 10
+#define MDY_FP8_ABI_VERSION 12
 
 /* error codes (negative = argument rejected before any launch) */
 #define MDY_OK 0
@@ -97,6 +97,10 @@ int mdy_act_quant_typed(const void* x, int x_dtype, int block_size, void* y, flo
 int mdy_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t, int64_t N, int64_t K,
                      int64_t w_row_stride, int64_t w_col_stride, int64_t PN, int64_t PK, int mode,
                      void* stream);
+/* The same for a weight of type w_dtype (MDY_XT_BF16 / MDY_XT_F16 / MDY_XT_F32; strides in its elements): the reference
+ * kernels load with .to(tl.float32) (fp8.py:193), so an fp32 master weight is quantized from its exact values. */
+int mdy_weight_quant_typed(const void* w, int w_dtype, void* y, float* s, void* y_t, float* s_t, int64_t N, int64_t K,
+                           int64_t w_row_stride, int64_t w_col_stride, int64_t PN, int64_t PK, int mode, void* stream);
 
 /* Training-time quantizer: row-wise 1x128 quantization of x AND the quantized transpose,
  * one read of x.  DeepLinear dialect only (clamp 1e4 + eps 1e-8, saturating cast).
@@ -120,13 +124,17 @@ int mdy_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t, in
 int mdy_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
                         int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int64_t s_kb_stride,
                         int t_mode, void* stream);
+/* The same for an input of type x_dtype (MDY_XT_BF16 / MDY_XT_F16 / MDY_XT_F32; strides in its elements). */
+int mdy_quant_transpose_typed(const void* x, int x_dtype, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
+                        int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int64_t s_kb_stride,
+                        int t_mode, void* stream);
 
 /* Official-dialect training quantizer (s = amax / 448, no clamp, no eps): the row-wise 1x128 quantization of x and
  * the quantized transpose with one scale per column and 128 rows, one read of x.  Replaces the pair
  * act_quant_block(x) / act_quant_block(x, transpose=True) (triton_kernels/deepseekv3/fp8_kernel.py:62-87, kernel
  * :14-60) that the reference's Fp8Linear runs on x and on dy (:286-301).
  *
- *   x    bf16 [M, K], element (m, k) at x[m * x_row_stride + k * x_col_stride]
+ *   x    [M, K] of x_dtype (MDY_XT_BF16 / MDY_XT_F16 / MDY_XT_F32), element (m, k) at x[m * x_row_stride + k * x_col_stride]
  *   y    e4m3fn [PM, PK] row-major or NULL (then s must be NULL too: only the transposed copy is produced)
  *   s    fp32 [PM, PK/128] row-major
  *   y_t  e4m3fn [PK, PM] row-major: y_t[k, m] = x[m, k] / s_t[k, m / 128]
@@ -134,7 +142,7 @@ int mdy_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t,
  * PM >= M and PK >= K are multiples of 128; padding reads as 0 (an all-zero group has scale 0 and NaN bytes, as in the
  * reference).  y / y_t 8-byte aligned.
  */
-int mdy_act_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
+int mdy_act_quant_transpose(const void* x, int x_dtype, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
                             int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, void* stream);
 
 /* Block-scaled FP8 GEMM, NT layout, with 1x128 scales on both operands:
@@ -315,6 +323,9 @@ int mdy_group_pad_rows(const void* x, void* y, const int64_t* m_splits, int64_t 
 /* In-place x[m, :] = bf16(fp32(x[m, :]) + fp32(b)) on bf16 x [M, N] row-major, bf16 b [N].
  * Replaces add_bias (fp8.py:297-305, kernel :283-295). */
 int mdy_add_bias(void* x, const void* b, int64_t M, int64_t N, void* stream);
+/* The same with a bias of type b_dtype (MDY_XT_BF16 / MDY_XT_F16 / MDY_XT_F32): the reference loads the bias with
+ * .to(tl.float32) (fp8.py:291), so an fp32 bias is added at full precision. */
+int mdy_add_bias_typed(void* x, const void* b, int b_dtype, int64_t M, int64_t N, void* stream);
 
 /* In-place gradient accumulation over n elements: x[i] = T(fp32(x[i]) + fp32(y[i])), x of x_dtype, y of y_dtype
  * (MDY_DT_BF16 / MDY_DT_F32 each).  Replaces add_grad (triton_kernels/megatron_patchs/add_kernel.py:55-62, kernel

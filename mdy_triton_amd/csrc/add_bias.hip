@@ -8,19 +8,26 @@
 
 namespace mdy {
 
-template <bool VEC>
-__global__ __launch_bounds__(256) void add_bias_kernel(uint16_t* __restrict__ x, const uint16_t* __restrict__ b, int M,
+// BT: type of the bias (0 bf16, 1 fp16, 2 fp32; the reference loads it with .to(tl.float32), fp8.py:291); VEC: whole
+// 16-byte pieces of x, and of a bf16 bias.
+template <bool VEC, int BT>
+__global__ __launch_bounds__(256) void add_bias_kernel(uint16_t* __restrict__ x, const void* __restrict__ bv, int M,
                                                         int N) {
     const int col = (blockIdx.x * 256 + threadIdx.x) * 8;
     if (col >= N) return;
     float bias[8];
-    if (VEC) {
-        const uint4 v = *reinterpret_cast<const uint4*>(b + col);
+    if (VEC && BT == 0) {
+        const uint4 v = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(bv) + col);
         bias[0] = bf16_lo(v.x); bias[1] = bf16_hi(v.x); bias[2] = bf16_lo(v.y); bias[3] = bf16_hi(v.y);
         bias[4] = bf16_lo(v.z); bias[5] = bf16_hi(v.z); bias[6] = bf16_lo(v.w); bias[7] = bf16_hi(v.w);
     } else {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) bias[i] = (col + i < N) ? bf16_one(b[col + i]) : 0.0f;
+        for (int i = 0; i < 8; ++i) {
+            bias[i] = 0.0f;
+            if (col + i < N)
+                bias[i] = BT == 0 ? bf16_one(static_cast<const uint16_t*>(bv)[col + i])
+                        : BT == 1 ? (float)static_cast<const _Float16*>(bv)[col + i] : static_cast<const float*>(bv)[col + i];
+        }
     }
     for (int row = blockIdx.y; row < M; row += gridDim.y) {
         uint16_t* p = x + (int64_t)row * N + col;
@@ -39,18 +46,18 @@ __global__ __launch_bounds__(256) void add_bias_kernel(uint16_t* __restrict__ x,
     }
 }
 
-int launch_add_bias(void* x, const void* b, int64_t M, int64_t N, hipStream_t stream) {
+int launch_add_bias(void* x, const void* b, int b_dtype, int64_t M, int64_t N, hipStream_t stream) {
     if (M == 0 || N == 0) return 0;
     const unsigned gy = (unsigned)(M < 4096 ? M : 4096);
     dim3 grid((unsigned)((N + 2047) / 2048), gy);
     const bool vec = (N % 8 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0) &&
                      ((reinterpret_cast<uintptr_t>(b) & 15) == 0);
-    if (vec)
-        hipLaunchKernelGGL(add_bias_kernel<true>, grid, dim3(256), 0, stream, static_cast<uint16_t*>(x),
-                           static_cast<const uint16_t*>(b), (int)M, (int)N);
-    else
-        hipLaunchKernelGGL(add_bias_kernel<false>, grid, dim3(256), 0, stream, static_cast<uint16_t*>(x),
-                           static_cast<const uint16_t*>(b), (int)M, (int)N);
+    uint16_t* xp = static_cast<uint16_t*>(x);
+#define MDY_AB(VEC, BT) hipLaunchKernelGGL((add_bias_kernel<VEC, BT>), grid, dim3(256), 0, stream, xp, b, (int)M, (int)N)
+    if (b_dtype == 0) { if (vec) MDY_AB(true, 0); else MDY_AB(false, 0); }
+    else if (b_dtype == 1) { if (vec) MDY_AB(true, 1); else MDY_AB(false, 1); }
+    else { if (vec) MDY_AB(true, 2); else MDY_AB(false, 2); }
+#undef MDY_AB
     return (int)hipGetLastError();
 }
 

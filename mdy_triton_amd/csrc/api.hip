@@ -97,8 +97,9 @@ int mdy_act_quant_typed(const void* x, int x_dtype, int block_size, void* y, flo
                     "act_quant_typed");
 }
 
-int mdy_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t, int64_t N, int64_t K,
-                     int64_t w_row_stride, int64_t w_col_stride, int64_t PN, int64_t PK, int mode, void* stream) {
+int mdy_weight_quant_typed(const void* w, int w_dtype, void* y, float* s, void* y_t, float* s_t, int64_t N, int64_t K,
+                           int64_t w_row_stride, int64_t w_col_stride, int64_t PN, int64_t PK, int mode, void* stream) {
+    if (w_dtype != MDY_XT_BF16 && w_dtype != MDY_XT_F16 && w_dtype != MDY_XT_F32) return fail(MDY_E_DTYPE, "weight_quant: unknown w_dtype %d", w_dtype);
     if (mode != MDY_QUANT_OFFICIAL && mode != MDY_QUANT_DEEPLINEAR) return fail(MDY_E_DTYPE, "weight_quant: unknown mode %d", mode);
     if (N < 0 || K < 0 || PN < N || PK < K || PN > kMaxDim || PK > kMaxDim)
         return fail(MDY_E_SHAPE, "weight_quant: need 0 <= N <= PN, 0 <= K <= PK");
@@ -108,14 +109,20 @@ int mdy_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t, in
     if (!y || !s || (!w && N > 0 && K > 0)) return fail(MDY_E_NULL, "weight_quant: null pointer");
     if (!aligned(y, 8) || (y_t && !aligned(y_t, 8))) return fail(MDY_E_ALIGN, "weight_quant: y / y_t must be 8-byte aligned");
     if (int e = check_device()) return e;
-    return launched(mdy::launch_weight_quant(w, y, s, y_t, s_t, N, K, w_row_stride, w_col_stride, PN, PK, mode,
+    return launched(mdy::launch_weight_quant(w, w_dtype, y, s, y_t, s_t, N, K, w_row_stride, w_col_stride, PN, PK, mode,
                                              static_cast<hipStream_t>(stream)),
                     "weight_quant");
 }
 
-int mdy_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
-                        int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int64_t s_kb_stride, int t_mode,
-                        void* stream) {
+int mdy_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t, int64_t N, int64_t K,
+                     int64_t w_row_stride, int64_t w_col_stride, int64_t PN, int64_t PK, int mode, void* stream) {
+    return mdy_weight_quant_typed(w, MDY_XT_BF16, y, s, y_t, s_t, N, K, w_row_stride, w_col_stride, PN, PK, mode, stream);
+}
+
+int mdy_quant_transpose_typed(const void* x, int x_dtype, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
+                              int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int64_t s_kb_stride, int t_mode,
+                              void* stream) {
+    if (x_dtype != MDY_XT_BF16 && x_dtype != MDY_XT_F16 && x_dtype != MDY_XT_F32) return fail(MDY_E_DTYPE, "quant_transpose: unknown x_dtype %d", x_dtype);
     if (t_mode != MDY_T_COLUMN && t_mode != MDY_T_BLOCK) return fail(MDY_E_DTYPE, "quant_transpose: unknown t_mode %d", t_mode);
     if (M < 0 || K < 0 || PM < M || PK < K || PM > kMaxDim || PK > kMaxDim)
         return fail(MDY_E_SHAPE, "quant_transpose: need 0 <= M <= PM, 0 <= K <= PK");
@@ -124,15 +131,23 @@ int mdy_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t,
     if (PM == 0 || PK == 0) return 0;
     if (!y || !s || !y_t || !s_t || (!x && M > 0 && K > 0)) return fail(MDY_E_NULL, "quant_transpose: null pointer");
     if (!aligned(y, 8) || !aligned(y_t, 8)) return fail(MDY_E_ALIGN, "quant_transpose: y / y_t must be 8-byte aligned");
-    if (!aligned(x, 2) || !aligned(s, 4) || !aligned(s_t, 4)) return fail(MDY_E_ALIGN, "quant_transpose: x/s/s_t misaligned for their element type");
+    if (!aligned(x, x_dtype == MDY_XT_F32 ? 4 : 2) || !aligned(s, 4) || !aligned(s_t, 4)) return fail(MDY_E_ALIGN, "quant_transpose: x/s/s_t misaligned for their element type");
     if (int e = check_device()) return e;
-    return launched(mdy::launch_quant_transpose(x, y, s, y_t, s_t, M, K, x_row_stride, x_col_stride, PM, PK, s_kb_stride, t_mode,
-                                                static_cast<hipStream_t>(stream)),
+    return launched(mdy::launch_quant_transpose(x, x_dtype, y, s, y_t, s_t, M, K, x_row_stride, x_col_stride, PM, PK, s_kb_stride,
+                                                t_mode, static_cast<hipStream_t>(stream)),
                     "quant_transpose");
 }
 
-int mdy_act_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
+int mdy_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
+                        int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int64_t s_kb_stride, int t_mode,
+                        void* stream) {
+    return mdy_quant_transpose_typed(x, MDY_XT_BF16, y, s, y_t, s_t, M, K, x_row_stride, x_col_stride, PM, PK, s_kb_stride, t_mode,
+                                     stream);
+}
+
+int mdy_act_quant_transpose(const void* x, int x_dtype, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
                             int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, void* stream) {
+    if (x_dtype != MDY_XT_BF16 && x_dtype != MDY_XT_F16 && x_dtype != MDY_XT_F32) return fail(MDY_E_DTYPE, "act_quant_transpose: unknown x_dtype %d", x_dtype);
     if (M < 0 || K < 0 || PM < M || PK < K || PM > kMaxDim || PK > kMaxDim)
         return fail(MDY_E_SHAPE, "act_quant_transpose: need 0 <= M <= PM, 0 <= K <= PK");
     if (PM % 128 != 0 || PK % 128 != 0) return fail(MDY_E_SHAPE, "act_quant_transpose: PM=%lld, PK=%lld must be multiples of 128", (long long)PM, (long long)PK);
@@ -140,9 +155,9 @@ int mdy_act_quant_transpose(const void* x, void* y, float* s, void* y_t, float* 
     if (PM == 0 || PK == 0) return 0;
     if (!y_t || !s_t || (!x && M > 0 && K > 0)) return fail(MDY_E_NULL, "act_quant_transpose: null pointer");
     if ((y && !aligned(y, 8)) || !aligned(y_t, 8)) return fail(MDY_E_ALIGN, "act_quant_transpose: y / y_t must be 8-byte aligned");
-    if (!aligned(x, 2) || (s && !aligned(s, 4)) || !aligned(s_t, 4)) return fail(MDY_E_ALIGN, "act_quant_transpose: x/s/s_t misaligned for their element type");
+    if (!aligned(x, x_dtype == MDY_XT_F32 ? 4 : 2) || (s && !aligned(s, 4)) || !aligned(s_t, 4)) return fail(MDY_E_ALIGN, "act_quant_transpose: x/s/s_t misaligned for their element type");
     if (int e = check_device()) return e;
-    return launched(mdy::launch_act_quant_transpose(x, y, s, y_t, s_t, M, K, x_row_stride, x_col_stride, PM, PK,
+    return launched(mdy::launch_act_quant_transpose(x, x_dtype, y, s, y_t, s_t, M, K, x_row_stride, x_col_stride, PM, PK,
                                                     static_cast<hipStream_t>(stream)),
                     "act_quant_transpose");
 }
@@ -353,13 +368,18 @@ int mdy_group_pad_rows(const void* x, void* y, const int64_t* m_splits, int64_t 
                     "group_pad_rows");
 }
 
-int mdy_add_bias(void* x, const void* b, int64_t M, int64_t N, void* stream) {
+int mdy_add_bias_typed(void* x, const void* b, int b_dtype, int64_t M, int64_t N, void* stream) {
+    if (b_dtype != MDY_XT_BF16 && b_dtype != MDY_XT_F16 && b_dtype != MDY_XT_F32) return fail(MDY_E_DTYPE, "add_bias: unknown b_dtype %d", b_dtype);
     if (M < 0 || N < 0 || M > kMaxDim || N > kMaxDim) return fail(MDY_E_SHAPE, "add_bias: bad shape");
     if (M == 0 || N == 0) return 0;
     if (!x || !b) return fail(MDY_E_NULL, "add_bias: null pointer");
-    if (!aligned(x, 2) || !aligned(b, 2)) return fail(MDY_E_ALIGN, "add_bias: misaligned pointer");
+    if (!aligned(x, 2) || !aligned(b, b_dtype == MDY_XT_F32 ? 4 : 2)) return fail(MDY_E_ALIGN, "add_bias: misaligned pointer");
     if (int e = check_device()) return e;
-    return launched(mdy::launch_add_bias(x, b, M, N, static_cast<hipStream_t>(stream)), "add_bias");
+    return launched(mdy::launch_add_bias(x, b, b_dtype, M, N, static_cast<hipStream_t>(stream)), "add_bias");
+}
+
+int mdy_add_bias(void* x, const void* b, int64_t M, int64_t N, void* stream) {
+    return mdy_add_bias_typed(x, b, MDY_XT_BF16, M, N, stream);
 }
 
 int mdy_add_grad(void* x, const void* y, int64_t n, int x_dtype, int y_dtype, void* stream) {

@@ -158,6 +158,60 @@ __device__ __forceinline__ void store_nt8(void* p, const uint2& v) {
     __builtin_nontemporal_store(u, static_cast<uintx2_t*>(p));
 }
 
+// 8 values of row `row`, columns c0 .. c0+7, of an [N, K] matrix of type XT (0 bf16, 1 fp16, 2 fp32; element (n, k) at
+// base[n * rs + k * cs]) as fp32, zeros outside the matrix.  VEC: cs == 1, all 8 columns in range, 16-byte aligned rows.
+// The reference kernels load with .to(tl.float32): every input type is quantized from its exact fp32 value.
+template <int XT, bool VEC>
+__device__ __forceinline__ void load_row8_f32(const void* __restrict__ base, int row, int c0, int N, int K, int64_t rs, int64_t cs,
+                                              float (&f)[8]) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) f[j] = 0.0f;
+    if (row >= N || c0 >= K) return;
+    if (XT == 0) {
+        const uint16_t* p = static_cast<const uint16_t*>(base) + (int64_t)row * rs;
+        if (VEC) {
+            const uint4 v = load_nt16(p + c0);
+            f[0] = bf16_lo(v.x); f[1] = bf16_hi(v.x); f[2] = bf16_lo(v.y); f[3] = bf16_hi(v.y);
+            f[4] = bf16_lo(v.z); f[5] = bf16_hi(v.z); f[6] = bf16_lo(v.w); f[7] = bf16_hi(v.w);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (c0 + j < K) f[j] = bf16_one(p[(int64_t)(c0 + j) * cs]);
+        }
+    } else if (XT == 1) {
+        const _Float16* p = static_cast<const _Float16*>(base) + (int64_t)row * rs;
+        if (VEC) {
+            const uint4 v = load_nt16(p + c0);
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                f[2 * j] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[j] & 0xFFFFu));
+                f[2 * j + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[j] >> 16));
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (c0 + j < K) f[j] = (float)p[(int64_t)(c0 + j) * cs];
+        }
+    } else {
+        const float* p = static_cast<const float*>(base) + (int64_t)row * rs;
+        if (VEC) {
+            const uint4 a = load_nt16(p + c0), b = load_nt16(p + c0 + 4);
+            f[0] = __uint_as_float(a.x); f[1] = __uint_as_float(a.y); f[2] = __uint_as_float(a.z); f[3] = __uint_as_float(a.w);
+            f[4] = __uint_as_float(b.x); f[5] = __uint_as_float(b.y); f[6] = __uint_as_float(b.z); f[7] = __uint_as_float(b.w);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (c0 + j < K) f[j] = p[(int64_t)(c0 + j) * cs];
+        }
+    }
+}
+// true when the vector form of load_row8_f32 applies to a matrix of element size esz
+inline bool rows_vectorizable(const void* base, int64_t K, int64_t rs, int64_t cs, int esz) {
+    return cs == 1 && K % 8 == 0 && (rs * esz) % 16 == 0 && (reinterpret_cast<uintptr_t>(base) & 15) == 0;
+}
+inline int xt_size(int xt) { return xt == 2 ? 4 : 2; }
+
 __device__ __forceinline__ uint32_t pack2_bf16(float a, float b) {
     floatx2 f = {a, b};
     bf16x2 h = __builtin_convertvector(f, bf16x2);
@@ -187,13 +241,13 @@ int launch_act_quant(const void* x, void* y, float* s, int64_t M, int64_t K, int
 int launch_act_quant_typed(const void* x, int x_dtype, int block_size, void* y, float* s, int64_t M, int64_t K,
                            int64_t x_row_stride, int64_t PM, int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode,
                            hipStream_t stream);
-int launch_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t, int64_t N, int64_t K,
+int launch_weight_quant(const void* w, int w_dtype, void* y, float* s, void* y_t, float* s_t, int64_t N, int64_t K,
                         int64_t w_row_stride, int64_t w_col_stride, int64_t PN, int64_t PK, int mode,
                         hipStream_t stream);
-int launch_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
+int launch_quant_transpose(const void* x, int x_dtype, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
                            int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int64_t s_kb_stride,
                            int t_mode, hipStream_t stream);
-int launch_act_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
+int launch_act_quant_transpose(const void* x, int x_dtype, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
                                int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, hipStream_t stream);
 int launch_fp8_gemm_nt_rowscaled(const void* a, const float* a_s, int64_t as_rs, int64_t as_cs, const void* b,
                                  const float* b_s, int64_t bs_rs, int64_t bs_cs, void* c, int64_t M, int64_t N, int64_t K,
@@ -228,7 +282,7 @@ int launch_fp8_grouped_gemm_nt(const void* a, const float* a_s, int64_t as_row_s
 int launch_group_pad(const void* x, void* y, const int64_t* m_splits, int64_t G, int64_t row_bytes, int64_t multiple,
                      int unpad, hipStream_t stream);
 int launch_add_grad(void* x, const void* y, int64_t n, int x_dtype, int y_dtype, hipStream_t stream);
-int launch_add_bias(void* x, const void* b, int64_t M, int64_t N, hipStream_t stream);
+int launch_add_bias(void* x, const void* b, int b_dtype, int64_t M, int64_t N, hipStream_t stream);
 int launch_cast_f32_to_e4m3(const float* x, void* y, int64_t n, int saturate, hipStream_t stream);
 int launch_quotient_selfcheck(uint64_t* out, int amax_lo, int amax_hi, int mode, hipStream_t stream);
 

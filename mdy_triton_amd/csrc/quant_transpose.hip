@@ -35,8 +35,9 @@ __device__ __forceinline__ float qt_quot(float x, float s, float r) {
 // Scale layouts: row scale of row m, K group kb at s[kb * s_kb_stride + m * s_m_stride]; column-group scale of
 // column k, row group a at s_t[a * st_a_stride + k * st_k_stride] (TMODE 0) / block scale at s_t[kb * (PM/128) + a]
 // (TMODE 1).  y may be null (MODE 0 callers that only want the transposed copy): the row-wise outputs are skipped.
-template <int MODE, int TMODE, bool VEC, int RPT>
-__global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ y,
+// XT: input type (0 bf16, 1 fp16, 2 fp32); the reciprocal quotient is proven for bf16 inputs only, other types divide.
+template <int MODE, int TMODE, bool VEC, int RPT, int XT>
+__global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const void* __restrict__ x, uint8_t* __restrict__ y,
                                                                float* __restrict__ s, uint8_t* __restrict__ y_t,
                                                                float* __restrict__ s_t, int M, int K,
                                                                int64_t x_row_stride, int64_t x_col_stride, int PM,
@@ -67,25 +68,10 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
     for (int j = 0; j < 8; ++j) cmax[j] = 0.0f;
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
-        const int row = bm * 128 + rg * RPT + i;
-        uint32_t wd[4] = {0u, 0u, 0u, 0u};
-        if (row < M && c0 < K) {
-            if (VEC) {
-                const uint4 v = load_nt16(x + (int64_t)row * x_row_stride + c0);
-                wd[0] = v.x; wd[1] = v.y; wd[2] = v.z; wd[3] = v.w;
-            } else {
-#pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    if (c0 + j < K)
-                        wd[j >> 1] |= (uint32_t)x[(int64_t)row * x_row_stride + (int64_t)(c0 + j) * x_col_stride]
-                                      << ((j & 1) * 16);
-            }
-        }
+        load_row8_f32<XT, VEC>(x, bm * 128 + rg * RPT + i, c0, M, K, x_row_stride, x_col_stride, f[i]);
         float m = 0.0f;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            f[i][2 * j] = bf16_lo(wd[j]);
-            f[i][2 * j + 1] = bf16_hi(wd[j]);
             m = fmaxf(fmaxf(fabsf(f[i][2 * j]), fabsf(f[i][2 * j + 1])), m);
             cmax[2 * j] = fmaxf(cmax[2 * j], fabsf(f[i][2 * j]));
             cmax[2 * j + 1] = fmaxf(cmax[2 * j + 1], fabsf(f[i][2 * j + 1]));
@@ -100,7 +86,7 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
         const float sc = group_scale<MODE>(rmax[i]);
         const float r = 1.0f / sc;
         float q[8];
-        if (group_is_fast<MODE>(rmax[i])) {
+        if (XT == 0 && group_is_fast<MODE>(rmax[i])) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) q[j] = qt_quot<MODE, true>(f[i][j], sc, r);
         } else {
@@ -162,7 +148,7 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
             tr[j] = brc;
         }
     }
-    bool tfast = true;
+    bool tfast = XT == 0;
 #pragma unroll
     for (int j = 0; j < 8; ++j) tfast = tfast && group_is_fast<MODE>(tamax[j]);
     uint32_t qlo[RPT], qhi[RPT];   // row i of the transposed copy's bytes: columns 0..3 | 4..7
@@ -214,7 +200,7 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const uint1
 
 // Shared launcher.  mode: dialect (0 official, column groups only; 1 DeepLinear); t_mode: 0 per column group, 1 per
 // 128x128 block.
-static int launch_qt(int mode, const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
+static int launch_qt(int mode, const void* x, int x_dtype, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
                      int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int64_t s_kb_stride,
                      int64_t s_m_stride, int64_t st_a_stride, int64_t st_k_stride, int t_mode, hipStream_t stream) {
     if (PM == 0 || PK == 0) return 0;
@@ -223,44 +209,42 @@ static int launch_qt(int mode, const void* x, void* y, float* s, void* y_t, floa
     // 512 threads (4 rows each) when there are few tiles per CU: more waves to hide the load and store latency
     const bool wide = (PK / 128) * (PM / 128) < 256 * 24;
     dim3 block(wide ? 512 : 256);
-    const bool vec = (x_col_stride == 1) && (K % 8 == 0) && (x_row_stride % 8 == 0) &&
-                     ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
-    const uint16_t* xp = static_cast<const uint16_t*>(x);
+    const bool vec = rows_vectorizable(x, K, x_row_stride, x_col_stride, xt_size(x_dtype));
     uint8_t* yp = static_cast<uint8_t*>(y);
     uint8_t* ytp = static_cast<uint8_t*>(y_t);
-#define MDY_QT(MODE, TM, VEC)                                                                                           \
-    do {                                                                                                                \
-        if (wide)                                                                                                       \
-            hipLaunchKernelGGL((quant_transpose_kernel<MODE, TM, VEC, 4>), grid, block, 0, stream, xp, yp, s, ytp, s_t, \
-                               (int)M, (int)K, x_row_stride, x_col_stride, (int)PM, (int)PK, s_kb_stride, s_m_stride,   \
-                               st_a_stride, st_k_stride);                                                               \
-        else                                                                                                            \
-            hipLaunchKernelGGL((quant_transpose_kernel<MODE, TM, VEC, 8>), grid, block, 0, stream, xp, yp, s, ytp, s_t, \
-                               (int)M, (int)K, x_row_stride, x_col_stride, (int)PM, (int)PK, s_kb_stride, s_m_stride,   \
-                               st_a_stride, st_k_stride);                                                               \
+#define MDY_QT(MODE, TM, VEC, XT)                                                                                         \
+    do {                                                                                                                  \
+        if (wide)                                                                                                         \
+            hipLaunchKernelGGL((quant_transpose_kernel<MODE, TM, VEC, 4, XT>), grid, block, 0, stream, x, yp, s, ytp, s_t, \
+                               (int)M, (int)K, x_row_stride, x_col_stride, (int)PM, (int)PK, s_kb_stride, s_m_stride,     \
+                               st_a_stride, st_k_stride);                                                                 \
+        else                                                                                                              \
+            hipLaunchKernelGGL((quant_transpose_kernel<MODE, TM, VEC, 8, XT>), grid, block, 0, stream, x, yp, s, ytp, s_t, \
+                               (int)M, (int)K, x_row_stride, x_col_stride, (int)PM, (int)PK, s_kb_stride, s_m_stride,     \
+                               st_a_stride, st_k_stride);                                                                 \
     } while (0)
-    if (mode == 0) {
-        if (vec) MDY_QT(0, 0, true); else MDY_QT(0, 0, false);
-    } else if (t_mode == 0) {
-        if (vec) MDY_QT(1, 0, true); else MDY_QT(1, 0, false);
-    } else {
-        if (vec) MDY_QT(1, 1, true); else MDY_QT(1, 1, false);
-    }
+#define MDY_QT_V(MODE, TM, XT) do { if (vec) MDY_QT(MODE, TM, true, XT); else MDY_QT(MODE, TM, false, XT); } while (0)
+#define MDY_QT_X(MODE, TM) do { if (x_dtype == 0) MDY_QT_V(MODE, TM, 0); else if (x_dtype == 1) MDY_QT_V(MODE, TM, 1); else MDY_QT_V(MODE, TM, 2); } while (0)
+    if (mode == 0) MDY_QT_X(0, 0);
+    else if (t_mode == 0) MDY_QT_X(1, 0);
+    else MDY_QT_X(1, 1);
+#undef MDY_QT_X
+#undef MDY_QT_V
 #undef MDY_QT
     return (int)hipGetLastError();
 }
 
-int launch_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
+int launch_quant_transpose(const void* x, int x_dtype, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
                            int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int64_t s_kb_stride,
                            int t_mode, hipStream_t stream) {
     // DeepLinear layouts: row scales [PK/128][s_kb_stride >= PM], column-group scales [PM/128][PK]
-    return launch_qt(1, x, y, s, y_t, s_t, M, K, x_row_stride, x_col_stride, PM, PK, s_kb_stride, 1, PK, 1, t_mode, stream);
+    return launch_qt(1, x, x_dtype, y, s, y_t, s_t, M, K, x_row_stride, x_col_stride, PM, PK, s_kb_stride, 1, PK, 1, t_mode, stream);
 }
 
-int launch_act_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
+int launch_act_quant_transpose(const void* x, int x_dtype, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
                                int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, hipStream_t stream) {
     // official layouts, both row-major: s [PM][PK/128], s_t [PK][PM/128]
-    return launch_qt(0, x, y, s, y_t, s_t, M, K, x_row_stride, x_col_stride, PM, PK, 1, PK / 128, 1, PM / 128, 0, stream);
+    return launch_qt(0, x, x_dtype, y, s, y_t, s_t, M, K, x_row_stride, x_col_stride, PM, PK, 1, PK / 128, 1, PM / 128, 0, stream);
 }
 
 }  // namespace mdy

@@ -19,8 +19,9 @@
 
 namespace mdy {
 
-template <int MODE, bool VEC>
-__global__ __launch_bounds__(512) void weight_quant_kernel(const uint16_t* __restrict__ w, uint8_t* __restrict__ y,
+// XT: input type (0 bf16, 1 fp16, 2 fp32); the reciprocal quotient is proven for bf16 inputs, other types divide.
+template <int MODE, bool VEC, int XT>
+__global__ __launch_bounds__(512) void weight_quant_kernel(const void* __restrict__ w, uint8_t* __restrict__ y,
                                                             float* __restrict__ s, uint8_t* __restrict__ y_t,
                                                             float* __restrict__ s_t, int N, int K, int64_t w_row_stride,
                                                             int64_t w_col_stride, int PN, int PK) {
@@ -43,26 +44,9 @@ __global__ __launch_bounds__(512) void weight_quant_kernel(const uint16_t* __res
     float m = 0.0f;
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
-        const int row = rbase + i;
-        uint32_t wd[4] = {0u, 0u, 0u, 0u};
-        if (row < N && c0 < K) {
-            if (VEC) {
-                const uint4 v = load_nt16(w + (int64_t)row * w_row_stride + c0);
-                wd[0] = v.x; wd[1] = v.y; wd[2] = v.z; wd[3] = v.w;
-            } else {
+        load_row8_f32<XT, VEC>(w, rbase + i, c0, N, K, w_row_stride, w_col_stride, f[i]);
 #pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    if (c0 + j < K)
-                        wd[j >> 1] |= (uint32_t)w[(int64_t)row * w_row_stride + (int64_t)(c0 + j) * w_col_stride]
-                                      << ((j & 1) * 16);
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            f[i][2 * j] = bf16_lo(wd[j]);
-            f[i][2 * j + 1] = bf16_hi(wd[j]);
-            m = fmaxf(fmaxf(fabsf(f[i][2 * j]), fabsf(f[i][2 * j + 1])), m);
-        }
+        for (int j = 0; j < 4; ++j) m = fmaxf(fmaxf(fabsf(f[i][2 * j]), fabsf(f[i][2 * j + 1])), m);
     }
     // wave-wide max, then across the waves
 #pragma unroll
@@ -74,7 +58,7 @@ __global__ __launch_bounds__(512) void weight_quant_kernel(const uint16_t* __res
     for (int w = 1; w < WAVES; ++w) amax = fmaxf(amax, wave_max[w]);
 
     const float sc = group_scale<MODE>(amax);
-    const bool fast = group_is_fast<MODE>(amax);
+    const bool fast = XT == 0 && group_is_fast<MODE>(amax);
     const float r = 1.0f / sc;
     if (t == 0) {
         s[(int64_t)bn * (PK >> 7) + bk] = sc;
@@ -112,7 +96,7 @@ __global__ __launch_bounds__(512) void weight_quant_kernel(const uint16_t* __res
     }
 }
 
-int launch_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t, int64_t N, int64_t K,
+int launch_weight_quant(const void* w, int w_dtype, void* y, float* s, void* y_t, float* s_t, int64_t N, int64_t K,
                         int64_t w_row_stride, int64_t w_col_stride, int64_t PN, int64_t PK, int mode,
                         hipStream_t stream) {
     if (PN == 0 || PK == 0) return 0;
@@ -121,19 +105,17 @@ int launch_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t,
     // 512 threads per tile: 4 rows per thread, 56 VGPRs, 8 waves per SIMD (256 threads with 8 rows each need 89
     // VGPRs and measured 1-5 % slower at every size tried)
     dim3 block(512);
-    const bool vec = (w_col_stride == 1) && (K % 8 == 0) && (w_row_stride % 8 == 0) &&
-                     ((reinterpret_cast<uintptr_t>(w) & 15) == 0);
-    const uint16_t* wp = static_cast<const uint16_t*>(w);
+    const bool vec = rows_vectorizable(w, K, w_row_stride, w_col_stride, xt_size(w_dtype));
     uint8_t* yp = static_cast<uint8_t*>(y);
     uint8_t* ytp = static_cast<uint8_t*>(y_t);
-#define MDY_WQ(MODE, VEC)                                                                                          \
-    hipLaunchKernelGGL((weight_quant_kernel<MODE, VEC>), grid, block, 0, stream, wp, yp, s, ytp, s_t, (int)N, \
+#define MDY_WQ(MODE, VEC, XT)                                                                                      \
+    hipLaunchKernelGGL((weight_quant_kernel<MODE, VEC, XT>), grid, block, 0, stream, w, yp, s, ytp, s_t, (int)N, \
                        (int)K, w_row_stride, w_col_stride, (int)PN, (int)PK)
-    if (mode == 0) {
-        if (vec) MDY_WQ(0, true); else MDY_WQ(0, false);
-    } else {
-        if (vec) MDY_WQ(1, true); else MDY_WQ(1, false);
-    }
+#define MDY_WQ_V(MODE, XT) do { if (vec) MDY_WQ(MODE, true, XT); else MDY_WQ(MODE, false, XT); } while (0)
+#define MDY_WQ_X(MODE) do { if (w_dtype == 0) MDY_WQ_V(MODE, 0); else if (w_dtype == 1) MDY_WQ_V(MODE, 1); else MDY_WQ_V(MODE, 2); } while (0)
+    if (mode == 0) MDY_WQ_X(0); else MDY_WQ_X(1);
+#undef MDY_WQ_X
+#undef MDY_WQ_V
 #undef MDY_WQ
     return (int)hipGetLastError();
 }

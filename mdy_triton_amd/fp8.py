@@ -21,8 +21,7 @@ def _quant_transpose(x: torch.Tensor, t_mode: int, who: str):
     """Shared launcher of the two training-time quantizers (row-wise copy + quantized transpose)."""
     if x.dim() != 2:
         raise ValueError("%s expects a 2-D tensor" % who)
-    if x.dtype != torch.bfloat16:
-        raise TypeError("%s expects bfloat16, got %s" % (who, x.dtype))
+    xt = xt_code(x, who)
     dev = require_gpu(x)
     M, K = x.shape
     PM, PN = _cdiv(M, 256) * 256, _cdiv(K, 256) * 256
@@ -32,7 +31,7 @@ def _quant_transpose(x: torch.Tensor, t_mode: int, who: str):
     y_t = torch.empty(PN, PM, device=dev, dtype=FP8)
     s_t = torch.empty((A, PN) if t_mode == 0 else (B, A), device=dev, dtype=torch.float32)
     with on_device(dev):
-        check(lib().mdy_quant_transpose(ptr(x), ptr(y), ptr(s), ptr(y_t), ptr(s_t), M, K, x.stride(0), x.stride(1),
+        check(lib().mdy_quant_transpose_typed(ptr(x), xt, ptr(y), ptr(s), ptr(y_t), ptr(s_t), M, K, x.stride(0), x.stride(1),
                                         PM, PN, PM, t_mode, stream_ptr(dev)), who)
     return y, s.transpose(0, 1), y_t, s_t
 
@@ -89,8 +88,7 @@ def quant_weight(x: torch.Tensor, only_forward: bool = True):
     """
     if x.dim() != 2:
         raise ValueError("quant_weight expects a 2-D tensor")
-    if x.dtype != torch.bfloat16:
-        raise TypeError("quant_weight expects bfloat16, got %s" % x.dtype)
+    xt = xt_code(x, "quant_weight")
     dev = require_gpu(x)
     N, K = x.shape
     BA = 128 if only_forward else 256
@@ -103,15 +101,16 @@ def quant_weight(x: torch.Tensor, only_forward: bool = True):
         y_t = torch.empty(PN, PM, device=dev, dtype=FP8)
         s_t = torch.empty(B, A, device=dev, dtype=torch.float32)
     with on_device(dev):
-        check(lib().mdy_weight_quant(ptr(x), ptr(y), ptr(s), ptr(y_t), ptr(s_t), N, K, x.stride(0), x.stride(1),
+        check(lib().mdy_weight_quant_typed(ptr(x), xt, ptr(y), ptr(s), ptr(y_t), ptr(s_t), N, K, x.stride(0), x.stride(1),
                                      PM, PN, 1, stream_ptr(dev)), "quant_weight")
     return y, s, y_t, s_t
 
 
 def add_bias(x: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     """In-place x[..., :] += b in fp32, stored back as bf16 (fp8.py:297-305)."""
-    if x.dtype != torch.bfloat16 or b.dtype != torch.bfloat16:
-        raise TypeError("add_bias expects bfloat16 tensors")
+    if x.dtype != torch.bfloat16:
+        raise TypeError("add_bias expects a bfloat16 x (the GEMM's output type), got %s" % x.dtype)
+    bt = xt_code(b, "add_bias")
     if not x.is_contiguous() or not b.is_contiguous():
         raise ValueError("add_bias expects contiguous tensors")
     dev = require_gpu(x, b)
@@ -120,7 +119,7 @@ def add_bias(x: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
         raise ValueError("bias has %d elements, rows have %d" % (b.numel(), N))
     M = x.numel() // N if N else 0
     with on_device(dev):
-        check(lib().mdy_add_bias(ptr(x), ptr(b), M, N, stream_ptr(dev)), "add_bias")
+        check(lib().mdy_add_bias_typed(ptr(x), ptr(b), bt, M, N, stream_ptr(dev)), "add_bias")
     return x
 
 
@@ -189,6 +188,7 @@ class _DeepLinear(torch.autograd.Function):
             ctx.dims = (M, N, K)
             ctx.quantized = (q_inp_t, s_inp_t, q_weight_t, s_weight_t)
             ctx.has_bias = bias is not None
+        fuse_bias = bool(fuse_bias and bias is not None and bias.dtype == torch.bfloat16)    # the epilogue takes a bf16 bias
         out = fp8_matmul(q_inp[:M], s_inp[:M], q_weight[:N], s_weight[:_cdiv(N, 128)],
                          bias=bias if fuse_bias else None)
         if bias is not None and not fuse_bias:

@@ -13,7 +13,7 @@ from typing import Optional, Tuple
 
 import torch
 
-from ._torch_glue import FP8, check, lib, on_device, ptr, require_gpu, stream_ptr
+from ._torch_glue import FP8, check, lib, on_device, ptr, require_gpu, stream_ptr, xt_code
 
 _ORDERS = ("up-gate", "gate-up")
 
@@ -129,8 +129,9 @@ def weight_quant_block(x: torch.Tensor, BLOCK_M: int = 128, BLOCK_N: int = 128,
         raise ValueError("only 128x128 blocks are implemented (the reference default)")
     if dtype != FP8:
         raise TypeError("only torch.float8_e4m3fn is implemented")
-    if x.dim() != 2 or x.dtype != torch.bfloat16:
-        raise TypeError("weight_quant_block expects a 2-D bfloat16 tensor")
+    if x.dim() != 2:
+        raise TypeError("weight_quant_block expects a 2-D tensor")
+    xt = xt_code(x, "weight_quant_block")
     dev = require_gpu(x)
     M, N = x.shape
     if M % 128 != 0:
@@ -138,7 +139,7 @@ def weight_quant_block(x: torch.Tensor, BLOCK_M: int = 128, BLOCK_N: int = 128,
     y = torch.empty(M, N, device=dev, dtype=FP8)
     s = torch.empty(M // 128, N // 128, device=dev, dtype=torch.float32)
     with on_device(dev):
-        check(lib().mdy_weight_quant(ptr(x), ptr(y), ptr(s), None, None, M, N, x.stride(0), x.stride(1), M, N, 0,
+        check(lib().mdy_weight_quant_typed(ptr(x), xt, ptr(y), ptr(s), None, None, M, N, x.stride(0), x.stride(1), M, N, 0,
                                      stream_ptr(dev)), "weight_quant_block")
     return y, s
 
@@ -146,8 +147,7 @@ def weight_quant_block(x: torch.Tensor, BLOCK_M: int = 128, BLOCK_N: int = 128,
 def _act_quant_transposed(x2: torch.Tensor, with_rows: bool, who: str):
     """x2 [M, N] bf16 (any strides) -> (y, s, y_t_padded, s_t): the official-dialect row-wise quantization (None, None
     unless with_rows) and the quantized transpose y_t [N, PM] with s_t [N, PM/128], PM = cdiv(M, 128) * 128."""
-    if x2.dtype != torch.bfloat16:
-        raise TypeError("%s expects a bfloat16 tensor, got %s" % (who, x2.dtype))
+    xt = xt_code(x2, who)
     dev = require_gpu(x2)
     M, N = x2.shape
     PM = (M + 127) // 128 * 128
@@ -157,7 +157,7 @@ def _act_quant_transposed(x2: torch.Tensor, with_rows: bool, who: str):
     s_t = torch.empty(N, PM // 128, device=dev, dtype=torch.float32)
     if PM * N > 0:
         with on_device(dev):
-            check(lib().mdy_act_quant_transpose(ptr(x2), ptr(y), ptr(s), ptr(y_t), ptr(s_t), M, N, x2.stride(0), x2.stride(1),
+            check(lib().mdy_act_quant_transpose(ptr(x2), xt, ptr(y), ptr(s), ptr(y_t), ptr(s_t), M, N, x2.stride(0), x2.stride(1),
                                                 PM, N, stream_ptr(dev)), who)
     return y, s, y_t, s_t
 
@@ -198,9 +198,13 @@ def fp8_matmul(x: torch.Tensor, w: torch.Tensor, scale_x: torch.Tensor, scale_w:
         assert x.size(-1) % 128 == 0, 'in forward x @ w.T'
         from .offical_kernel import fp8_gemm
         x2 = x.reshape(-1, x.size(-1))
+        fused = bias is not None and bias.dtype == torch.bfloat16        # the GEMM epilogue takes a bf16 bias
         y = fp8_gemm(x2 if x2.is_contiguous() else x2.contiguous(), scale_x.reshape(-1, scale_x.size(-1)).contiguous(),
                      w if w.is_contiguous() else w.contiguous(), scale_w.contiguous(), out_dtype=torch.bfloat16,
-                     bias=None if bias is None else bias.to(torch.bfloat16).contiguous())
+                     bias=bias.contiguous() if fused else None)
+        if bias is not None and not fused:                               # fp16 / fp32 bias: added in fp32 afterwards
+            from .fp8 import add_bias
+            add_bias(y, bias.contiguous())
         return y.view(*x.shape[:-1], w.size(0))
     assert x.size(0) % 128 == 0, 'in backward dy.T @ x or dy @ w'
     assert bias is None

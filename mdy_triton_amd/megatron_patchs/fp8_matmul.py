@@ -11,13 +11,15 @@ from typing import List, Optional, Sequence
 
 import torch
 
-from .._torch_glue import FP8, check, lib, on_device, ptr, require_gpu, stream_ptr
+from .._torch_glue import FP8, check, lib, on_device, ptr, require_gpu, stream_ptr, xt_code
 from ..fp8 import _cdiv, fp8_matmul, quant_input  # noqa: F401  (fp8_matmul is re-exported under the reference's name)
 
 
-def _check_bf16_2d(x, who):
-    if x.dim() != 2 or x.dtype != torch.bfloat16:
-        raise TypeError("%s expects a 2-D bfloat16 tensor" % who)
+def _check_2d(x, who):
+    """2-D bf16 / fp16 / fp32 input; returns its type code for the typed entry points."""
+    if x.dim() != 2:
+        raise TypeError("%s expects a 2-D tensor" % who)
+    return xt_code(x, who)
 
 
 def per_token_cast_to_fp8(x: torch.Tensor, output_transpose: bool = False):
@@ -30,7 +32,7 @@ def per_token_cast_to_fp8(x: torch.Tensor, output_transpose: bool = False):
     """
     if not output_transpose:
         return quant_input(x, only_forward=True)
-    _check_bf16_2d(x, "per_token_cast_to_fp8")
+    xt = _check_2d(x, "per_token_cast_to_fp8")
     dev = require_gpu(x)
     M, N = x.shape
     PM, PN = _cdiv(M, 128) * 128, _cdiv(N, 256) * 256
@@ -40,7 +42,7 @@ def per_token_cast_to_fp8(x: torch.Tensor, output_transpose: bool = False):
     s_t = torch.empty(PM // 128, PN, device=dev, dtype=torch.float32)
     if PM * PN > 0:
         with on_device(dev):
-            check(lib().mdy_quant_transpose(ptr(x), ptr(y), ptr(s), ptr(y_t), ptr(s_t), M, N, x.stride(0), x.stride(1), PM, PN,
+            check(lib().mdy_quant_transpose_typed(ptr(x), xt, ptr(y), ptr(s), ptr(y_t), ptr(s_t), M, N, x.stride(0), x.stride(1), PM, PN,
                                             PM, 0, stream_ptr(dev)), "per_token_cast_to_fp8")
     return y, s.transpose(0, 1), y_t, s_t.transpose(0, 1)
 
@@ -52,7 +54,7 @@ def group_per_token_cast_to_fp8(x_all: torch.Tensor, m_splits: Sequence[int]):
     Returns (y_all [M, N], s_all logical [M, N/128] with strides (1, M), [y_t of group g: [N, m_g]],
     [s_t of group g: logical [N, m_g/128]]).
     """
-    _check_bf16_2d(x_all, "group_per_token_cast_to_fp8")
+    xt = _check_2d(x_all, "group_per_token_cast_to_fp8")
     dev = require_gpu(x_all)
     Mtot, N = x_all.shape
     if sum(m_splits) != Mtot:
@@ -68,7 +70,7 @@ def group_per_token_cast_to_fp8(x_all: torch.Tensor, m_splits: Sequence[int]):
             s_t = torch.empty(mg // 128, N, device=dev, dtype=torch.float32)
             if mg > 0:
                 x = x_all[row:row + mg]
-                check(lib().mdy_quant_transpose(ptr(x), ptr(y_all[row:]), s_all.data_ptr() + 4 * row, ptr(y_t), ptr(s_t), mg, N,
+                check(lib().mdy_quant_transpose_typed(ptr(x), xt, ptr(y_all[row:]), s_all.data_ptr() + 4 * row, ptr(y_t), ptr(s_t), mg, N,
                                                 x.stride(0), x.stride(1), mg, N, Mtot, 0, stream_ptr(dev)),
                       "group_per_token_cast_to_fp8")
             yt_all.append(y_t)
@@ -85,8 +87,8 @@ def per_block_cast_to_fp8(x, output_normal: bool = True, output_transpose: bool 
     """
     xs: List[torch.Tensor] = list(x) if isinstance(x, (list, tuple)) else [x]
     for w in xs:
-        _check_bf16_2d(w, "per_block_cast_to_fp8")
-        if w.shape != xs[0].shape:
+        xt = _check_2d(w, "per_block_cast_to_fp8")
+        if w.shape != xs[0].shape or w.dtype != xs[0].dtype:
             raise ValueError("per_block_cast_to_fp8: all weights must have the same shape")
     dev = require_gpu(*xs)
     G = len(xs)
@@ -102,7 +104,7 @@ def per_block_cast_to_fp8(x, output_normal: bool = True, output_transpose: bool 
     if PM * PN > 0:
         with on_device(dev):
             for g, w in enumerate(xs):
-                check(lib().mdy_weight_quant(ptr(w), ptr(y[g]), ptr(s[g]), ptr(y_t[g]) if output_transpose else None,
+                check(lib().mdy_weight_quant_typed(ptr(w), xt, ptr(y[g]), ptr(s[g]), ptr(y_t[g]) if output_transpose else None,
                                              ptr(s_t[g]) if output_transpose else None, M, N, w.stride(0), w.stride(1), PM, PN, 1,
                                              stream_ptr(dev)), "per_block_cast_to_fp8")
     post = (lambda t: t.squeeze(0)) if G == 1 else (lambda t: t)

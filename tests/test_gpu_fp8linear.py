@@ -104,7 +104,8 @@ def test_rowscaled_gemm_random_and_ragged_k():
     assert L.mdy_fp8_gemm_nt_rowscaled(p + 1, p, 1, 1, p, p, 1, 1, p, 4, 4, 128, 0, None) == -3
     assert L.mdy_fp8_gemm_nt_rowscaled(None, p, 1, 1, p, p, 1, 1, p, 4, 4, 128, 0, None) == -1
     assert L.mdy_fp8_gemm_nt_rowscaled(p, p, -1, 1, p, p, 1, 1, p, 4, 4, 128, 0, None) == -2
-    assert L.mdy_act_quant_transpose(p, None, p, p, p, 4, 128, 128, 1, 128, 128, None) == -1
+    assert L.mdy_act_quant_transpose(p, 0, None, p, p, p, 4, 128, 128, 1, 128, 128, None) == -1
+    assert L.mdy_act_quant_transpose(p, 7, p, p, p, p, 4, 128, 128, 1, 128, 128, None) == -4
 
 
 @pytest.mark.parametrize("bias", [True, False])

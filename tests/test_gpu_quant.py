@@ -470,3 +470,69 @@ def test_act_quant_and_weight_dequant_other_block_sizes(bs, dtype):
         m.act_quant(x.to(DEV)[:, :960].contiguous(), 96)
     with pytest.raises(ValueError):
         m.weight_dequant(wq.to(DEV), ws.to(DEV), 100)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_weight_and_training_quantizers_fp16_fp32_inputs(dtype):
+    """Every quantizer takes fp16 and fp32 tensors like the reference's kernels (.to(tl.float32) on load): the block
+    weight quantizers (an fp32 master weight), the training quantizers with their transposed copies, and the
+    official-dialect pair; all bit-exact against the oracle, whose arithmetic is dtype-agnostic."""
+    g = torch.Generator().manual_seed(17)
+    w = (torch.randn(300, 520, generator=g) * 0.02).to(dtype)
+    for only_forward in (True, False):
+        got = m.quant_weight(w.to(DEV), only_forward)
+        ref = O.quant_weight(w, only_forward)
+        for a, b in zip(got, ref):
+            assert (a is None) == (b is None)
+            if a is not None:
+                assert torch.equal(a.cpu().contiguous().view(torch.uint8) if a.dtype == FP8 else a.cpu(), b.contiguous().view(torch.uint8) if b.dtype == FP8 else b)
+    wb = (torch.randn(256, 384, generator=g) * 0.02).to(dtype)
+    y, s = m.weight_quant_block(wb.to(DEV))
+    yr, sr = O.weight_quant_block(wb)
+    assert torch.equal(y.cpu().view(torch.uint8), yr.view(torch.uint8)) and torch.equal(s.cpu(), sr)
+    yt, st = m.weight_quant_block(wb.to(DEV).t())                   # strided (transposed view)
+    ytr, str_ = O.weight_quant_block(wb.t().contiguous())
+    assert torch.equal(yt.cpu().view(torch.uint8), ytr.view(torch.uint8)) and torch.equal(st.cpu(), str_)
+    x = torch.randn(300, 512, generator=g).to(dtype)
+    for fn, ofn in ((lambda t: m.quant_input(t, False), lambda t: O.quant_input(t, False)), (m.quant_grad_output, O.quant_grad_output),
+                    (lambda t: m.per_token_cast_to_fp8(t, True), lambda t: O.per_token_cast_to_fp8(t, True))):
+        for a, b in zip(fn(x.to(DEV)), ofn(x)):
+            a, b = a.cpu().contiguous(), b.contiguous()
+            assert a.shape == b.shape and torch.equal(a.view(torch.uint8) if a.dtype == FP8 else a, b.view(torch.uint8) if b.dtype == FP8 else b)
+    yb, sb = m.act_quant_block(x.to(DEV), transpose=True)
+    ybr, sbr = O.act_quant_block(x, transpose=True)
+    assert torch.equal(yb.cpu().view(torch.uint8), ybr.view(torch.uint8)) and torch.equal(sb.cpu(), sbr)
+    q = m.per_block_cast_to_fp8([w.to(DEV), (w * 2).to(DEV)], output_transpose=True)
+    qr = O.per_block_cast_to_fp8([w, w * 2], output_transpose=True)
+    for a, b in zip(q, qr):
+        assert torch.equal(a.cpu().view(torch.uint8) if a.dtype == FP8 else a.cpu(), b.view(torch.uint8) if b.dtype == FP8 else b)
+
+
+def test_deep_linear_and_fp8_linear_with_fp32_parameters():
+    """nn.Linear's default dtype: fp32 weight, bias and input.  The forward quantizes them from their exact values and
+    returns bf16 like the reference's GEMM; the bias is added in fp32."""
+    g = torch.Generator().manual_seed(23)
+    x = torch.randn(64, 512, generator=g)
+    with torch.no_grad():
+        lin = m.DeepLinear(512, 256, bias=True)
+        assert lin.weight.dtype == torch.float32
+        lin.weight.copy_(torch.randn(256, 512, generator=g) * 0.03)
+        lin.bias.copy_(torch.randn(256, generator=g))
+        ref = O.deep_linear_forward(x, lin.weight.detach(), None).float() + lin.bias.detach()
+        lin = lin.to(DEV)
+        out = lin(x.to(DEV))
+        lin.fuse_bias = True                       # not fusable with an fp32 bias: falls back to the separate add
+        assert torch.equal(lin(x.to(DEV)), out)
+    assert out.dtype == torch.bfloat16
+    mag = torch.maximum(ref.abs(), (ref - lin.bias.detach().cpu()).abs())
+    assert bool(((out.float().cpu() - ref).abs() <= 2e-2 + 1e-2 * mag).all())
+    nb = torch.randn(8, 200, generator=g).bfloat16()
+    bias = torch.randn(200, generator=g)
+    got = m.add_bias(nb.clone().to(DEV), bias.to(DEV))
+    assert torch.equal(got.cpu(), (nb.float() + bias).bfloat16())
+    with torch.no_grad():
+        fl = m.Fp8Linear(512, 256, bias=True)
+        fl.weight.copy_(lin.weight.cpu()); fl.bias.copy_(lin.bias.cpu())
+        ref2 = O.fp8_linear_forward(x, fl.weight.detach(), None).float() + fl.bias.detach()
+        out2 = fl.to(DEV)(x.to(DEV))
+    assert bool(((out2.float().cpu() - ref2).abs() <= 2e-2 + 1e-2 * mag).all())
