@@ -222,3 +222,37 @@ def test_rowscaled_gemm_non_finite_values():
     assert torch.equal(torch.isinf(got), torch.isinf(ref)) and torch.equal(got[torch.isinf(ref)], ref[torch.isinf(ref)])
     fin = torch.isfinite(ref)
     assert fin[4:].any() and torch.allclose(got[fin], ref[fin], rtol=1e-4, atol=1e-2)
+
+
+def test_fp8_linear_reproduces_the_reference_notebook_error_magnitudes():
+    """The one numeric record the reference keeps for this layer (deepseekv3/fp8-benchmark.ipynb cell 6, outputs at raw
+    lines 195 / 216 / 236 / 256): Fp8Linear (e4m3fn) against a bf16 nn.Linear with the same parameters, bs = 4,
+    seq = 4096, d = 4096, bias, x ~ randn, dy ~ rand: forward max / mean |error| 0.1172 / 0.0167, input gradient
+    0.0669 / 0.0095, weight gradient 14.0 / 2.11, bias gradient allclose.  The data there is unseeded, so the
+    statistics are what can be compared: a quantizer or GEMM that computed something else (another scale rule, a
+    dropped K block, transposed scales) moves the means by far more than the 6 % bands below (measured here: 0.1172-0.125 / 0.0167, 0.0664-0.0669 / 0.0095,
+    14.5-14.9 / 2.113)."""
+    torch.manual_seed(0)
+    bs, seq, d = 4, 4096, 4096
+    x1 = torch.randn(bs, seq, d, dtype=torch.bfloat16, device=DEV).requires_grad_(True)
+    x2 = x1.detach().clone().requires_grad_(True)
+    fc1 = torch.nn.Linear(d, d, bias=True, device=DEV, dtype=torch.bfloat16)
+    fc2 = m.Fp8Linear(d, d, bias=True, device=DEV, dtype=torch.bfloat16, fp8_dtype=torch.float8_e4m3fn)
+    with torch.no_grad():
+        fc2.weight.copy_(fc1.weight)
+        fc2.bias.copy_(fc1.bias)
+    y1, y2 = fc1(x1), fc2(x2)
+    dy = torch.rand_like(y1)
+    y1.backward(dy)
+    y2.backward(dy)
+
+    def err(a, b):
+        e = (a.float() - b.float()).abs()
+        return e.max().item(), e.mean().item()
+    fmax, fmean = err(y1, y2)
+    gmax, gmean = err(x1.grad, x2.grad)
+    wmax, wmean = err(fc1.weight.grad, fc2.weight.grad)
+    assert 0.94 * 0.0167 < fmean < 1.06 * 0.0167 and 0.5 * 0.1172 < fmax < 2 * 0.1172, (fmax, fmean)
+    assert 0.94 * 0.0095 < gmean < 1.06 * 0.0095 and 0.5 * 0.0669 < gmax < 2 * 0.0669, (gmax, gmean)
+    assert 0.94 * 2.11 < wmean < 1.06 * 2.11 and 0.5 * 14.0 < wmax < 2 * 14.0, (wmax, wmean)
+    assert torch.allclose(fc1.bias.grad, fc2.bias.grad)
