@@ -85,6 +85,16 @@ def fp8_gemm(a: torch.Tensor, a_s: torch.Tensor, b: torch.Tensor, b_s: torch.Ten
         raise ValueError("bias must be a contiguous bfloat16 [N] tensor")
     dtype = out_dtype or torch.get_default_dtype()
     c = a.new_empty(*a.size()[:-1], N, dtype=dtype)
+    if K % 128 != 0 and M * N * K >= (1 << 24):
+        # A K tail (the masked loads of offical_kernel.py:82-83) would send the whole problem to the one-thread-per-output
+        # kernel; zero bytes contribute nothing to any sum, so a problem of any size is completed with zero columns to the
+        # next multiple of 128 instead (the scales already have one column for the partial block) and runs on the MFMA kernels.
+        PK = KB * 128
+        a2 = torch.zeros(M, PK, dtype=torch.uint8, device=dev)
+        a2[:, :K] = a.reshape(M, K).view(torch.uint8)
+        b2 = torch.zeros(N, PK, dtype=torch.uint8, device=dev)
+        b2[:, :K] = b.view(torch.uint8)
+        a, b, K = a2.view(FP8), b2.view(FP8), PK
     with on_device(dev):
         warn_if_scalar_gemm(a, b, KB, 1, M, N, K, "fp8_gemm")
         ws = gemm_workspace(dev, M, N, K)      # scratch for shapes that are split along K, else None

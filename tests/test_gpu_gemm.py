@@ -381,6 +381,32 @@ def test_gemm_ragged_k_scalar_path(M, N, K):
     assert torch.allclose(got.cpu(), ref, rtol=1e-4, atol=1e-6)
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 512, 1000), (16, 4096, 300), (1000, 260, 7170)])
+def test_gemm_ragged_k_large_shapes_run_padded(M, N, K):
+    """A larger problem with K % 128 != 0 is completed with zero columns and runs on the MFMA kernels: exact on
+    integer operands, and equal to the scalar kernel's masked tail within fp32 summation order."""
+    g = torch.Generator().manual_seed(K)
+    ai = torch.randint(-4, 5, (M, K), generator=g)
+    bi = torch.randint(-4, 5, (N, K), generator=g)
+    KB, NB = (K + 127) // 128, (N + 127) // 128
+    ae = torch.randint(-2, 3, (M, KB), generator=g)
+    be = torch.randint(-2, 3, (NB, KB), generator=g)
+    c = torch.zeros(M, N, dtype=torch.float64)
+    for kb in range(KB):
+        part = ai[:, kb * 128:(kb + 1) * 128].double() @ bi[:, kb * 128:(kb + 1) * 128].double().t()
+        c += part * torch.exp2((ae[:, kb][:, None] + be[torch.arange(N) // 128, kb][None, :]).double())
+    a, b = ai.float().to(FP8).to(DEV), bi.float().to(FP8).to(DEV)
+    a_s, b_s = torch.exp2(ae.float()).to(DEV), torch.exp2(be.float()).to(DEV)
+    got = m.fp8_gemm(a, a_s, b, b_s, out_dtype=torch.float32)
+    assert torch.equal(got.cpu().double(), c)
+    lib = _lib.load()
+    ref = torch.full((M, N), float("nan"), device=DEV)
+    assert lib.mdy_fp8_gemm_nt(a.data_ptr(), a_s.data_ptr(), KB, 1, b.data_ptr(), b_s.data_ptr(), ref.data_ptr(), None, M, N, K, 1,
+                               None) == 0                       # the C entry point itself: scalar kernel, masked tail
+    torch.cuda.synchronize()
+    assert torch.equal(ref.cpu().double(), c)
+
+
 def test_gemm_leading_dims_default_dtype_and_bias():
     a, a_s, wq, ws = quantized_problem("normal", 96, 384, 256, 5)
     a3, a3_s = a.reshape(2, 48, 256), a_s.reshape(2, 48, 2)
