@@ -628,7 +628,7 @@ def table(torch, m, timer, dev):
              6.0 * Mr * Nr * Kr, "TFLOP/s", PEAK_FP8_TFLOPS)
         del lin, xg, dy
     for d in (4096, 7168, 8192):          # fp8-benchmark.ipynb:351-359 (fwd), :456-464 (bwd): x = [8192, d], W = [d, d]
-        lin = m.Fp8Linear(d, d, bias=False, dtype=torch.bfloat16, device=dev)
+        lin = m.Fp8Linear(d, d, bias=False, dtype=torch.bfloat16, device=dev, fp8_dtype=torch.float8_e4m3fn)
         xg = torch.randn(8192, d, device=dev).bfloat16().requires_grad_(True)
         dy = torch.randn(8192, d, device=dev).bfloat16()
         with torch.no_grad():

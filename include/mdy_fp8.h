@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define MDY_FP8_ABI_VERSION 12
+#define MDY_FP8_ABI_VERSION 13
 
 /* error codes (negative = argument rejected before any launch) */
 #define MDY_OK 0
@@ -45,6 +45,13 @@ extern "C" {
 /* quantizer dialects */
 #define MDY_QUANT_OFFICIAL 0 /* s = amax / 448                      offical_kernel.py:14 */
 #define MDY_QUANT_DEEPLINEAR 1 /* s = (min(amax,1e4) + 1e-8) / 448, saturating cast  fp8.py:109-111 */
+#define MDY_QUANT_OFFICIAL_E5M2 2 /* s = amax / 57344, e5m2 bytes: the default fp8 dtype of triton_kernels/deepseekv3/
+                                   * fp8_kernel.py (:62, :124, :303); accepted by mdy_act_quant_typed, mdy_weight_quant(_typed)
+                                   * and mdy_act_quant_transpose */
+
+/* operand byte formats of mdy_fp8_gemm_nt_rowscaled */
+#define MDY_FMT_E4M3 0
+#define MDY_FMT_E5M2 1
 
 int mdy_fp8_abi_version(void);
 const char* mdy_fp8_last_error(void);
@@ -129,7 +136,8 @@ int mdy_quant_transpose_typed(const void* x, int x_dtype, void* y, float* s, voi
                         int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int64_t s_kb_stride,
                         int t_mode, void* stream);
 
-/* Official-dialect training quantizer (s = amax / 448, no clamp, no eps): the row-wise 1x128 quantization of x and
+/* Official-dialect training quantizer (mode MDY_QUANT_OFFICIAL: s = amax / 448, e4m3fn; MDY_QUANT_OFFICIAL_E5M2:
+ * s = amax / 57344, e5m2; no clamp, no eps): the row-wise 1x128 quantization of x and
  * the quantized transpose with one scale per column and 128 rows, one read of x.  Replaces the pair
  * act_quant_block(x) / act_quant_block(x, transpose=True) (triton_kernels/deepseekv3/fp8_kernel.py:62-87, kernel
  * :14-60) that the reference's Fp8Linear runs on x and on dy (:286-301).
@@ -143,7 +151,7 @@ int mdy_quant_transpose_typed(const void* x, int x_dtype, void* y, float* s, voi
  * reference).  y / y_t 8-byte aligned.
  */
 int mdy_act_quant_transpose(const void* x, int x_dtype, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
-                            int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, void* stream);
+                            int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int mode, void* stream);
 
 /* Block-scaled FP8 GEMM, NT layout, with 1x128 scales on both operands:
  *   c[m, n] = sum_kb (sum_{k in kb} a[m,k] * b[n,k]) * a_s[m, kb] * b_s[n, kb]
@@ -153,11 +161,14 @@ int mdy_act_quant_transpose(const void* x, int x_dtype, void* y, float* s, void*
  *   a   e4m3fn [M, K] row-major, 16-byte aligned     a_s fp32, element (m, kb) at a_s[m * as_row_stride + kb * as_col_stride]
  *   b   e4m3fn [N, K] row-major, 16-byte aligned     b_s fp32, element (n, kb) at b_s[n * bs_row_stride + kb * bs_col_stride]
  *   c   [M, N] row-major of out_dtype
+ * fmt: byte format of BOTH operands, MDY_FMT_E4M3 or MDY_FMT_E5M2.  A weight with 128x128 block scales runs here too
+ * with its scales expanded to one per row (bs_row_stride of the expanded tensor): the Python wrappers do that for e5m2
+ * operands, which the block-scaled kernels of mdy_fp8_gemm_nt (e4m3fn only) do not take.
  * K % 128 == 0, K <= 2^20; scale strides non-negative, each scale tensor spanning less than 2^31 bytes.
  */
 int mdy_fp8_gemm_nt_rowscaled(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
                               const void* b, const float* b_s, int64_t bs_row_stride, int64_t bs_col_stride, void* c,
-                              int64_t M, int64_t N, int64_t K, int out_dtype, void* stream);
+                              int64_t M, int64_t N, int64_t K, int fmt, int out_dtype, void* stream);
 
 /* SwiGLU, alone or fused with the 1x128 activation quantizer that feeds the next GEMM.
  *   act[m, n] = bf16( silu(gate[m, n]) * up[m, n] ), silu(g) = g / (1 + exp(-g)) in fp32;
@@ -337,6 +348,8 @@ int mdy_add_grad(void* x, const void* y, int64_t n, int x_dtype, int y_dtype, vo
  * counterpart in the reference (the cast is implicit in tl.store, fp8.py:112);
  * exists so that the cast can be checked against the format definition. */
 int mdy_cast_f32_to_e4m3(const float* x, void* y, int64_t n, int saturate, void* stream);
+/* The same for the e5m2 conversion (round to nearest even, overflow to infinity), used by MDY_QUANT_OFFICIAL_E5M2. */
+int mdy_cast_f32_to_e5m2(const float* x, void* y, int64_t n, void* stream);
 
 /* Diagnostic: returns in out[0..3] the number of (amax, x) bf16 pairs, of fp32
  * quotient mismatches and of e4m3fn byte mismatches between the quantizers'

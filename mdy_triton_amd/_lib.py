@@ -10,7 +10,7 @@ import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libmdyfp8.so")
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 _lock = threading.Lock()
 _lib = None
@@ -28,8 +28,8 @@ SIGNATURES = {
     "mdy_quant_transpose": [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p],
     "mdy_quant_transpose_typed": [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p],
     "mdy_fp8_grouped_gemm_nt": [_p, _p, _i64, _i64, _p, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p],
-    "mdy_act_quant_transpose": [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p],
-    "mdy_fp8_gemm_nt_rowscaled": [_p, _p, _i64, _i64, _p, _p, _i64, _i64, _p, _i64, _i64, _i64, _int, _p],
+    "mdy_act_quant_transpose": [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _int, _p],
+    "mdy_fp8_gemm_nt_rowscaled": [_p, _p, _i64, _i64, _p, _p, _i64, _i64, _p, _i64, _i64, _i64, _int, _int, _p],
     "mdy_swiglu": [_p, _p, _p, _p, _i64, _i64, _i64, _int, _i64, _i64, _i64, _i64, _int, _p],
     "mdy_swiglu_bwd": [_p, _p, _p, _i64, _i64, _i64, _int, _p],
     "mdy_weight_dequant": [_p, _p, _p, _i64, _i64, _int, _p],
@@ -47,6 +47,7 @@ SIGNATURES = {
     "mdy_add_bias": [_p, _p, _i64, _i64, _p],
     "mdy_add_bias_typed": [_p, _p, _int, _i64, _i64, _p],
     "mdy_cast_f32_to_e4m3": [_p, _p, _i64, _int, _p],
+    "mdy_cast_f32_to_e5m2": [_p, _p, _i64, _p],
     "mdy_quotient_selfcheck": [_p, _int, _int, _int, _p],
     "mdy_fp8_abi_version": [],
     "mdy_fp8_last_error": [],

@@ -223,7 +223,7 @@ __global__ __launch_bounds__(256) void act_quant_typed_kernel(const void* __rest
 int launch_act_quant_typed(const void* x, int x_dtype, int block_size, void* y, float* s, int64_t M, int64_t K,
                            int64_t x_row_stride, int64_t PM, int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode,
                            hipStream_t stream) {
-    if (x_dtype == 0 && block_size == 128)
+    if (x_dtype == 0 && block_size == 128 && mode != 2)
         return launch_act_quant(x, y, s, M, K, x_row_stride, PM, PK, s_row_stride, s_col_stride, mode, stream);
     if (PM == 0 || PK == 0) return 0;
     const int esz = x_dtype == 2 ? 4 : 2;
@@ -239,7 +239,7 @@ int launch_act_quant_typed(const void* x, int x_dtype, int block_size, void* y, 
                        x_row_stride, (int)PM, (int)PK, s_row_stride, s_col_stride, lanes, shift)
 #define MDY_AQT_V(MODE, XT) do { if (vec) MDY_AQT(MODE, XT, true); else MDY_AQT(MODE, XT, false); } while (0)
 #define MDY_AQT_X(MODE) do { if (x_dtype == 0) MDY_AQT_V(MODE, 0); else if (x_dtype == 1) MDY_AQT_V(MODE, 1); else MDY_AQT_V(MODE, 2); } while (0)
-    if (mode == 0) MDY_AQT_X(0); else MDY_AQT_X(1);
+    if (mode == 0) MDY_AQT_X(0); else if (mode == 1) MDY_AQT_X(1); else MDY_AQT_X(2);
 #undef MDY_AQT_X
 #undef MDY_AQT_V
 #undef MDY_AQT
@@ -306,6 +306,19 @@ __global__ void cast_f32_to_e4m3_kernel(const float* __restrict__ x, uint8_t* __
         v = (v != v) ? v : c;
     }
     y[i] = (uint8_t)(pack4_e4m3(v, 0.0f, 0.0f, 0.0f) & 0xFFu);
+}
+
+__global__ void cast_f32_to_e5m2_kernel(const float* __restrict__ x, uint8_t* __restrict__ y, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    y[i] = (uint8_t)(pack4_e5m2(x[i], 0.0f, 0.0f, 0.0f) & 0xFFu);
+}
+
+int launch_cast_f32_to_e5m2(const float* x, void* y, int64_t n, hipStream_t stream) {
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(cast_f32_to_e5m2_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x,
+                       static_cast<uint8_t*>(y), n);
+    return (int)hipGetLastError();
 }
 
 int launch_cast_f32_to_e4m3(const float* x, void* y, int64_t n, int saturate, hipStream_t stream) {

@@ -78,10 +78,10 @@ static bool block_size_ok(int64_t bs, int64_t lo, int64_t hi) { return bs >= lo 
 
 int mdy_act_quant_typed(const void* x, int x_dtype, int block_size, void* y, float* s, int64_t M, int64_t K, int64_t x_row_stride,
                         int64_t PM, int64_t PK, int64_t s_row_stride, int64_t s_col_stride, int mode, void* stream) {
-    if (x_dtype == MDY_XT_BF16 && block_size == 128)
+    if (x_dtype == MDY_XT_BF16 && block_size == 128 && mode != MDY_QUANT_OFFICIAL_E5M2)
         return mdy_act_quant(x, y, s, M, K, x_row_stride, PM, PK, s_row_stride, s_col_stride, mode, stream);
     if (x_dtype != MDY_XT_BF16 && x_dtype != MDY_XT_F16 && x_dtype != MDY_XT_F32) return fail(MDY_E_DTYPE, "act_quant_typed: unknown x_dtype %d", x_dtype);
-    if (mode != MDY_QUANT_OFFICIAL && mode != MDY_QUANT_DEEPLINEAR) return fail(MDY_E_DTYPE, "act_quant_typed: unknown mode %d", mode);
+    if (mode != MDY_QUANT_OFFICIAL && mode != MDY_QUANT_DEEPLINEAR && mode != MDY_QUANT_OFFICIAL_E5M2) return fail(MDY_E_DTYPE, "act_quant_typed: unknown mode %d", mode);
     if (!block_size_ok(block_size, 8, 512)) return fail(MDY_E_SHAPE, "act_quant_typed: block_size=%d must be a power of two from 8 to 512", block_size);
     if (M < 0 || K < 0 || PM < M || PK < K || PM > kMaxDim || PK > kMaxDim)
         return fail(MDY_E_SHAPE, "act_quant_typed: need 0 <= M <= PM, 0 <= K <= PK");
@@ -100,7 +100,7 @@ int mdy_act_quant_typed(const void* x, int x_dtype, int block_size, void* y, flo
 int mdy_weight_quant_typed(const void* w, int w_dtype, void* y, float* s, void* y_t, float* s_t, int64_t N, int64_t K,
                            int64_t w_row_stride, int64_t w_col_stride, int64_t PN, int64_t PK, int mode, void* stream) {
     if (w_dtype != MDY_XT_BF16 && w_dtype != MDY_XT_F16 && w_dtype != MDY_XT_F32) return fail(MDY_E_DTYPE, "weight_quant: unknown w_dtype %d", w_dtype);
-    if (mode != MDY_QUANT_OFFICIAL && mode != MDY_QUANT_DEEPLINEAR) return fail(MDY_E_DTYPE, "weight_quant: unknown mode %d", mode);
+    if (mode != MDY_QUANT_OFFICIAL && mode != MDY_QUANT_DEEPLINEAR && mode != MDY_QUANT_OFFICIAL_E5M2) return fail(MDY_E_DTYPE, "weight_quant: unknown mode %d", mode);
     if (N < 0 || K < 0 || PN < N || PK < K || PN > kMaxDim || PK > kMaxDim)
         return fail(MDY_E_SHAPE, "weight_quant: need 0 <= N <= PN, 0 <= K <= PK");
     if (PN % 128 != 0 || PK % 128 != 0) return fail(MDY_E_SHAPE, "weight_quant: PN=%lld, PK=%lld must be multiples of 128", (long long)PN, (long long)PK);
@@ -146,7 +146,8 @@ int mdy_quant_transpose(const void* x, void* y, float* s, void* y_t, float* s_t,
 }
 
 int mdy_act_quant_transpose(const void* x, int x_dtype, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
-                            int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, void* stream) {
+                            int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int mode, void* stream) {
+    if (mode != MDY_QUANT_OFFICIAL && mode != MDY_QUANT_OFFICIAL_E5M2) return fail(MDY_E_DTYPE, "act_quant_transpose: mode must be MDY_QUANT_OFFICIAL or MDY_QUANT_OFFICIAL_E5M2");
     if (x_dtype != MDY_XT_BF16 && x_dtype != MDY_XT_F16 && x_dtype != MDY_XT_F32) return fail(MDY_E_DTYPE, "act_quant_transpose: unknown x_dtype %d", x_dtype);
     if (M < 0 || K < 0 || PM < M || PK < K || PM > kMaxDim || PK > kMaxDim)
         return fail(MDY_E_SHAPE, "act_quant_transpose: need 0 <= M <= PM, 0 <= K <= PK");
@@ -157,14 +158,15 @@ int mdy_act_quant_transpose(const void* x, int x_dtype, void* y, float* s, void*
     if ((y && !aligned(y, 8)) || !aligned(y_t, 8)) return fail(MDY_E_ALIGN, "act_quant_transpose: y / y_t must be 8-byte aligned");
     if (!aligned(x, x_dtype == MDY_XT_F32 ? 4 : 2) || (s && !aligned(s, 4)) || !aligned(s_t, 4)) return fail(MDY_E_ALIGN, "act_quant_transpose: x/s/s_t misaligned for their element type");
     if (int e = check_device()) return e;
-    return launched(mdy::launch_act_quant_transpose(x, x_dtype, y, s, y_t, s_t, M, K, x_row_stride, x_col_stride, PM, PK,
+    return launched(mdy::launch_act_quant_transpose(x, x_dtype, y, s, y_t, s_t, M, K, x_row_stride, x_col_stride, PM, PK, mode,
                                                     static_cast<hipStream_t>(stream)),
                     "act_quant_transpose");
 }
 
 int mdy_fp8_gemm_nt_rowscaled(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,
                               const float* b_s, int64_t bs_row_stride, int64_t bs_col_stride, void* c, int64_t M, int64_t N,
-                              int64_t K, int out_dtype, void* stream) {
+                              int64_t K, int fmt, int out_dtype, void* stream) {
+    if (fmt != MDY_FMT_E4M3 && fmt != MDY_FMT_E5M2) return fail(MDY_E_DTYPE, "fp8_gemm_nt_rowscaled: unknown operand format %d", fmt);
     if (out_dtype != MDY_DT_BF16 && out_dtype != MDY_DT_F32) return fail(MDY_E_DTYPE, "fp8_gemm_nt_rowscaled: unknown out_dtype %d", out_dtype);
     if (M < 0 || N < 0 || K < 128 || K % 128 != 0 || M > kMaxDim || N > kMaxDim || K > (1 << 20))
         return fail(MDY_E_SHAPE, "fp8_gemm_nt_rowscaled: needs K a multiple of 128 up to 2^20 (M=%lld N=%lld K=%lld)", (long long)M,
@@ -175,7 +177,7 @@ int mdy_fp8_gemm_nt_rowscaled(const void* a, const float* a_s, int64_t as_row_st
         return fail(MDY_E_ALIGN, "fp8_gemm_nt_rowscaled: a and b must be 16-byte aligned, c and the scales aligned for their type");
     if (int e = check_device()) return e;
     const int rc = mdy::launch_fp8_gemm_nt_rowscaled(a, a_s, as_row_stride, as_col_stride, b, b_s, bs_row_stride, bs_col_stride, c,
-                                                     M, N, K, out_dtype, static_cast<hipStream_t>(stream));
+                                                     M, N, K, fmt, out_dtype, static_cast<hipStream_t>(stream));
     if (rc == -1) return fail(MDY_E_SHAPE, "fp8_gemm_nt_rowscaled: scale strides must be non-negative and span less than 2^31 bytes");
     return launched(rc, "fp8_gemm_nt_rowscaled");
 }
@@ -400,6 +402,14 @@ int mdy_cast_f32_to_e4m3(const float* x, void* y, int64_t n, int saturate, void*
     if (!x || !y) return fail(MDY_E_NULL, "cast_f32_to_e4m3: null pointer");
     if (int e = check_device()) return e;
     return launched(mdy::launch_cast_f32_to_e4m3(x, y, n, saturate, static_cast<hipStream_t>(stream)), "cast_f32_to_e4m3");
+}
+
+int mdy_cast_f32_to_e5m2(const float* x, void* y, int64_t n, void* stream) {
+    if (n < 0) return fail(MDY_E_SHAPE, "cast_f32_to_e5m2: n < 0");
+    if (n == 0) return 0;
+    if (!x || !y) return fail(MDY_E_NULL, "cast_f32_to_e5m2: null pointer");
+    if (int e = check_device()) return e;
+    return launched(mdy::launch_cast_f32_to_e5m2(x, y, n, static_cast<hipStream_t>(stream)), "cast_f32_to_e5m2");
 }
 
 int mdy_quotient_selfcheck(uint64_t* out, int amax_lo, int amax_hi, int mode, void* stream) {

@@ -11,7 +11,11 @@ typedef int intx4 __attribute__((ext_vector_type(4)));
 typedef int intx8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
-constexpr float kFp8Max = 448.0f;
+constexpr float kFp8Max = 448.0f;        // largest e4m3fn value
+constexpr float kBf8Max = 57344.0f;      // largest e5m2 value
+// Quantizer dialects (the MODE template parameter): 0 official (s = amax / 448, e4m3fn), 1 DeepLinear (clamp 1e4 + eps
+// 1e-8, saturating e4m3fn cast), 2 official with e5m2 bytes (s = amax / 57344: the default fp8 dtype of
+// /root/reference/triton_kernels/deepseekv3/fp8_kernel.py:62,124 is torch.float8_e5m2).
 constexpr int kGroup = 128;  // quantization group / block edge
 
 // Smallest biased exponent of amax for which the reciprocal + 2-FMA quotient is
@@ -29,6 +33,7 @@ __device__ __forceinline__ float bf16_one(uint16_t h) { return __uint_as_float((
 template <int MODE>
 __device__ __forceinline__ float group_scale(float amax) {
     if (MODE == 0) return amax / kFp8Max;
+    if (MODE == 2) return amax / kBf8Max;
     // clamp(amax, 0, 1e4) + 1e-8, NaN kept (fminf would drop it)
     float c = amax > 1e4f ? 1e4f : amax;
     return (c + 1e-8f) / kFp8Max;
@@ -38,6 +43,7 @@ __device__ __forceinline__ float group_scale(float amax) {
 template <int MODE>
 __device__ __forceinline__ bool fast_quotient_ok(float amax) {
     uint32_t b = __float_as_uint(amax);
+    if (MODE == 2) return false;            // the exhaustive proof covers e4m3fn bytes only
     if (MODE == 0) return b >= (kFastQuotientMinExp << 23) && b < 0x7F800000u;
     return b < 0x7F800000u;
 }
@@ -53,7 +59,7 @@ __device__ __forceinline__ float fast_quotient(float x, float s, float r) {
 template <int MODE>
 __device__ __forceinline__ float sat_for_mode(float q) {
     // v_med3_f32 returns a non-NaN operand for a NaN input, so keep NaN by hand.
-    if (MODE == 0) return q;
+    if (MODE != 1) return q;
     float c = __builtin_amdgcn_fmed3f(q, -kFp8Max, kFp8Max);
     return q != q ? q : c;
 }
@@ -64,6 +70,18 @@ __device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float 
     w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, w, false);
     w = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
     return (uint32_t)w;
+}
+
+// four fp32 -> four e5m2 bytes (RNE) packed little-endian into one dword
+__device__ __forceinline__ uint32_t pack4_e5m2(float a, float b, float c, float d) {
+    int w = 0;
+    w = __builtin_amdgcn_cvt_pk_bf8_f32(a, b, w, false);
+    w = __builtin_amdgcn_cvt_pk_bf8_f32(c, d, w, true);
+    return (uint32_t)w;
+}
+template <int MODE>
+__device__ __forceinline__ uint32_t pack4_fp8(float a, float b, float c, float d) {
+    return MODE == 2 ? pack4_e5m2(a, b, c, d) : pack4_e4m3(a, b, c, d);
 }
 
 // One lane's 8 values of a 128-element group with absmax `amax` -> 8 e4m3fn bytes and the group's scale: the
@@ -79,15 +97,15 @@ __device__ __forceinline__ uint2 quantize8_scaled(const float (&f)[8], float s, 
         for (int i = 0; i < 8; ++i) q[i] = sat_for_mode<MODE>(f[i] / s);
     }
     uint2 out;
-    out.x = pack4_e4m3(q[0], q[1], q[2], q[3]);
-    out.y = pack4_e4m3(q[4], q[5], q[6], q[7]);
+    out.x = pack4_fp8<MODE>(q[0], q[1], q[2], q[3]);
+    out.y = pack4_fp8<MODE>(q[4], q[5], q[6], q[7]);
     return out;
 }
 // True when a group with this absmax may take the reciprocal form in its dialect (the DeepLinear dialect also
 // needs |x / s| <= 448 without the saturating clamp, i.e. an absmax within the 1e4 clamp).
 template <int MODE>
 __device__ __forceinline__ bool group_is_fast(float amax) {
-    return MODE == 0 ? fast_quotient_ok<0>(amax) : (amax <= 1e4f);
+    return MODE == 0 ? fast_quotient_ok<0>(amax) : MODE == 2 ? false : (amax <= 1e4f);
 }
 template <int MODE>
 __device__ __forceinline__ uint2 quantize8(const float (&f)[8], float amax, float& scale_out) {
@@ -248,10 +266,10 @@ int launch_quant_transpose(const void* x, int x_dtype, void* y, float* s, void* 
                            int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int64_t s_kb_stride,
                            int t_mode, hipStream_t stream);
 int launch_act_quant_transpose(const void* x, int x_dtype, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
-                               int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, hipStream_t stream);
+                               int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int mode, hipStream_t stream);
 int launch_fp8_gemm_nt_rowscaled(const void* a, const float* a_s, int64_t as_rs, int64_t as_cs, const void* b,
                                  const float* b_s, int64_t bs_rs, int64_t bs_cs, void* c, int64_t M, int64_t N, int64_t K,
-                                 int out_dtype, hipStream_t stream);
+                                 int fmt, int out_dtype, hipStream_t stream);
 int launch_swiglu(const void* x, void* act, void* y, float* s, int64_t M, int64_t N, int64_t x_row_stride,
                   int gate_first, int64_t PM, int64_t PN, int64_t s_row_stride, int64_t s_col_stride, int mode,
                   hipStream_t stream);
@@ -284,6 +302,7 @@ int launch_group_pad(const void* x, void* y, const int64_t* m_splits, int64_t G,
 int launch_add_grad(void* x, const void* y, int64_t n, int x_dtype, int y_dtype, hipStream_t stream);
 int launch_add_bias(void* x, const void* b, int b_dtype, int64_t M, int64_t N, hipStream_t stream);
 int launch_cast_f32_to_e4m3(const float* x, void* y, int64_t n, int saturate, hipStream_t stream);
+int launch_cast_f32_to_e5m2(const float* x, void* y, int64_t n, hipStream_t stream);
 int launch_quotient_selfcheck(uint64_t* out, int amax_lo, int amax_hi, int mode, hipStream_t stream);
 
 }  // namespace mdy

@@ -15,7 +15,8 @@
 
 namespace mdy {
 
-template <typename OUT>
+// FMT: byte format of both operands, 0 e4m3fn, 1 e5m2 (the MFMA's cbsz / blgp operand-format fields).
+template <typename OUT, int FMT>
 __global__ __launch_bounds__(256) void fp8_gemm_rowscaled_kernel(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, int bs_rs, int bs_cs, uint32_t bs_bytes,
@@ -92,7 +93,8 @@ __global__ __launch_bounds__(256) void fp8_gemm_rowscaled_kernel(
             const float sa = lds_sa[buf][wm * 64 + i * 16 + frow];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const floatx4 p = mfma_block(fb[j], fa);
+                const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+                const floatx4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j], fa, zero, FMT, FMT, 0, 0, 0, 0);
                 acc[i][j][0] = __builtin_fmaf(p[0], sa * sbv[j][0], acc[i][j][0]);
                 acc[i][j][1] = __builtin_fmaf(p[1], sa * sbv[j][1], acc[i][j][1]);
                 acc[i][j][2] = __builtin_fmaf(p[2], sa * sbv[j][2], acc[i][j][2]);
@@ -118,7 +120,7 @@ __global__ __launch_bounds__(256) void fp8_gemm_rowscaled_kernel(
 // returns hipError_t, or -1 when the operands do not qualify (K % 128 != 0, misaligned, scale extents >= 2^31 bytes)
 int launch_fp8_gemm_nt_rowscaled(const void* a, const float* a_s, int64_t as_rs, int64_t as_cs, const void* b,
                                  const float* b_s, int64_t bs_rs, int64_t bs_cs, void* c, int64_t M, int64_t N, int64_t K,
-                                 int out_dtype, hipStream_t stream) {
+                                 int fmt, int out_dtype, hipStream_t stream) {
     if (M == 0 || N == 0) return 0;
     const int64_t KB = K / 128;
     const int64_t a_ext = ((M - 1) * as_rs + (KB - 1) * as_cs + 1) * 4, b_ext = ((N - 1) * bs_rs + (KB - 1) * bs_cs + 1) * 4;
@@ -129,14 +131,13 @@ int launch_fp8_gemm_nt_rowscaled(const void* a, const float* a_s, int64_t as_rs,
     const int tiles_m = (int)((M + 127) / 128), tiles_n = (int)((N + 127) / 128);
     if ((int64_t)tiles_m * tiles_n > 0x7FFFFFFF) return kErrTooManyBlocks;
     dim3 grid((unsigned)(tiles_m * tiles_n)), block(256);
-    if (out_dtype == 0)
-        hipLaunchKernelGGL(fp8_gemm_rowscaled_kernel<uint16_t>, grid, block, 0, stream, static_cast<const uint8_t*>(a), a_s,
-                           (int)as_rs, (int)as_cs, (uint32_t)a_ext, static_cast<const uint8_t*>(b), b_s, (int)bs_rs, (int)bs_cs,
-                           (uint32_t)b_ext, static_cast<uint16_t*>(c), (int)M, (int)N, (int)K, tiles_n);
-    else
-        hipLaunchKernelGGL(fp8_gemm_rowscaled_kernel<float>, grid, block, 0, stream, static_cast<const uint8_t*>(a), a_s,
-                           (int)as_rs, (int)as_cs, (uint32_t)a_ext, static_cast<const uint8_t*>(b), b_s, (int)bs_rs, (int)bs_cs,
-                           (uint32_t)b_ext, static_cast<float*>(c), (int)M, (int)N, (int)K, tiles_n);
+#define MDY_RS(OUT_T, FMT)                                                                                                 \
+    hipLaunchKernelGGL((fp8_gemm_rowscaled_kernel<OUT_T, FMT>), grid, block, 0, stream, static_cast<const uint8_t*>(a), a_s, \
+                       (int)as_rs, (int)as_cs, (uint32_t)a_ext, static_cast<const uint8_t*>(b), b_s, (int)bs_rs, (int)bs_cs, \
+                       (uint32_t)b_ext, static_cast<OUT_T*>(c), (int)M, (int)N, (int)K, tiles_n)
+    if (out_dtype == 0) { if (fmt == 0) MDY_RS(uint16_t, 0); else MDY_RS(uint16_t, 1); }
+    else { if (fmt == 0) MDY_RS(float, 0); else MDY_RS(float, 1); }
+#undef MDY_RS
     return (int)hipGetLastError();
 }
 

@@ -93,7 +93,7 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const void*
 #pragma unroll
             for (int j = 0; j < 8; ++j) q[j] = qt_quot<MODE, false>(f[i][j], sc, r);
         }
-        store_nt8(y + (int64_t)row * PK + c0, make_uint2(pack4_e4m3(q[0], q[1], q[2], q[3]), pack4_e4m3(q[4], q[5], q[6], q[7])));
+        store_nt8(y + (int64_t)row * PK + c0, make_uint2(pack4_fp8<MODE>(q[0], q[1], q[2], q[3]), pack4_fp8<MODE>(q[4], q[5], q[6], q[7])));
         if ((t & 15) == 0) row_sc[rg * RPT + i] = sc;
     }
 
@@ -162,8 +162,8 @@ __global__ __launch_bounds__(2048 / RPT) void quant_transpose_kernel(const void*
 #pragma unroll
             for (int j = 0; j < 8; ++j) q[j] = qt_quot<MODE, false>(f[i][j], tsc[j], tr[j]);
         }
-        qlo[i] = pack4_e4m3(q[0], q[1], q[2], q[3]);
-        qhi[i] = pack4_e4m3(q[4], q[5], q[6], q[7]);
+        qlo[i] = pack4_fp8<MODE>(q[0], q[1], q[2], q[3]);
+        qhi[i] = pack4_fp8<MODE>(q[4], q[5], q[6], q[7]);
     }
     // column j of the thread's RPT x 8 bytes = RPT consecutive bytes of row cl+j of the transposed tile
     if (RPT == 8) {
@@ -226,6 +226,7 @@ static int launch_qt(int mode, const void* x, int x_dtype, void* y, float* s, vo
 #define MDY_QT_V(MODE, TM, XT) do { if (vec) MDY_QT(MODE, TM, true, XT); else MDY_QT(MODE, TM, false, XT); } while (0)
 #define MDY_QT_X(MODE, TM) do { if (x_dtype == 0) MDY_QT_V(MODE, TM, 0); else if (x_dtype == 1) MDY_QT_V(MODE, TM, 1); else MDY_QT_V(MODE, TM, 2); } while (0)
     if (mode == 0) MDY_QT_X(0, 0);
+    else if (mode == 2) MDY_QT_X(2, 0);
     else if (t_mode == 0) MDY_QT_X(1, 0);
     else MDY_QT_X(1, 1);
 #undef MDY_QT_X
@@ -242,9 +243,9 @@ int launch_quant_transpose(const void* x, int x_dtype, void* y, float* s, void* 
 }
 
 int launch_act_quant_transpose(const void* x, int x_dtype, void* y, float* s, void* y_t, float* s_t, int64_t M, int64_t K,
-                               int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, hipStream_t stream) {
-    // official layouts, both row-major: s [PM][PK/128], s_t [PK][PM/128]
-    return launch_qt(0, x, x_dtype, y, s, y_t, s_t, M, K, x_row_stride, x_col_stride, PM, PK, 1, PK / 128, 1, PM / 128, 0, stream);
+                               int64_t x_row_stride, int64_t x_col_stride, int64_t PM, int64_t PK, int mode, hipStream_t stream) {
+    // official layouts, both row-major: s [PM][PK/128], s_t [PK][PM/128]; mode 0 (e4m3fn) or 2 (e5m2)
+    return launch_qt(mode == 2 ? 2 : 0, x, x_dtype, y, s, y_t, s_t, M, K, x_row_stride, x_col_stride, PM, PK, 1, PK / 128, 1, PM / 128, 0, stream);
 }
 
 }  // namespace mdy

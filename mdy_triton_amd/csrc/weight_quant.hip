@@ -113,7 +113,7 @@ int launch_weight_quant(const void* w, int w_dtype, void* y, float* s, void* y_t
                        (int)K, w_row_stride, w_col_stride, (int)PN, (int)PK)
 #define MDY_WQ_V(MODE, XT) do { if (vec) MDY_WQ(MODE, true, XT); else MDY_WQ(MODE, false, XT); } while (0)
 #define MDY_WQ_X(MODE) do { if (w_dtype == 0) MDY_WQ_V(MODE, 0); else if (w_dtype == 1) MDY_WQ_V(MODE, 1); else MDY_WQ_V(MODE, 2); } while (0)
-    if (mode == 0) MDY_WQ_X(0); else MDY_WQ_X(1);
+    if (mode == 0) MDY_WQ_X(0); else if (mode == 1) MDY_WQ_X(1); else MDY_WQ_X(2);
 #undef MDY_WQ_X
 #undef MDY_WQ_V
 #undef MDY_WQ

@@ -6,8 +6,10 @@ weight_quant_block (:124-138), plus silu_act_quant, which fuses the `silu_fwd ->
 pair of the FP8 MLP (fp8_kernel.py:447-450, 500-515) into one pass over the up/gate tensor; and for
 that file's own linear layer in the official dialect (s = amax / finfo.max, no clamp, no eps):
 act_quant_block (:62-87), fp8_matmul (:214-252), fp8_matmul_bwd (:254-257), Fp8Linear (:259-313).
-Only float8_e4m3fn is implemented (the reference defaults to e5m2 but its notebook passes
-e4m3fn, deepseekv3/fp8-benchmark.ipynb line 78).
+Both float8_e4m3fn and float8_e5m2 (the reference's default dtype, fp8_kernel.py:62, 124, 303) are implemented for the
+official-dialect functions; e4m3fn runs the tuned kernels, e5m2 the general quantizer kernels and the GEMM with row scales
+on both operands (a weight's 128x128 block scales are expanded to one per row for it).  The DeepLinear dialect and the
+fused silu_act_quant are e4m3fn only.
 """
 from typing import Optional, Tuple
 
@@ -18,10 +20,21 @@ from ._torch_glue import FP8, check, lib, on_device, ptr, require_gpu, stream_pt
 _ORDERS = ("up-gate", "gate-up")
 
 
+E5M2 = torch.float8_e5m2
+
+
 def _require_e4m3(fp8_dtype, who: str):
     if fp8_dtype != FP8:
-        raise TypeError("%s: only torch.float8_e4m3fn is implemented, got %s (the reference defaults to "
-                        "float8_e5m2; pass fp8_dtype=torch.float8_e4m3fn)" % (who, fp8_dtype))
+        raise TypeError("%s: only torch.float8_e4m3fn is implemented here, got %s" % (who, fp8_dtype))
+
+
+def _fp8_mode(fp8_dtype, who: str):
+    """(quantizer mode, GEMM operand format) of an fp8 dtype: official dialect with e4m3fn bytes, or with e5m2 bytes."""
+    if fp8_dtype == FP8:
+        return 0, 0
+    if fp8_dtype == E5M2:
+        return 2, 1
+    raise TypeError("%s: fp8 dtype must be torch.float8_e4m3fn or torch.float8_e5m2, got %s" % (who, fp8_dtype))
 
 
 def _flatten_up_gate(x: torch.Tensor, order: str, who: str):
@@ -119,16 +132,16 @@ def silu_act_quant(x: torch.Tensor, order: str = "up-gate", return_act: bool = F
 
 
 def weight_quant_block(x: torch.Tensor, BLOCK_M: int = 128, BLOCK_N: int = 128,
-                       dtype: torch.dtype = FP8) -> Tuple[torch.Tensor, torch.Tensor]:
-    """128x128 block quantizer with s = amax / 448 (fp8_kernel.py:124-138, kernel :88-122).
+                       dtype: torch.dtype = E5M2) -> Tuple[torch.Tensor, torch.Tensor]:
+    """128x128 block quantizer with s = amax / finfo(dtype).max (fp8_kernel.py:124-138, kernel :88-122); dtype
+    defaults to float8_e5m2 as in the reference.
 
-    x [M, N] bf16 with N % 128 == 0 (any strides); returns y [M, N] e4m3fn and s [M//128, N//128].
+    x [M, N] (any strides, N % 128 == 0); returns y [M, N] of `dtype` and s [M//128, N//128].
     """
     assert x.size(-1) % BLOCK_N == 0
     if BLOCK_M != 128 or BLOCK_N != 128:
         raise ValueError("only 128x128 blocks are implemented (the reference default)")
-    if dtype != FP8:
-        raise TypeError("only torch.float8_e4m3fn is implemented")
+    mode, _ = _fp8_mode(dtype, "weight_quant_block")
     if x.dim() != 2:
         raise TypeError("weight_quant_block expects a 2-D tensor")
     xt = xt_code(x, "weight_quant_block")
@@ -136,73 +149,98 @@ def weight_quant_block(x: torch.Tensor, BLOCK_M: int = 128, BLOCK_N: int = 128,
     M, N = x.shape
     if M % 128 != 0:
         raise ValueError("weight_quant_block: M must be a multiple of 128 (the reference drops the ragged rows)")
-    y = torch.empty(M, N, device=dev, dtype=FP8)
+    y = torch.empty(M, N, device=dev, dtype=dtype)
     s = torch.empty(M // 128, N // 128, device=dev, dtype=torch.float32)
     with on_device(dev):
-        check(lib().mdy_weight_quant_typed(ptr(x), xt, ptr(y), ptr(s), None, None, M, N, x.stride(0), x.stride(1), M, N, 0,
-                                     stream_ptr(dev)), "weight_quant_block")
+        check(lib().mdy_weight_quant_typed(ptr(x), xt, ptr(y), ptr(s), None, None, M, N, x.stride(0), x.stride(1), M, N, mode,
+                                           stream_ptr(dev)), "weight_quant_block")
     return y, s
 
 
-def _act_quant_transposed(x2: torch.Tensor, with_rows: bool, who: str):
-    """x2 [M, N] bf16 (any strides) -> (y, s, y_t_padded, s_t): the official-dialect row-wise quantization (None, None
+def _act_quant_transposed(x2: torch.Tensor, with_rows: bool, who: str, dtype: torch.dtype = FP8):
+    """x2 [M, N] (any strides) -> (y, s, y_t_padded, s_t): the official-dialect row-wise quantization (None, None
     unless with_rows) and the quantized transpose y_t [N, PM] with s_t [N, PM/128], PM = cdiv(M, 128) * 128."""
+    mode, _ = _fp8_mode(dtype, who)
     xt = xt_code(x2, who)
     dev = require_gpu(x2)
     M, N = x2.shape
     PM = (M + 127) // 128 * 128
-    y = torch.empty(PM, N, device=dev, dtype=FP8) if with_rows else None
+    y = torch.empty(PM, N, device=dev, dtype=dtype) if with_rows else None
     s = torch.empty(PM, N // 128, device=dev, dtype=torch.float32) if with_rows else None
-    y_t = torch.empty(N, PM, device=dev, dtype=FP8)
+    y_t = torch.empty(N, PM, device=dev, dtype=dtype)
     s_t = torch.empty(N, PM // 128, device=dev, dtype=torch.float32)
     if PM * N > 0:
         with on_device(dev):
             check(lib().mdy_act_quant_transpose(ptr(x2), xt, ptr(y), ptr(s), ptr(y_t), ptr(s_t), M, N, x2.stride(0), x2.stride(1),
-                                                PM, N, stream_ptr(dev)), who)
+                                                PM, N, mode, stream_ptr(dev)), who)
     return y, s, y_t, s_t
 
 
-def act_quant_block(x: torch.Tensor, transpose: bool = False, dtype: torch.dtype = FP8,
+def act_quant_block(x: torch.Tensor, transpose: bool = False, dtype: torch.dtype = E5M2,
                     BLOCK_N: int = 128) -> Tuple[torch.Tensor, torch.Tensor]:
-    """1x128 quantizer with s = amax / 448 (fp8_kernel.py:62-87).
+    """1x128 quantizer with s = amax / finfo(dtype).max (fp8_kernel.py:62-87); dtype defaults to float8_e5m2 as in the
+    reference.
 
-    transpose=False: (y like x, s [..., N/128]), the same as offical_kernel.act_quant.  transpose=True: the
-    flattened [M, N] input is quantized along M: y [N, M], s [N, cdiv(M, 128)] (a last group shorter than 128 is
-    completed with zeros, as the reference's masked loads do).
+    transpose=False: (y like x, s [..., N/128]); with float8_e4m3fn the same as offical_kernel.act_quant.
+    transpose=True: the flattened [M, N] input is quantized along M: y [N, M], s [N, cdiv(M, 128)] (a last group
+    shorter than 128 is completed with zeros, as the reference's masked loads do).
     """
     assert x.size(-1) % BLOCK_N == 0
     if BLOCK_N != 128:
         raise ValueError("only BLOCK_N=128 is implemented (the reference default)")
-    _require_e4m3(dtype, "act_quant_block")
+    mode, _ = _fp8_mode(dtype, "act_quant_block")
     if not transpose:
-        from .offical_kernel import act_quant
-        return act_quant(x if x.is_contiguous() else x.contiguous())
+        xc = x if x.is_contiguous() else x.contiguous()
+        if mode == 0:
+            from .offical_kernel import act_quant
+            return act_quant(xc)
+        xt = xt_code(xc, "act_quant_block")
+        dev = require_gpu(xc)
+        K = xc.size(-1)
+        M = xc.numel() // K if K else 0
+        y = torch.empty_like(xc, dtype=dtype)
+        s = xc.new_empty(*xc.size()[:-1], K // 128, dtype=torch.float32)
+        with on_device(dev):
+            check(lib().mdy_act_quant_typed(ptr(xc), xt, 128, ptr(y), ptr(s), M, K, K, M, K, K // 128, 1, mode, stream_ptr(dev)),
+                  "act_quant_block")
+        return y, s
     x2 = x.reshape(-1, x.size(-1))
     M = x2.size(0)
-    _, _, y_t, s_t = _act_quant_transposed(x2, False, "act_quant_block")
+    _, _, y_t, s_t = _act_quant_transposed(x2, False, "act_quant_block", dtype)
     return (y_t if y_t.size(1) == M else y_t[:, :M].contiguous()), s_t
 
 
 def fp8_matmul(x: torch.Tensor, w: torch.Tensor, scale_x: torch.Tensor, scale_w: torch.Tensor,
                bias: Optional[torch.Tensor] = None, have_w: bool = True) -> torch.Tensor:
-    """bf16 y = x . w^T on block-scaled FP8 operands (fp8_kernel.py:214-252).
+    """bf16 y = x . w^T on block-scaled FP8 operands, both float8_e4m3fn or both float8_e5m2 (fp8_kernel.py:214-252).
 
     have_w=True (forward, input gradient): x [..., K] with scale_x [..., K/128], w [N, K] with 128x128 block scales
     scale_w [N/128, K/128], optional bias [N] added in fp32.  have_w=False (weight gradient): x [M, K] and w [N, K]
     both carry one scale per row and 128 columns, scale_x [M, cdiv(K,128)], scale_w [N, cdiv(K,128)]; a K that is not a
     multiple of 128 is completed with zeros.
     """
-    if x.dtype != FP8 or w.dtype != FP8:
-        raise TypeError("fp8_matmul expects float8_e4m3fn operands")
+    if x.dtype != w.dtype:
+        raise TypeError("fp8_matmul expects operands of one fp8 dtype, got %s and %s" % (x.dtype, w.dtype))
+    _, fmt = _fp8_mode(x.dtype, "fp8_matmul")
     if have_w:
         assert x.size(-1) % 128 == 0, 'in forward x @ w.T'
-        from .offical_kernel import fp8_gemm
         x2 = x.reshape(-1, x.size(-1))
-        fused = bias is not None and bias.dtype == torch.bfloat16        # the GEMM epilogue takes a bf16 bias
-        y = fp8_gemm(x2 if x2.is_contiguous() else x2.contiguous(), scale_x.reshape(-1, scale_x.size(-1)).contiguous(),
-                     w if w.is_contiguous() else w.contiguous(), scale_w.contiguous(), out_dtype=torch.bfloat16,
-                     bias=bias.contiguous() if fused else None)
-        if bias is not None and not fused:                               # fp16 / fp32 bias: added in fp32 afterwards
+        sx2 = scale_x.reshape(-1, scale_x.size(-1))
+        if fmt == 0:
+            from .offical_kernel import fp8_gemm
+            fused = bias is not None and bias.dtype == torch.bfloat16        # the GEMM epilogue takes a bf16 bias
+            y = fp8_gemm(x2 if x2.is_contiguous() else x2.contiguous(), sx2.contiguous(),
+                         w if w.is_contiguous() else w.contiguous(), scale_w.contiguous(), out_dtype=torch.bfloat16,
+                         bias=bias.contiguous() if fused else None)
+        else:
+            # e5m2: the GEMM with row scales on both operands, the weight's block scales expanded to one per row
+            fused = False
+            dev = require_gpu(x, w, scale_x, scale_w)
+            M, K = x2.shape
+            N = w.size(0)
+            sw_rows = scale_w.repeat_interleave(128, dim=0)[:N].contiguous()
+            y = _matmul_rowscaled(x2, sx2, w, sw_rows, M, N, K, dev, fmt)
+        if bias is not None and not fused:                               # added in fp32 afterwards
             from .fp8 import add_bias
             add_bias(y, bias.contiguous())
         return y.view(*x.shape[:-1], w.size(0))
@@ -215,10 +253,10 @@ def fp8_matmul(x: torch.Tensor, w: torch.Tensor, scale_x: torch.Tensor, scale_w:
     if w.size(1) != K or tuple(scale_x.shape[-2:]) != (M, (K + 127) // 128) or tuple(scale_w.shape) != (N, (K + 127) // 128):
         raise ValueError("shape mismatch: x %s scale_x %s w %s scale_w %s" % (tuple(x.shape), tuple(scale_x.shape), tuple(w.shape),
                                                                                 tuple(scale_w.shape)))
-    return _matmul_rowscaled(x2, scale_x.reshape(M, -1), w, scale_w, M, N, K, dev)
+    return _matmul_rowscaled(x2, scale_x.reshape(M, -1), w, scale_w, M, N, K, dev, fmt)
 
 
-def _matmul_rowscaled(x2, sx, w, sw, M, N, K, dev):
+def _matmul_rowscaled(x2, sx, w, sw, M, N, K, dev, fmt=0):
     """[M, K] . [N, K]^T with per-row scales on both sides; operands may be column slices of K-padded buffers."""
     PK = (K + 127) // 128 * 128
 
@@ -227,14 +265,14 @@ def _matmul_rowscaled(x2, sx, w, sw, M, N, K, dev):
             return t
         full = torch.zeros(t.size(0), PK, device=dev, dtype=torch.uint8)
         full[:, :K] = t.view(torch.uint8)
-        return full.view(FP8)
+        return full
     a, b = k_padded(x2), k_padded(w)
     out = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
     if M * N == 0:
         return out
     with on_device(dev):
         check(lib().mdy_fp8_gemm_nt_rowscaled(ptr(a), ptr(sx), sx.stride(0), sx.stride(1), ptr(b), ptr(sw), sw.stride(0),
-                                              sw.stride(1), ptr(out), M, N, PK, 0, stream_ptr(dev)), "fp8_matmul")
+                                              sw.stride(1), ptr(out), M, N, PK, fmt, 0, stream_ptr(dev)), "fp8_matmul")
     return out
 
 
@@ -250,23 +288,24 @@ def _official_linear_backward(x2, w, dy2, need_dx, need_dw, fp8_dtype=FP8):
     and the block-quantized w^T, dw = dy^T . x on the transposed copies of dy and x (row scales on both operands).
     One kernel pass over dy gives both of its copies; the transposed copies keep their zero padding to a multiple of
     128 tokens."""
+    _, fmt = _fp8_mode(fp8_dtype, "Fp8Linear.backward")
     M, K = x2.shape
     N = w.size(0)
     dev = x2.device
     dx = dw = None
-    qdy, sdy, qdyt, sdyt = _act_quant_transposed(dy2, need_dx, "Fp8Linear.backward")
+    qdy, sdy, qdyt, sdyt = _act_quant_transposed(dy2, need_dx, "Fp8Linear.backward", fp8_dtype)
     if need_dx:
         qwt, swt = weight_quant_block(w.t(), dtype=fp8_dtype)       # [K, N]: the 128x128 blocks of w, transposed
         dx = fp8_matmul(qdy[:M], qwt, sdy[:M], swt, have_w=True)
     if need_dw:
-        _, _, qxt, sxt = _act_quant_transposed(x2, False, "Fp8Linear.backward")
+        _, _, qxt, sxt = _act_quant_transposed(x2, False, "Fp8Linear.backward", fp8_dtype)
         dw = torch.empty(N, K, device=dev, dtype=torch.bfloat16)
         if qdyt.size(1) == 0:
             dw.zero_()                                   # no tokens: an empty sum
         elif N * K > 0:
             with on_device(dev):
                 check(lib().mdy_fp8_gemm_nt_rowscaled(ptr(qdyt), ptr(sdyt), sdyt.stride(0), sdyt.stride(1), ptr(qxt), ptr(sxt),
-                                                      sxt.stride(0), sxt.stride(1), ptr(dw), N, K, qdyt.size(1), 0,
+                                                      sxt.stride(0), sxt.stride(1), ptr(dw), N, K, qdyt.size(1), fmt, 0,
                                                       stream_ptr(dev)), "Fp8Linear.backward")
     return dx, dw
 
@@ -279,7 +318,7 @@ class _Fp8LinearFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, w, bias, fp8_dtype):
-        _require_e4m3(fp8_dtype, "Fp8Linear")
+        _fp8_mode(fp8_dtype, "Fp8Linear")
         input_shape = x.shape
         x2 = x.reshape(-1, input_shape[-1])
         qx, sx = act_quant_block(x2, dtype=fp8_dtype)
@@ -306,12 +345,12 @@ fp8_linear_with_quant_ops = _Fp8LinearFunction.apply
 
 
 class Fp8Linear(torch.nn.Linear):
-    """nn.Linear on the official-dialect FP8 path (fp8_kernel.py:303-313).  Only float8_e4m3fn is implemented; the
-    reference's default, float8_e5m2, raises TypeError."""
+    """nn.Linear on the official-dialect FP8 path (fp8_kernel.py:303-313); fp8_dtype float8_e5m2 (the reference's
+    default) or float8_e4m3fn (what its notebook passes, and the faster one here)."""
 
-    def __init__(self, in_features, out_features, bias=True, device=None, dtype=None, fp8_dtype=FP8):
+    def __init__(self, in_features, out_features, bias=True, device=None, dtype=None, fp8_dtype=E5M2):
         super().__init__(in_features, out_features, bias, device, dtype)
-        _require_e4m3(fp8_dtype, "Fp8Linear")
+        _fp8_mode(fp8_dtype, "Fp8Linear")
         self.fp8_dtype = fp8_dtype
 
     def forward(self, x):
@@ -374,15 +413,18 @@ class _Fp8MlpCkptOfficial(torch.autograd.Function):
     forward (same bytes as silu_fwd + act_quant_block), x the only activation kept."""
 
     @staticmethod
-    def forward(ctx, x, w_up_gate, w_down, fp8_dtype=FP8, order="up-gate"):
-        _require_e4m3(fp8_dtype, "fp8_ckpt_mlp")
+    def forward(ctx, x, w_up_gate, w_down, fp8_dtype=E5M2, order="up-gate"):
+        mode, _ = _fp8_mode(fp8_dtype, "fp8_ckpt_mlp")
         shape = x.shape
         x2 = x.reshape(-1, shape[-1])
         qx, sx = act_quant_block(x2, dtype=fp8_dtype)
         qwu, swu = weight_quant_block(w_up_gate, dtype=fp8_dtype)
         qwd, swd = weight_quant_block(w_down, dtype=fp8_dtype)
         up_gate = fp8_matmul(qx, qwu, sx, swu)
-        qact, sact = silu_act_quant(up_gate, order, dialect="official")
+        if mode == 0:
+            qact, sact = silu_act_quant(up_gate, order, dialect="official")       # one pass, e4m3fn
+        else:
+            qact, sact = act_quant_block(silu_fwd(up_gate, order), dtype=fp8_dtype)
         y = fp8_matmul(qact, qwd, sact, swd)
         ctx.save_for_backward(x2, w_up_gate, w_down)
         ctx.order, ctx.shape, ctx.fp8_dtype = order, shape, fp8_dtype
@@ -404,11 +446,11 @@ class _Fp8MlpCkptOfficial(torch.autograd.Function):
         return dx.view(ctx.shape), dw_up_gate, dw_down, None, None
 
 
-def fp8_ckpt_mlp(x, w_up_gate, w_down, fp8_dtype=FP8, order="up-gate", dialect="official"):
-    """Memory-saving FP8 MLP step with the reference's positional order (fp8_kernel.py:436-494:
-    `fp8_ckpt_mlp(h, w1, w2, self.fp8_dtype, self.order)`).  Only float8_e4m3fn is implemented: the reference's
-    default, float8_e5m2, raises TypeError here.  dialect "official" (the reference's: s = amax / 448) or
-    "deeplinear" (clamp 1e4 + eps 1e-8, the quantizers of dpsk_fp8linear/fp8.py)."""
+def fp8_ckpt_mlp(x, w_up_gate, w_down, fp8_dtype=E5M2, order="up-gate", dialect="official"):
+    """Memory-saving FP8 MLP step with the reference's positional order and default dtype (fp8_kernel.py:436-494:
+    `fp8_ckpt_mlp(h, w1, w2, self.fp8_dtype, self.order)`).  dialect "official" (the reference's: s = amax /
+    finfo(fp8_dtype).max, float8_e5m2 or float8_e4m3fn) or "deeplinear" (clamp 1e4 + eps 1e-8, the quantizers of
+    dpsk_fp8linear/fp8.py; float8_e4m3fn only)."""
     if dialect == "official":
         return _Fp8MlpCkptOfficial.apply(x, w_up_gate, w_down, fp8_dtype, order)
     if dialect != "deeplinear":
@@ -418,20 +460,25 @@ def fp8_ckpt_mlp(x, w_up_gate, w_down, fp8_dtype=FP8, order="up-gate", dialect="
 
 class Fp8MLP(torch.nn.Module):
     """SwiGLU MLP on the FP8 linear path (fp8_kernel.py:500-515): up/gate projection, silu(gate) * up, down
-    projection, both projections block-wise FP8 (e4m3fn, 1x128 activation and 128x128 weight scales), no biases.
+    projection, both projections block-wise FP8 (1x128 activation and 128x128 weight scales), no biases.  fp8_dtype
+    float8_e5m2 (the reference's default) or float8_e4m3fn.
 
     dialect "official" (default, what the reference's Fp8MLP computes: its projections are `Fp8Linear`s,
-    s = amax / 448) or "deeplinear" (`DeepLinear` projections: clamp 1e4 + eps 1e-8, optional weight cache).
+    s = amax / finfo.max) or "deeplinear" (`DeepLinear` projections: clamp 1e4 + eps 1e-8, optional weight cache;
+    e4m3fn only).
     Without gradients the activation goes from the up/gate GEMM to the down GEMM through the fused
     SwiGLU + quantizer (one pass, the bf16 activation is never written).  With gradients the default is the
     composition linear -> triton_silu -> linear; `low_memory` (attribute or call argument, as in the
     reference) keeps only the input for the backward pass and recomputes up/gate and the activation there.
     """
 
-    def __init__(self, hidden_size, intermediate_size, order="up-gate", fp8_dtype=FP8, low_memory=False,
+    def __init__(self, hidden_size, intermediate_size, order="up-gate", fp8_dtype=E5M2, low_memory=False,
                  device=None, dtype=torch.bfloat16, dialect="official"):
         super().__init__()
-        _require_e4m3(fp8_dtype, "Fp8MLP")
+        if dialect == "deeplinear":
+            _require_e4m3(fp8_dtype, "Fp8MLP(dialect='deeplinear')")
+        else:
+            _fp8_mode(fp8_dtype, "Fp8MLP")
         assert order in _ORDERS, "please indicate the order of input, up-gate or gate-up"
         if dialect not in ("official", "deeplinear"):
             raise ValueError("dialect must be 'official' or 'deeplinear'")

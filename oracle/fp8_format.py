@@ -103,3 +103,58 @@ def f32_to_bf16_bits_rne(x: np.ndarray) -> np.ndarray:
     nan = np.isnan(x)
     r[nan] = ((bits[nan] >> np.uint64(16)).astype(np.uint16)) | np.uint16(0x0040)
     return r
+
+
+# ---------------------------------------------------------------------------
+# OCP FP8 E5M2: bit 7 sign, bits 6..2 exponent (bias 15), bits 1..0 mantissa; IEEE-like (the top byte of a binary16):
+#   exponent 0 -> subnormal, value = m * 2**-16; exponent 1..30 -> (1 + m/4) * 2**(e-15); exponent 31 -> inf (m = 0) / NaN.
+#   largest finite = 0x7B = 57344.
+# ---------------------------------------------------------------------------
+E5M2_MAX = 57344.0
+
+
+def decode_table_e5m2() -> np.ndarray:
+    """float32[256]: value of every e5m2 code."""
+    out = np.empty(256, dtype=np.float32)
+    for code in range(256):
+        sign = -1.0 if code & 0x80 else 1.0
+        e = (code >> 2) & 0x1F
+        m = code & 0x3
+        if e == 0x1F:
+            v = sign * float("inf") if m == 0 else float("nan")
+        elif e == 0:
+            v = sign * m * 2.0 ** -16
+        else:
+            v = sign * (1.0 + m / 4.0) * 2.0 ** (e - 15)
+        out[code] = v
+    return out
+
+
+_DECODE_E5M2 = decode_table_e5m2()
+
+
+def decode_e5m2(codes: np.ndarray) -> np.ndarray:
+    return _DECODE_E5M2[np.asarray(codes, dtype=np.uint8)]
+
+
+def encode_rne_e5m2(x: np.ndarray) -> np.ndarray:
+    """float32 -> uint8 e5m2 codes; round-to-nearest-even, overflow -> inf, NaN -> 0x7F (sign kept)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    bits = x.view(np.uint32)
+    sign = ((bits >> 24) & 0x80).astype(np.uint8)
+    mag = bits & np.uint32(0x7FFFFFFF)
+    out = np.empty(x.shape, dtype=np.uint8)
+    is_nan = mag > np.uint32(0x7F800000)
+    small = mag < np.uint32(0x38800000)            # 2**-14, the smallest normal e5m2
+    ax = np.abs(x.astype(np.float64))
+    sub_code = np.where(small, np.rint(ax * 65536.0), 0).astype(np.uint8)     # m = value / 2**-16, half-even; 4 carries into e = 1
+    lsb = (mag >> 21) & np.uint32(1)
+    rounded = (mag.astype(np.uint64) + np.uint64(0xFFFFF) + lsb.astype(np.uint64)) & np.uint64(0xFFE00000)
+    e32 = (rounded >> np.uint64(23)).astype(np.int64) - 127
+    m2 = ((rounded >> np.uint64(21)) & np.uint64(3)).astype(np.int64)
+    norm_code = ((e32 + 15) << 2) | m2
+    norm_code = np.where(norm_code >= 0x7C, 0x7C, norm_code)                  # rounded above 57344 (or was inf): inf
+    norm_code = np.clip(norm_code, 0, 0x7C).astype(np.uint8)
+    out[...] = np.where(small, sub_code, norm_code)
+    out[is_nan] = 0x7F
+    return out | sign

@@ -161,18 +161,18 @@ def fp8_gemm_blockwise(a, a_s, b, b_s, dtype: torch.dtype = torch.bfloat16) -> t
     return acc.to(dtype).reshape(*a.shape[:-1], N)
 
 
-def weight_quant_block(w: torch.Tensor, block_size: int = BLOCK) -> Tuple[torch.Tensor, torch.Tensor]:
-    """128x128 block quantizer without eps: s = max|blk| / 448 ; y = blk / s.
+def weight_quant_block(w: torch.Tensor, block_size: int = BLOCK, dtype: torch.dtype = FP8) -> Tuple[torch.Tensor, torch.Tensor]:
+    """128x128 block quantizer without eps: s = max|blk| / MAX ; y = blk / s.
 
     Follows triton_kernels/deepseekv3/fp8_kernel.py:117-122 with
-    MAX = finfo(e4m3fn).max (:133); this is how block-quantized test weights
-    are produced.  Requires both dims % 128 == 0 (U = M // BLOCK_M at :128-129).
+    MAX = finfo(dtype).max (:133: 448 for e4m3fn, 57344 for the reference's default e5m2); this is how
+    block-quantized test weights are produced.  Requires both dims % 128 == 0 (U = M // BLOCK_M at :128-129).
     """
     N, K = w.shape
     assert N % block_size == 0 and K % block_size == 0
     wf = w.detach().cpu().float().reshape(N // block_size, block_size, K // block_size, block_size)
-    s = wf.abs().amax(dim=(1, 3)) / FP8_MAX
-    y = (wf / s[:, None, :, None]).to(FP8).reshape(N, K)
+    s = wf.abs().amax(dim=(1, 3)) / torch.finfo(dtype).max
+    y = (wf / s[:, None, :, None]).to(dtype).reshape(N, K)
     return y, s
 
 
@@ -460,9 +460,9 @@ def fp8_unpadding(inp: torch.Tensor, m_splits, multiple: int = 256) -> torch.Ten
 # ---------------------------------------------------------------------------
 # The official-dialect linear layer of deepseekv3/fp8_kernel.py (Fp8Linear)
 # ---------------------------------------------------------------------------
-def act_quant_block(x: torch.Tensor, transpose: bool = False):
-    """fp8_kernel.py:62-87 (kernel :14-60): s = max|group| / 448 over 128 consecutive elements of a row, y = x / s
-    cast to e4m3fn, no clamp, no eps.  transpose=True quantizes x^T (the flattened [M, N] input along M); a last
+def act_quant_block(x: torch.Tensor, transpose: bool = False, dtype: torch.dtype = FP8):
+    """fp8_kernel.py:62-87 (kernel :14-60): s = max|group| / finfo(dtype).max over 128 consecutive elements of a row
+    (MAX at :82; 448 for e4m3fn, 57344 for e5m2), y = x / s cast to dtype, no clamp, no eps.  transpose=True quantizes x^T (the flattened [M, N] input along M); a last
     group shorter than 128 is completed with zeros (the kernel's boundary_check / padding_option='zero', :47-50).
     Returns (y, s): y like x and s [..., N/128], or y [N, M] and s [N, cdiv(M, 128)]."""
     x2 = x.detach().cpu().float().reshape(-1, x.shape[-1])
@@ -473,8 +473,8 @@ def act_quant_block(x: torch.Tensor, transpose: bool = False):
     xp = torch.zeros(R, PC, dtype=torch.float32)
     xp[:, :C] = x2
     g = xp.reshape(R, PC // BLOCK, BLOCK)
-    s = g.abs().amax(-1) / FP8_MAX
-    y = (g / s[:, :, None]).to(FP8).reshape(R, PC)[:, :C].contiguous()
+    s = g.abs().amax(-1) / torch.finfo(dtype).max
+    y = (g / s[:, :, None]).to(dtype).reshape(R, PC)[:, :C].contiguous()
     if transpose:
         return y, s
     return y.reshape(x.shape), s.reshape(*x.shape[:-1], PC // BLOCK)
@@ -500,23 +500,23 @@ def fp8_matmul_official(x, w, scale_x, scale_w, bias: Optional[torch.Tensor] = N
     return (deq(x, scale_x) @ deq(w, scale_w).t()).to(torch.bfloat16)
 
 
-def fp8_linear_forward(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+def fp8_linear_forward(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], dtype: torch.dtype = FP8) -> torch.Tensor:
     """_Fp8LinearFunction.forward (fp8_kernel.py:261-272)."""
     x2 = x.detach().cpu().reshape(-1, x.shape[-1])
-    qx, sx = act_quant_block(x2)
-    qw, sw = weight_quant_block(w.detach().cpu())
+    qx, sx = act_quant_block(x2, dtype=dtype)
+    qw, sw = weight_quant_block(w.detach().cpu(), dtype=dtype)
     return fp8_matmul_official(qx, qw, sx, sw, bias, True).reshape(*x.shape[:-1], -1)
 
 
-def fp8_linear_backward(x: torch.Tensor, w: torch.Tensor, dy: torch.Tensor, has_bias: bool = True):
+def fp8_linear_backward(x: torch.Tensor, w: torch.Tensor, dy: torch.Tensor, has_bias: bool = True, dtype: torch.dtype = FP8):
     """_Fp8LinearFunction.backward (fp8_kernel.py:274-301): (dx, dw, dbias)."""
     x2 = x.detach().cpu().reshape(-1, x.shape[-1])
     dy2 = dy.detach().cpu().reshape(-1, dy.shape[-1])
     dbias = dy2.sum(0) if has_bias else None
-    qxt, sxt = act_quant_block(x2, transpose=True)
-    qdy, sdy = act_quant_block(dy2)
-    qdyt, sdyt = act_quant_block(dy2, transpose=True)
-    qwt, swt = weight_quant_block(w.detach().cpu().t().contiguous())
+    qxt, sxt = act_quant_block(x2, transpose=True, dtype=dtype)
+    qdy, sdy = act_quant_block(dy2, dtype=dtype)
+    qdyt, sdyt = act_quant_block(dy2, transpose=True, dtype=dtype)
+    qwt, swt = weight_quant_block(w.detach().cpu().t().contiguous(), dtype=dtype)
     dx = fp8_matmul_official(qdy, qwt, sdy, swt, None, True)
     dw = fp8_matmul_official(qdyt, qxt, sdyt, sxt, None, False)
     return dx.reshape(x.shape), dw, dbias

@@ -85,3 +85,32 @@ def test_bf16_helpers():
     ref = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
     assert np.array_equal(F.f32_to_bf16_bits_rne(x), ref)
     assert np.array_equal(F.bf16_bits_to_f32(ref), torch.from_numpy(x).to(torch.bfloat16).float().numpy())
+
+
+def test_e5m2_codec_against_torch_cpu_cast():
+    """The from-definition e5m2 codec (the top byte of a binary16: 5 exponent bits, 2 mantissa bits, inf and NaN) and
+    torch's CPU cast pin each other: every code decodes alike, and every rounding midpoint with its fp32 neighbours,
+    the subnormal grid, the overflow edge (57344 | 61440 rounds to inf), signed zeros, inf and NaN encode alike."""
+    codes = np.arange(256, dtype=np.uint8)
+    vals = F.decode_e5m2(codes)
+    tvals = torch.from_numpy(codes).view(torch.float8_e5m2).float().numpy()
+    assert np.array_equal(np.isnan(vals), np.isnan(tvals)) and np.array_equal(vals[~np.isnan(vals)], tvals[~np.isnan(tvals)])
+    finite = np.sort(vals[np.isfinite(vals) & (vals >= 0)])
+    mids = (finite[:-1].astype(np.float64) + finite[1:].astype(np.float64)) / 2
+    pts = []
+    for v in np.concatenate([finite.astype(np.float64), mids]):
+        f = np.float32(v)
+        pts += [f, np.nextafter(f, np.float32(np.inf)), np.nextafter(f, np.float32(-np.inf))]
+    pts += [57344.0, 61439.0, 61440.0, 61441.0, 65536.0, 1e30, 2.0 ** -16, 2.0 ** -17, 1.5 * 2.0 ** -17, 2.0 ** -18, np.inf]
+    x = np.array(pts, dtype=np.float32)
+    x = np.concatenate([x, -x, np.array([np.nan], dtype=np.float32)])
+    rng = np.random.default_rng(3)
+    x = np.concatenate([x, (rng.standard_normal(500000) * 10.0 ** rng.integers(-6, 5, 500000)).astype(np.float32)])
+    mine = F.encode_rne_e5m2(x)
+    theirs = torch.from_numpy(x).to(torch.float8_e5m2).view(torch.uint8).numpy()
+    nan = np.isnan(x)
+    assert np.array_equal(mine[~nan], theirs[~nan])
+    assert np.all((mine[nan] & 0x7F) > 0x7C) and np.all((theirs[nan] & 0x7F) > 0x7C)
+    # round trip: every finite code encodes to itself
+    back = F.encode_rne_e5m2(vals[np.isfinite(vals)])
+    assert np.array_equal(back, codes[np.isfinite(vals)])

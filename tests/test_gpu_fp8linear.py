@@ -31,8 +31,8 @@ def test_act_quant_block_both_directions_bit_exact(M, N):
     x[min(3, M - 1), 5] = 300.0                      # an outlier sets one row group's and one column group's scale
     y_ref, s_ref = O.act_quant_block(x)
     yt_ref, st_ref = O.act_quant_block(x, transpose=True)
-    y, s = m.act_quant_block(x.to(DEV))
-    yt, st = m.act_quant_block(x.to(DEV), transpose=True)
+    y, s = m.act_quant_block(x.to(DEV), dtype=FP8)
+    yt, st = m.act_quant_block(x.to(DEV), transpose=True, dtype=FP8)
     assert y.shape == (M, N) and s.shape == (M, N // 128) and yt.shape == (N, M) and st.shape == (N, (M + 127) // 128)
     assert yt.is_contiguous() and st.is_contiguous()
     assert np.array_equal(u8(y), u8(y_ref)) and torch.equal(s.cpu(), s_ref)
@@ -42,7 +42,7 @@ def test_act_quant_block_both_directions_bit_exact(M, N):
     assert np.array_equal(u8(y2[:M]), u8(y_ref)) and torch.equal(s2[:M].cpu(), s_ref)
     assert np.array_equal(u8(yt2[:, :M]), u8(yt_ref)) and torch.equal(st2.cpu(), st_ref)
     wide = torch.randn(M, N + 64, generator=g).bfloat16().to(DEV)
-    yt3, st3 = m.act_quant_block(wide[:, 32:32 + N], transpose=True)
+    yt3, st3 = m.act_quant_block(wide[:, 32:32 + N], transpose=True, dtype=FP8)
     yt3_ref, st3_ref = O.act_quant_block(wide[:, 32:32 + N].cpu(), transpose=True)
     assert np.array_equal(u8(yt3), u8(yt3_ref)) and torch.equal(st3.cpu(), st3_ref)
 
@@ -50,16 +50,16 @@ def test_act_quant_block_both_directions_bit_exact(M, N):
 def test_act_quant_block_leading_dims_and_asserts():
     g = torch.Generator().manual_seed(2)
     x = torch.randn(2, 3, 64, 256, generator=g).bfloat16()
-    y, s = m.act_quant_block(x.to(DEV))
+    y, s = m.act_quant_block(x.to(DEV), dtype=FP8)
     yr, sr = O.act_quant_block(x)
     assert y.shape == x.shape and s.shape == (2, 3, 64, 2) and np.array_equal(u8(y), u8(yr)) and torch.equal(s.cpu(), sr)
-    yt, st = m.act_quant_block(x.to(DEV), transpose=True)
+    yt, st = m.act_quant_block(x.to(DEV), transpose=True, dtype=FP8)
     ytr, str_ = O.act_quant_block(x, transpose=True)
     assert yt.shape == (256, 384) and np.array_equal(u8(yt), u8(ytr)) and torch.equal(st.cpu(), str_)
     with pytest.raises(AssertionError):
         m.act_quant_block(torch.zeros(4, 100, device=DEV, dtype=torch.bfloat16))
     with pytest.raises(TypeError):
-        m.act_quant_block(x.to(DEV), dtype=torch.float8_e5m2)
+        m.act_quant_block(x.to(DEV), dtype=torch.float16)
 
 
 @pytest.mark.parametrize("M,N,K", [(128, 128, 128), (256, 384, 512), (130, 200, 384), (1000, 260, 1024), (64, 64, 2304)])
@@ -100,12 +100,14 @@ def test_rowscaled_gemm_random_and_ragged_k():
     L = _lib.load()
     one = torch.zeros(64, dtype=torch.uint8, device=DEV)
     p = one.data_ptr()
-    assert L.mdy_fp8_gemm_nt_rowscaled(p, p, 1, 1, p, p, 1, 1, p, 4, 4, 100, 0, None) == -2
-    assert L.mdy_fp8_gemm_nt_rowscaled(p + 1, p, 1, 1, p, p, 1, 1, p, 4, 4, 128, 0, None) == -3
-    assert L.mdy_fp8_gemm_nt_rowscaled(None, p, 1, 1, p, p, 1, 1, p, 4, 4, 128, 0, None) == -1
-    assert L.mdy_fp8_gemm_nt_rowscaled(p, p, -1, 1, p, p, 1, 1, p, 4, 4, 128, 0, None) == -2
-    assert L.mdy_act_quant_transpose(p, 0, None, p, p, p, 4, 128, 128, 1, 128, 128, None) == -1
-    assert L.mdy_act_quant_transpose(p, 7, p, p, p, p, 4, 128, 128, 1, 128, 128, None) == -4
+    assert L.mdy_fp8_gemm_nt_rowscaled(p, p, 1, 1, p, p, 1, 1, p, 4, 4, 100, 0, 0, None) == -2
+    assert L.mdy_fp8_gemm_nt_rowscaled(p + 1, p, 1, 1, p, p, 1, 1, p, 4, 4, 128, 0, 0, None) == -3
+    assert L.mdy_fp8_gemm_nt_rowscaled(None, p, 1, 1, p, p, 1, 1, p, 4, 4, 128, 0, 0, None) == -1
+    assert L.mdy_fp8_gemm_nt_rowscaled(p, p, -1, 1, p, p, 1, 1, p, 4, 4, 128, 0, 0, None) == -2
+    assert L.mdy_fp8_gemm_nt_rowscaled(p, p, 1, 1, p, p, 1, 1, p, 4, 4, 128, 5, 0, None) == -4
+    assert L.mdy_act_quant_transpose(p, 0, None, p, p, p, 4, 128, 128, 1, 128, 128, 0, None) == -1
+    assert L.mdy_act_quant_transpose(p, 7, p, p, p, p, 4, 128, 128, 1, 128, 128, 0, None)
+    assert L.mdy_act_quant_transpose(p, 0, p, p, p, p, 4, 128, 128, 1, 128, 128, 1, None) == -4 == -4
 
 
 @pytest.mark.parametrize("bias", [True, False])
@@ -147,18 +149,18 @@ def test_fp8_linear_forward_backward(shape, N, bias):
     lin(xg2).backward(dy.to(DEV))
     assert close(xg2.grad, ref_dx)
     with pytest.raises(TypeError, match="float8_e4m3fn"):
-        m.Fp8Linear(K, N, dtype=torch.bfloat16, fp8_dtype=torch.float8_e5m2)
+        m.Fp8Linear(K, N, dtype=torch.bfloat16, fp8_dtype=torch.bfloat16)
 
 
 def test_fp8_linear_without_tokens():
     """An empty batch: empty output, zero weight gradient, empty input gradient (no kernel is given a zero extent)."""
-    lin = m.Fp8Linear(256, 128, bias=True, dtype=torch.bfloat16, device=DEV)
+    lin = m.Fp8Linear(256, 128, bias=True, dtype=torch.bfloat16, device=DEV, fp8_dtype=FP8)
     x = torch.zeros(0, 256, device=DEV, dtype=torch.bfloat16, requires_grad=True)
     out = lin(x)
     assert out.shape == (0, 128)
     out.sum().backward()
     assert x.grad.shape == (0, 256) and torch.count_nonzero(lin.weight.grad) == 0 and torch.count_nonzero(lin.bias.grad) == 0
-    yt, st = m.act_quant_block(x.detach(), transpose=True)
+    yt, st = m.act_quant_block(x.detach(), transpose=True, dtype=FP8)
     assert yt.shape == (256, 0) and st.shape == (256, 0)
 
 
@@ -174,8 +176,8 @@ def test_act_quant_block_non_finite_and_zero_groups():
     x[7, 128:256] = 0.0                   # row group (7, 1) all zero
     x[200, 17] = float("inf")
     x[130, 140] = float("nan")
-    y, s = m.act_quant_block(x.to(DEV))
-    yt, st = m.act_quant_block(x.to(DEV), transpose=True)
+    y, s = m.act_quant_block(x.to(DEV), dtype=FP8)
+    yt, st = m.act_quant_block(x.to(DEV), transpose=True, dtype=FP8)
     xz = torch.where(torch.isnan(x), torch.zeros_like(x), x)
     yr, sr = O.act_quant_block(xz)
     ytr, str_ = O.act_quant_block(xz, transpose=True)
@@ -214,7 +216,7 @@ def test_rowscaled_gemm_non_finite_values():
     from mdy_triton_amd import _lib
     ad, bd, sad, sbd = a.to(DEV), b.to(DEV), sa.to(DEV), sb.to(DEV)
     rc = _lib.load().mdy_fp8_gemm_nt_rowscaled(ad.data_ptr(), sad.data_ptr(), 3, 1, bd.data_ptr(), sbd.data_ptr(), 3, 1,
-                                                out.data_ptr(), M, N, K, 1, None)
+                                                out.data_ptr(), M, N, K, 0, 1, None)
     torch.cuda.synchronize()
     assert rc == 0
     got = out.cpu()
@@ -256,3 +258,136 @@ def test_fp8_linear_reproduces_the_reference_notebook_error_magnitudes():
     assert 0.94 * 0.0095 < gmean < 1.06 * 0.0095 and 0.5 * 0.0669 < gmax < 2 * 0.0669, (gmax, gmean)
     assert 0.94 * 2.11 < wmean < 1.06 * 2.11 and 0.5 * 14.0 < wmax < 2 * 14.0, (wmax, wmean)
     assert torch.allclose(fc1.bias.grad, fc2.bias.grad)
+
+
+# ------------------------------------------------------------------ float8_e5m2: the reference's default fp8 dtype
+E5M2 = torch.float8_e5m2
+
+
+def test_e5m2_device_cast_matches_the_codec():
+    """v_cvt_pk_bf8_f32 against the from-definition e5m2 codec on every code's neighbourhood and random values."""
+    from oracle import fp8_format as F
+    from mdy_triton_amd import _lib
+    vals = F.decode_e5m2(np.arange(256, dtype=np.uint8))
+    finite = np.sort(vals[np.isfinite(vals) & (vals >= 0)]).astype(np.float64)
+    mids = (finite[:-1] + finite[1:]) / 2
+    pts = []
+    for v in np.concatenate([finite, mids]):
+        f = np.float32(v)
+        pts += [f, np.nextafter(f, np.float32(np.inf)), np.nextafter(f, np.float32(-np.inf))]
+    x = np.array(pts + [61439.0, 61440.0, 65536.0, 1e30], dtype=np.float32)
+    rng = np.random.default_rng(1)
+    x = np.concatenate([x, -x, (rng.standard_normal(200000) * 10.0 ** rng.integers(-6, 5, 200000)).astype(np.float32)])
+    xt = torch.from_numpy(x).to(DEV)
+    y = torch.empty(x.size, dtype=torch.uint8, device=DEV)
+    _lib.check(_lib.load().mdy_cast_f32_to_e5m2(xt.data_ptr(), y.data_ptr(), x.size, None), "cast")
+    assert np.array_equal(y.cpu().numpy(), F.encode_rne_e5m2(x))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_e5m2_quantizers_bit_exact(dtype):
+    """act_quant_block (both directions) and weight_quant_block with the reference's DEFAULT dtype, float8_e5m2
+    (fp8_kernel.py:62, 124): s = amax / 57344, bytes and scales bit-exact against the oracle."""
+    g = torch.Generator().manual_seed(11)
+    x = (torch.randn(200, 384, generator=g) * 3).to(dtype)
+    y, s = m.act_quant_block(x.to(DEV))                      # default dtype
+    yr, sr = O.act_quant_block(x, dtype=E5M2)
+    assert y.dtype == E5M2 and np.array_equal(u8(y), u8(yr)) and torch.equal(s.cpu(), sr)
+    assert float(y.float().abs().max()) == 57344.0           # every group's largest element maps to the format's maximum
+    yt, st = m.act_quant_block(x.to(DEV), transpose=True)
+    ytr, str_ = O.act_quant_block(x, transpose=True, dtype=E5M2)
+    assert yt.dtype == E5M2 and yt.shape == (384, 200) and np.array_equal(u8(yt), u8(ytr)) and torch.equal(st.cpu(), str_)
+    w = (torch.randn(256, 384, generator=g) * 0.02).to(dtype)
+    wq, ws = m.weight_quant_block(w.to(DEV))                 # default dtype
+    wqr, wsr = O.weight_quant_block(w, dtype=E5M2)
+    assert wq.dtype == E5M2 and np.array_equal(u8(wq), u8(wqr)) and torch.equal(ws.cpu(), wsr)
+    wq4, _ = m.weight_quant_block(w.to(DEV), dtype=FP8)
+    assert wq4.dtype == FP8
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 256, 256), (130, 200, 384), (256, 384, 1024)])
+def test_e5m2_gemms_exact_integer(M, N, K):
+    """e5m2 operands through both GEMM forms of fp8_kernel.fp8_matmul (block-scaled weight: its scales expanded to one
+    per row; row scales on both sides): integer operands and power-of-two scales are exact, so the result must equal
+    the float64 computation rounded once to bf16."""
+    g = torch.Generator().manual_seed(M + K)
+    ai = torch.randint(-4, 5, (M, K), generator=g)
+    bi = torch.randint(-4, 5, (N, K), generator=g)
+    KB, NB = K // 128, (N + 127) // 128
+    ea = torch.randint(-2, 3, (M, KB), generator=g)
+    eb_blk = torch.randint(-2, 3, (NB, KB), generator=g)
+    eb_row = torch.randint(-2, 3, (N, KB), generator=g)
+    a, b = ai.float().to(E5M2).to(DEV), bi.float().to(E5M2).to(DEV)
+    for have_w, eb in ((True, eb_blk), (False, eb_row)):
+        if not have_w and M % 128:
+            continue
+        exact = torch.zeros(M, N, dtype=torch.float64)
+        for kb in range(KB):
+            sbn = eb[torch.arange(N) // 128, kb] if have_w else eb[:, kb]
+            exact += (ai[:, kb * 128:(kb + 1) * 128].double() @ bi[:, kb * 128:(kb + 1) * 128].double().t()) * \
+                torch.exp2((ea[:, kb][:, None] + sbn[None, :]).double())
+        got = FK.fp8_matmul(a, b, torch.exp2(ea.float()).to(DEV), torch.exp2(eb.float()).to(DEV), have_w=have_w)
+        assert torch.equal(got.cpu().double(), exact.to(torch.bfloat16).double()), have_w
+    with pytest.raises(TypeError):
+        FK.fp8_matmul(a, b.view(torch.uint8).view(FP8), torch.exp2(ea.float()).to(DEV), torch.exp2(eb_blk.float()).to(DEV))
+
+
+@pytest.mark.parametrize("bias", [True, False])
+def test_fp8_linear_e5m2_default(bias):
+    """Fp8Linear as the reference constructs it by default (fp8_dtype = float8_e5m2): forward and all gradients within the
+    GEMM tolerance of the oracle computing in e5m2."""
+    g = torch.Generator().manual_seed(31)
+    shape, N = (3, 100, 512), 384
+    K = shape[-1]
+    w = (torch.randn(N, K, generator=g) * 0.02).bfloat16()
+    b = torch.randn(N, generator=g).bfloat16() if bias else None
+    x = torch.randn(*shape, generator=g).bfloat16()
+    dy = torch.randn(*shape[:-1], N, generator=g).bfloat16()
+    ref_out = O.fp8_linear_forward(x, w, b, dtype=E5M2)
+    ref_dx, ref_dw, ref_db = O.fp8_linear_backward(x, w, dy, bias, dtype=E5M2)
+    lin = m.Fp8Linear(K, N, bias=bias, dtype=torch.bfloat16)
+    assert lin.fp8_dtype == E5M2
+    with torch.no_grad():
+        lin.weight.copy_(w)
+        if bias:
+            lin.bias.copy_(b)
+    lin = lin.to(DEV)
+    xg = x.to(DEV).requires_grad_(True)
+    out = lin(xg)
+    out.backward(dy.to(DEV))
+    if bias:
+        mag = torch.maximum(ref_out.float().abs(), (ref_out.float() - b.float()).abs())
+        assert bool(((out.float().cpu() - ref_out.float()).abs() <= 2e-2 + 1e-2 * mag).all())
+    else:
+        assert close(out, ref_out)
+    assert close(xg.grad, ref_dx) and close(lin.weight.grad, ref_dw)
+    if bias:
+        assert torch.allclose(lin.bias.grad.float().cpu(), ref_db.float(), rtol=1e-2, atol=1e-2)
+
+
+def test_fp8_mlp_e5m2_default_paths_agree():
+    """Fp8MLP with the reference's defaults (Fp8Linear projections, float8_e5m2): the three execution paths agree bit for
+    bit, and the no-gradient result is within the GEMM tolerance of the oracle's composition stage by stage."""
+    g = torch.Generator().manual_seed(41)
+    H, inter = 256, 384
+    x = torch.randn(64, H, generator=g).bfloat16()
+    dy = torch.randn(64, H, generator=g).bfloat16()
+    mlp = m.Fp8MLP(H, inter, device=DEV)
+    assert mlp.fp8_dtype == E5M2 and mlp.up_gate_proj.fp8_dtype == E5M2
+    outs = []
+    for low in (False, True):
+        mlp.zero_grad()
+        xg = x.to(DEV).requires_grad_(True)
+        y = mlp(xg, low_memory=low)
+        y.backward(dy.to(DEV))
+        outs.append((y.detach(), xg.grad, mlp.up_gate_proj.weight.grad.clone(), mlp.down_proj.weight.grad.clone()))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    with torch.no_grad():
+        y0 = mlp(x.to(DEV))
+        assert torch.equal(y0, outs[0][0])
+        assert torch.equal(m.fp8_ckpt_mlp(x.to(DEV), mlp.up_gate_proj.weight, mlp.down_proj.weight), y0)   # reference defaults
+        ug = mlp.up_gate_proj(x.to(DEV))
+    assert close(ug, O.fp8_linear_forward(x, mlp.up_gate_proj.weight.detach().cpu(), None, dtype=E5M2))
+    act = O.silu_fwd(ug.cpu(), "up-gate")
+    assert close(y0, O.fp8_linear_forward(act, mlp.down_proj.weight.detach().cpu(), None, dtype=E5M2))

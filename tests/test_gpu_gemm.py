@@ -531,7 +531,7 @@ def test_deep_linear_cache_and_data_updates():
 
 
 def test_fp8_mlp_sees_data_updates_after_invalidation():
-    mlp = m.Fp8MLP(256, 256, device=DEV, dialect="deeplinear")
+    mlp = m.Fp8MLP(256, 256, device=DEV, dialect="deeplinear", fp8_dtype=torch.float8_e4m3fn)
     mlp.up_gate_proj.cache_weight = mlp.down_proj.cache_weight = True
     x = torch.randn(16, 256, device=DEV).bfloat16()
     with torch.no_grad():

@@ -33,7 +33,7 @@ def test_mlp_step_replays_bit_identically(M):
     with torch.no_grad():
         lin_in.weight.copy_(bf16(F, K, 1, 0.05))
         lin_in.bias.copy_(bf16(1, F, 2)[0])
-    w_down_q, w_down_s = m.weight_quant_block(bf16(K, F // 2, 3, 0.05))
+    w_down_q, w_down_s = m.weight_quant_block(bf16(K, F // 2, 3, 0.05), dtype=torch.float8_e4m3fn)
     inputs = [bf16(M, K, 10 + i) for i in range(4)]
     with torch.no_grad():
         eager = [mlp_step(x, lin_in, w_down_q, w_down_s).clone() for x in inputs]

@@ -77,7 +77,7 @@ def test_training_quantizers_beyond_2g_elements(x_big):
 
 def test_weight_quant_and_dequant_beyond_2g_elements(x_big):
     w = x_big                                              # any bf16 matrix with 128-aligned sides
-    y, s = m.weight_quant_block(w)
+    y, s = m.weight_quant_block(w, dtype=torch.float8_e4m3fn)
     assert s.shape == (M_BIG // 128, K_BIG // 128)
     for r in slabs(M_BIG, 32768):
         yr, sr = O.weight_quant_block(w[r:r + H].cpu())
@@ -195,7 +195,7 @@ def test_training_quantizers_with_more_than_65535_tile_rows():
         assert np.array_equal(u8(y_t[:, r:r + H]), u8(ytr)), r
         assert torch.equal(s_t[:, r // 128:(r + H) // 128].cpu(), str_), r
     del y, s, y_t, s_t
-    wq, ws = m.weight_quant_block(x)
+    wq, ws = m.weight_quant_block(x, dtype=torch.float8_e4m3fn)
     for r in slabs(M, M // 2):
         yr, sr = O.weight_quant_block(x[r:r + H].cpu())
         assert np.array_equal(u8(wq[r:r + H]), u8(yr)) and torch.equal(ws[r // 128:(r + H) // 128].cpu(), sr), r

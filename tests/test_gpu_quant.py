@@ -487,10 +487,10 @@ def test_weight_and_training_quantizers_fp16_fp32_inputs(dtype):
             if a is not None:
                 assert torch.equal(a.cpu().contiguous().view(torch.uint8) if a.dtype == FP8 else a.cpu(), b.contiguous().view(torch.uint8) if b.dtype == FP8 else b)
     wb = (torch.randn(256, 384, generator=g) * 0.02).to(dtype)
-    y, s = m.weight_quant_block(wb.to(DEV))
+    y, s = m.weight_quant_block(wb.to(DEV), dtype=FP8)
     yr, sr = O.weight_quant_block(wb)
     assert torch.equal(y.cpu().view(torch.uint8), yr.view(torch.uint8)) and torch.equal(s.cpu(), sr)
-    yt, st = m.weight_quant_block(wb.to(DEV).t())                   # strided (transposed view)
+    yt, st = m.weight_quant_block(wb.to(DEV).t(), dtype=FP8)                   # strided (transposed view)
     ytr, str_ = O.weight_quant_block(wb.t().contiguous())
     assert torch.equal(yt.cpu().view(torch.uint8), ytr.view(torch.uint8)) and torch.equal(st.cpu(), str_)
     x = torch.randn(300, 512, generator=g).to(dtype)
@@ -499,7 +499,7 @@ def test_weight_and_training_quantizers_fp16_fp32_inputs(dtype):
         for a, b in zip(fn(x.to(DEV)), ofn(x)):
             a, b = a.cpu().contiguous(), b.contiguous()
             assert a.shape == b.shape and torch.equal(a.view(torch.uint8) if a.dtype == FP8 else a, b.view(torch.uint8) if b.dtype == FP8 else b)
-    yb, sb = m.act_quant_block(x.to(DEV), transpose=True)
+    yb, sb = m.act_quant_block(x.to(DEV), transpose=True, dtype=FP8)
     ybr, sbr = O.act_quant_block(x, transpose=True)
     assert torch.equal(yb.cpu().view(torch.uint8), ybr.view(torch.uint8)) and torch.equal(sb.cpu(), sbr)
     q = m.per_block_cast_to_fp8([w.to(DEV), (w * 2).to(DEV)], output_transpose=True)
@@ -531,7 +531,7 @@ def test_deep_linear_and_fp8_linear_with_fp32_parameters():
     got = m.add_bias(nb.clone().to(DEV), bias.to(DEV))
     assert torch.equal(got.cpu(), (nb.float() + bias).bfloat16())
     with torch.no_grad():
-        fl = m.Fp8Linear(512, 256, bias=True)
+        fl = m.Fp8Linear(512, 256, bias=True, fp8_dtype=FP8)
         fl.weight.copy_(lin.weight.cpu()); fl.bias.copy_(lin.bias.cpu())
         ref2 = O.fp8_linear_forward(x, fl.weight.detach(), None).float() + fl.bias.detach()
         out2 = fl.to(DEV)(x.to(DEV))

@@ -136,7 +136,7 @@ def test_fp8_mlp_three_paths(shape, inter, order):
     w_d = (torch.randn(H, inter, generator=g) * 0.03).bfloat16()
     dy = torch.randn(*shape, generator=g).bfloat16()
 
-    mlp = m.Fp8MLP(H, inter, order=order, device=DEV, dialect="deeplinear")
+    mlp = m.Fp8MLP(H, inter, order=order, device=DEV, dialect="deeplinear", fp8_dtype=torch.float8_e4m3fn)
     up, down = mlp.up_gate_proj, mlp.down_proj
     with torch.no_grad():
         up.weight.copy_(w_ug)
@@ -193,18 +193,20 @@ def test_fp8_ckpt_mlp_reference_call_order():
     x = torch.randn(32, H, generator=g).bfloat16().to(DEV)
     w_ug = (torch.randn(2 * inter, H, generator=g) * 0.03).bfloat16().to(DEV)
     w_d = (torch.randn(H, inter, generator=g) * 0.03).bfloat16().to(DEV)
-    mlp = m.Fp8MLP(H, inter, order="gate-up", device=DEV, dialect="deeplinear")
+    mlp = m.Fp8MLP(H, inter, order="gate-up", device=DEV, dialect="deeplinear", fp8_dtype=torch.float8_e4m3fn)
     with torch.no_grad():
         mlp.up_gate_proj.weight.copy_(w_ug)
         mlp.down_proj.weight.copy_(w_d)
         want = mlp(x)
         got = m.fp8_ckpt_mlp(x, w_ug, w_d, torch.float8_e4m3fn, "gate-up", dialect="deeplinear")
         assert torch.equal(got, want)
-        assert torch.equal(m.fp8_ckpt_mlp(x, w_ug, w_d, order="gate-up", dialect="deeplinear"), want)
+        assert torch.equal(m.fp8_ckpt_mlp(x, w_ug, w_d, fp8_dtype=torch.float8_e4m3fn, order="gate-up", dialect="deeplinear"), want)
         with pytest.raises(TypeError, match="float8_e4m3fn"):
-            m.fp8_ckpt_mlp(x, w_ug, w_d, torch.float8_e5m2, "gate-up")
+            m.fp8_ckpt_mlp(x, w_ug, w_d, torch.float8_e5m2, "gate-up", dialect="deeplinear")      # the DeepLinear dialect is e4m3fn only
         with pytest.raises(TypeError, match="float8_e4m3fn"):
-            m.Fp8MLP(H, inter, fp8_dtype=torch.float8_e5m2, device=DEV)
+            m.Fp8MLP(H, inter, fp8_dtype=torch.float8_e5m2, device=DEV, dialect="deeplinear")
+        with pytest.raises(TypeError, match="float8_e4m3fn"):
+            m.Fp8MLP(H, inter, fp8_dtype=torch.float16, device=DEV)
 
 
 @pytest.mark.parametrize("order", ["up-gate", "gate-up"])
@@ -218,7 +220,7 @@ def test_fp8_mlp_official_dialect_three_paths(order):
     w_ug = (torch.randn(2 * inter, H, generator=g) * 0.03).bfloat16()
     w_d = (torch.randn(H, inter, generator=g) * 0.03).bfloat16()
     dy = torch.randn(*shape, generator=g).bfloat16()
-    mlp = m.Fp8MLP(H, inter, order=order, device=DEV)
+    mlp = m.Fp8MLP(H, inter, order=order, device=DEV, fp8_dtype=torch.float8_e4m3fn)
     assert mlp.dialect == "official" and isinstance(mlp.up_gate_proj, m.Fp8Linear)
     up, down = mlp.up_gate_proj, mlp.down_proj
     with torch.no_grad():
