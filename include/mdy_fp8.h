@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define MDY_FP8_ABI_VERSION 13
+#define MDY_FP8_ABI_VERSION 14
 
 /* error codes (negative = argument rejected before any launch) */
 #define MDY_OK 0
@@ -226,6 +226,14 @@ int mdy_weight_dequant_block(const void* x, const float* s, void* y, int64_t N, 
 int mdy_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
                     const void* b, const float* b_s, void* c, const void* bias, int64_t M, int64_t N,
                     int64_t K, int out_dtype, void* stream);
+
+/* mdy_fp8_gemm_nt on float8_e5m2 operands (the default fp8 dtype of triton_kernels/deepseekv3/fp8_kernel.py): the MFMA tile
+ * kernels with the instruction's operand format set to bf8.  Same arguments and formula; only problems with more than 64
+ * rows, K % 128 == 0, K <= 65536 and 16-byte aligned a / b (MDY_E_SHAPE otherwise: run those through
+ * mdy_fp8_gemm_nt_rowscaled with the weight's block scales expanded to one per row, as the Python wrapper does). */
+int mdy_fp8_gemm_nt_e5m2(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,
+                         const float* b_s, void* c, const void* bias, int64_t M, int64_t N, int64_t K, int out_dtype,
+                         void* stream);
 
 /* The same GEMM with a caller-provided scratch buffer.  Shapes whose output tiles do not fill the GPU
  * (roughly 32 < M <= 1024 against a long K: small-batch prefill, large-batch decode) are cut along K as

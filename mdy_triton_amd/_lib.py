@@ -10,7 +10,7 @@ import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libmdyfp8.so")
-ABI_VERSION = 13
+ABI_VERSION = 14
 
 _lock = threading.Lock()
 _lib = None
@@ -35,6 +35,7 @@ SIGNATURES = {
     "mdy_weight_dequant": [_p, _p, _p, _i64, _i64, _int, _p],
     "mdy_weight_dequant_block": [_p, _p, _p, _i64, _i64, _int, _int, _p],
     "mdy_fp8_gemm_nt": [_p, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p],
+    "mdy_fp8_gemm_nt_e5m2": [_p, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p],
     "mdy_fp8_gemm_nt_ws": [_p, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p, _i64, _p],
     "mdy_fp8_gemm_workspace_bytes": [_i64, _i64, _i64],
     "mdy_fp8_gemm_probe": [_int, _int, _p, _p, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _p],

@@ -249,6 +249,25 @@ int mdy_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int6
                     "fp8_gemm_nt");
 }
 
+int mdy_fp8_gemm_nt_e5m2(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,
+                         const float* b_s, void* c, const void* bias, int64_t M, int64_t N, int64_t K, int out_dtype,
+                         void* stream) {
+    if (out_dtype != MDY_DT_BF16 && out_dtype != MDY_DT_F32) return fail(MDY_E_DTYPE, "fp8_gemm_nt_e5m2: unknown out_dtype %d", out_dtype);
+    if (M < 0 || N < 0 || K < 1 || M > kMaxDim || N > kMaxDim || K > kMaxDim)
+        return fail(MDY_E_SHAPE, "fp8_gemm_nt_e5m2: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+    if (M == 0 || N == 0) return 0;
+    if (!a || !a_s || !b || !b_s || !c) return fail(MDY_E_NULL, "fp8_gemm_nt_e5m2: null pointer");
+    if (!aligned(c, out_dtype == MDY_DT_BF16 ? 2 : 4) || !aligned(a_s, 4) || !aligned(b_s, 4) || (bias && !aligned(bias, 2)))
+        return fail(MDY_E_ALIGN, "fp8_gemm_nt_e5m2: misaligned pointer");
+    if (int e = check_device()) return e;
+    const int rc = mdy::launch_fp8_gemm_nt_e5m2(a, a_s, as_row_stride, as_col_stride, b, b_s, c, bias, M, N, K, out_dtype,
+                                                static_cast<hipStream_t>(stream));
+    if (rc == -1)
+        return fail(MDY_E_SHAPE, "fp8_gemm_nt_e5m2: needs more than 64 rows, K a multiple of 128 up to 65536, 16-byte aligned a and b "
+                    "(other e5m2 problems: mdy_fp8_gemm_nt_rowscaled with the weight scales expanded to one per row)");
+    return launched(rc, "fp8_gemm_nt_e5m2");
+}
+
 int64_t mdy_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K < 1 || M > kMaxDim || N > kMaxDim || K > kMaxDim) return 0;
     return mdy::fp8_gemm_workspace_bytes(M, N, K);

@@ -280,6 +280,9 @@ int launch_weight_dequant(const void* x, const float* s, void* y, int64_t N, int
 int launch_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
                        const void* b, const float* b_s, void* c, const void* bias, int64_t M, int64_t N,
                        int64_t K, int out_dtype, hipStream_t stream);
+int launch_fp8_gemm_nt_e5m2(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
+                            const void* b, const float* b_s, void* c, const void* bias, int64_t M, int64_t N,
+                            int64_t K, int out_dtype, hipStream_t stream);
 int64_t fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int launch_fp8_gemm_nt_ws(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
                           const void* b, const float* b_s, void* c, const void* bias, int64_t M, int64_t N,

@@ -455,7 +455,7 @@ static bool pretouch_enabled() {
     return on;
 }
 
-template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT>
+template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT, int FMT = 0>
 static int launch_mfma(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, uint32_t as_bytes,
                        const uint8_t* b, const float* b_s, OUT* c, const uint16_t* bias, int M, int N, int K,
                        int ldc, hipStream_t stream) {
@@ -464,7 +464,7 @@ static int launch_mfma(const uint8_t* a, const float* a_s, int64_t as_rs, int64_
     // the 256x256 tile fills a CU's LDS: one workgroup per CU that walks its tiles itself
     const int wgs = (BM * BN >= 256 * 256 && tiles_m * tiles_n > cus) ? cus : tiles_m * tiles_n;
     dim3 grid((unsigned)wgs), block(WGM * WGN * 64);
-    hipLaunchKernelGGL((fp8_gemm_mfma_kernel<BM, BN, WGM, WGN, STAGES, OUT>), grid, block, 0, stream, a, a_s, (int)as_rs,
+    hipLaunchKernelGGL((fp8_gemm_mfma_kernel<BM, BN, WGM, WGN, STAGES, OUT, 0, 0, 0, FMT>), grid, block, 0, stream, a, a_s, (int)as_rs,
                        (int)as_cs, as_bytes, b, b_s, c, bias, M, N, K, ldc, tiles_m, tiles_n, pretouch_enabled() ? 1 : 0);
     return (int)hipGetLastError();
 }
@@ -554,6 +554,42 @@ static int launch_strip(const uint8_t* a, const float* a_s, int64_t as_rs, int64
 // 16-column kernel re-reads so little of a that it stays ahead)
 static bool strip_pays(int64_t max_rows, int64_t strips) { return max_rows > 4 && max_rows <= 64 && strips >= 200; }
 
+// The MFMA tile kernels for more than 64 rows (K % 128 == 0, aligned operands, scales within 2^31 bytes: the caller
+// checks).  FMT: operand byte format, 0 e4m3fn, 1 e5m2.
+template <typename OUT, int FMT>
+static int dispatch_tiles(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, int64_t as_extent, const uint8_t* b,
+                          const float* b_s, OUT* c, const uint16_t* bias, int M, int N, int K, hipStream_t stream) {
+    const int KB = K / 128;
+    if (big_tiles_pay(M, N)) {
+        const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
+        const int cols_main = main_tile_columns(tiles_m, tiles_n);
+        const int n_main = cols_main < tiles_n ? cols_main * 256 : N;
+        int rc = launch_mfma<256, 256, 2, 4, 2, OUT, FMT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, n_main, K, N,
+                                                       stream);
+        if (rc != 0 || n_main == N) return rc;
+        // remaining columns as 128x256 tiles (LDS has room for a ring of 3 K blocks there: 1-2 % of the whole
+        // call); n_main is a multiple of 256, so every pointer below keeps its alignment
+        return launch_mfma<128, 256, 2, 4, 3, OUT, FMT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b + (size_t)n_main * K,
+                                                     b_s + (size_t)(n_main >> 7) * KB, c + n_main,
+                                                     bias ? bias + n_main : nullptr, M, N - n_main, K, N, stream);
+    }
+    // Fewer tiles than that: the workgroups no longer fill the CUs, every K block's copy latency shows, and
+    // the time goes with K.  Use the LDS that the missing co-resident workgroups leave free for a deeper ring of
+    // K blocks in flight, and smaller tiles when even 128x128 tiles leave most CUs idle.
+#define MDY_FEW(BM_, BN_, WGM_, WGN_, ST_)                                                                            \
+    return launch_mfma<BM_, BN_, WGM_, WGN_, ST_, OUT, FMT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream)
+    switch (few_tiles_config(M, N, K)) {
+        case 1: MDY_FEW(128, 128, 2, 2, 4);
+        case 2: MDY_FEW(128, 64, 2, 2, 6);
+        case 3: MDY_FEW(64, 64, 2, 2, 8);
+        case 4: MDY_FEW(128, 256, 2, 4, 3);
+        case 5: MDY_FEW(256, 128, 2, 4, 3);
+        case 6: MDY_FEW(128, 192, 2, 4, 3);
+        default: MDY_FEW(128, 128, 2, 2, 2);
+    }
+#undef MDY_FEW
+}
+
 template <typename OUT>
 static int dispatch(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, const uint8_t* b,
                     const float* b_s, OUT* c, const uint16_t* bias, int M, int N, int K, hipStream_t stream) {
@@ -606,34 +642,7 @@ static int dispatch(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t a
 #undef MDY_SM
         return (int)hipGetLastError();
     }
-    if (big_tiles_pay(M, N)) {
-        const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
-        const int cols_main = main_tile_columns(tiles_m, tiles_n);
-        const int n_main = cols_main < tiles_n ? cols_main * 256 : N;
-        int rc = launch_mfma<256, 256, 2, 4, 2, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, n_main, K, N,
-                                                  stream);
-        if (rc != 0 || n_main == N) return rc;
-        // remaining columns as 128x256 tiles (LDS has room for a ring of 3 K blocks there: 1-2 % of the whole
-        // call); n_main is a multiple of 256, so every pointer below keeps its alignment
-        return launch_mfma<128, 256, 2, 4, 3, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b + (size_t)n_main * K,
-                                                b_s + (size_t)(n_main >> 7) * KB, c + n_main,
-                                                bias ? bias + n_main : nullptr, M, N - n_main, K, N, stream);
-    }
-    // Fewer tiles than that: the workgroups no longer fill the CUs, every K block's copy latency shows, and
-    // the time goes with K.  Use the LDS that the missing co-resident workgroups leave free for a deeper ring of
-    // K blocks in flight, and smaller tiles when even 128x128 tiles leave most CUs idle.
-#define MDY_FEW(BM_, BN_, ST_)                                                                                       \
-    return launch_mfma<BM_, BN_, 2, 2, ST_, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream)
-    switch (few_tiles_config(M, N, K)) {
-        case 1: MDY_FEW(128, 128, 4);
-        case 2: MDY_FEW(128, 64, 6);
-        case 3: MDY_FEW(64, 64, 8);
-        case 4: return launch_mfma<128, 256, 2, 4, 3, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
-        case 5: return launch_mfma<256, 128, 2, 4, 3, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
-        case 6: return launch_mfma<128, 192, 2, 4, 3, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
-        default: MDY_FEW(128, 128, 2);
-    }
-#undef MDY_FEW
+    return dispatch_tiles<OUT, 0>(a, a_s, as_rs, as_cs, as_extent, b, b_s, c, bias, M, N, K, stream);
 }
 
 // ---- split-K plan: which tile, how many K slices; ksplit == 1 means "do not split"
@@ -833,6 +842,28 @@ int launch_fp8_gemm_nt_static(const void* a, const float* a_s, int64_t as_row_st
     if (rc != 0) return rc;
     return launch_fp8_gemm_nt_ws(a, a_s, as_row_stride, as_col_stride, b, b_s, c, bias, M, N, K, out_dtype, ws,
                                  kStaticScratchBytes, stream);
+}
+
+// The tile kernels on e5m2 operands (the tuned kernels for fewer than 65 rows, the K split and the grouped GEMM are
+// e4m3fn only).  Returns -1 when the operands do not qualify for the tile kernels.
+int launch_fp8_gemm_nt_e5m2(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,
+                            const float* b_s, void* c, const void* bias, int64_t M, int64_t N, int64_t K, int out_dtype,
+                            hipStream_t stream) {
+    if (M == 0 || N == 0) return 0;
+    const int64_t KB = K / 128;
+    const int64_t as_extent = ((M - 1) * as_row_stride + (KB - 1) * as_col_stride + 1) * 4;
+    const bool ok = M > 64 && K % 128 == 0 && K <= (1 << 16) && as_row_stride >= 0 && as_col_stride >= 0 &&
+                    as_extent < ((int64_t)1 << 31) &&
+                    ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) == 0;
+    if (!ok) return -1;
+    const uint8_t* ap = static_cast<const uint8_t*>(a);
+    const uint8_t* bp = static_cast<const uint8_t*>(b);
+    const uint16_t* biasp = static_cast<const uint16_t*>(bias);
+    if (out_dtype == 0)
+        return dispatch_tiles<uint16_t, 1>(ap, a_s, as_row_stride, as_col_stride, as_extent, bp, b_s, static_cast<uint16_t*>(c), biasp,
+                                           (int)M, (int)N, (int)K, stream);
+    return dispatch_tiles<float, 1>(ap, a_s, as_row_stride, as_col_stride, as_extent, bp, b_s, static_cast<float*>(c), biasp, (int)M,
+                                    (int)N, (int)K, stream);
 }
 
 int launch_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,

@@ -12,9 +12,11 @@ __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1
 // One 128-deep scale block of a 16x16 sub-tile, from zero: v_mfma_f32_16x16x128_f8f6f4 with e4m3 operands and unit
 // hardware scales.  The weight rows go in as the MFMA's rows and the activation rows as its columns, so a lane's
 // four results are four consecutive n of one m.
+// FMT: byte format of both operands, 0 e4m3fn, 1 e5m2 (the instruction's cbsz / blgp fields).
+template <int FMT = 0>
 __device__ __forceinline__ floatx4 mfma_block(const intx8& weight_rows, const intx8& act_rows) {
     const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
-    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(weight_rows, act_rows, zero, 0, 0, 0, 0, 0, 0);
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(weight_rows, act_rows, zero, FMT, FMT, 0, 0, 0, 0);
 }
 
 // The promotion of one K block (offical_kernel.py:86): acc += (MFMA result of the block) * (its combined scale).
@@ -114,7 +116,7 @@ struct TileLds {
 //                  into buffer cur, one per GAP slots.
 // So the LDS latency after the barrier and the issue time of the copies sit in the shadow of the matrix
 // pipe instead of in front of the first MFMA of the next K block.
-template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT, int GAP_ = 0, int TD_ = 0, int ABL_ = 0>
+template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT, int GAP_ = 0, int TD_ = 0, int ABL_ = 0, int FMT_ = 0>
 __device__ __forceinline__ void fp8_gemm_tile(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
@@ -314,10 +316,10 @@ __device__ __forceinline__ void fp8_gemm_tile(
                 const intx8 fa_ = HOLD_A ? fh[h] : fx[si & 1];
                 const intx8 fb_ = HOLD_A ? fx[si & 1] : fh[h];
                 if (!NO_FOLD) {
-                    p[t % (DEPTH + 1)] = mfma_block(fb_, fa_);
+                    p[t % (DEPTH + 1)] = mfma_block<FMT_>(fb_, fa_);
                 } else {
                     floatx4& d = acc[HOLD_A ? h : si][HOLD_A ? si : h];
-                    d = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb_, fa_, d, 0, 0, 0, 0, 0, 0);
+                    d = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb_, fa_, d, FMT_, FMT_, 0, 0, 0, 0);
                 }
                 if (t == TB) {
                     // K block kb+1 has landed once only the younger loads are left in flight
@@ -413,7 +415,7 @@ __device__ __forceinline__ Duty tile_of(int local, int tiles_m, int tiles_n, int
     return d;
 }
 
-template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT, int GAP_ = 0, int TD_ = 0, int ABL_ = 0>
+template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT, int GAP_ = 0, int TD_ = 0, int ABL_ = 0, int FMT_ = 0>
 __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
@@ -428,8 +430,8 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
         int tm, tn;
         Duty duty = tile_of(xcd_contiguous(pid, ntiles), tiles_m, tiles_n, tm, tn);
         if (!pretouch) duty.a_sh = duty.b_sh = 0;
-        fp8_gemm_tile<BM, BN, WGM, WGN, STAGES, OUT, GAP_, TD_, ABL_>(a, a_s, as_rs, as_cs, as_bytes, b, b_s, c, bias, tm * BM, M, M,
-                                                                      tn * BN, N, K, ldc, duty, 0, K >> 7, pool);
+        fp8_gemm_tile<BM, BN, WGM, WGN, STAGES, OUT, GAP_, TD_, ABL_, FMT_>(a, a_s, as_rs, as_cs, as_bytes, b, b_s, c, bias, tm * BM, M,
+                                                                            M, tn * BN, N, K, ldc, duty, 0, K >> 7, pool);
         __syncthreads();   // every wave has left the tile's LDS buffers before the next tile's copies land in them
     }
 }

@@ -391,3 +391,35 @@ def test_fp8_mlp_e5m2_default_paths_agree():
     assert close(ug, O.fp8_linear_forward(x, mlp.up_gate_proj.weight.detach().cpu(), None, dtype=E5M2))
     act = O.silu_fwd(ug.cpu(), "up-gate")
     assert close(y0, O.fp8_linear_forward(act, mlp.down_proj.weight.detach().cpu(), None, dtype=E5M2))
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 512, 256), (300, 520, 384), (2000, 2304, 1024), (4096, 1536, 1152), (1000, 1090, 1664),
+                                   (520, 776, 1024), (512, 18432, 256)])
+def test_e5m2_tile_kernels_exact_integer(M, N, K):
+    """e5m2 operands on the tuned tile kernels (every tile configuration the dispatch picks for more than 64 rows): exact
+    on integer operands with power-of-two scales, fp32 and bf16 output, with a bias in the epilogue."""
+    from mdy_triton_amd import _lib
+    g = torch.Generator().manual_seed(M + N + K)
+    ai = torch.randint(-4, 5, (M, K), generator=g)
+    bi = torch.randint(-4, 5, (N, K), generator=g)
+    KB, NB = K // 128, (N + 127) // 128
+    ae = torch.randint(-2, 3, (M, KB), generator=g)
+    be = torch.randint(-2, 3, (NB, KB), generator=g)
+    exact = torch.zeros(M, N, dtype=torch.float64)
+    for kb in range(KB):
+        exact += (ai[:, kb * 128:(kb + 1) * 128].double() @ bi[:, kb * 128:(kb + 1) * 128].double().t()) * \
+            torch.exp2((ae[:, kb][:, None] + be[torch.arange(N) // 128, kb][None, :]).double())
+    a, b = ai.float().to(E5M2).to(DEV), bi.float().to(E5M2).to(DEV)
+    a_s, b_s = torch.exp2(ae.float()).to(DEV), torch.exp2(be.float()).to(DEV)
+    out = torch.full((M, N), float("nan"), device=DEV)
+    L = _lib.load()
+    assert L.mdy_fp8_gemm_nt_e5m2(a.data_ptr(), a_s.data_ptr(), KB, 1, b.data_ptr(), b_s.data_ptr(), out.data_ptr(), None, M, N, K, 1,
+                                  None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu().double(), exact)
+    bias = torch.randint(-8, 9, (N,), generator=g).float().bfloat16()
+    got = FK.fp8_matmul(a, b, a_s, b_s, bias.to(DEV))
+    assert torch.equal(got.cpu().double(), (exact + bias.double()).to(torch.bfloat16).double())
+    # what the entry point does not take is refused, not mis-run
+    assert L.mdy_fp8_gemm_nt_e5m2(a.data_ptr(), a_s.data_ptr(), KB, 1, b.data_ptr(), b_s.data_ptr(), out.data_ptr(), None, 64, N, K, 1,
+                                  None) == -2
