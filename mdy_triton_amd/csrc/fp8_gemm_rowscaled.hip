@@ -7,10 +7,10 @@
 // dimension (fp8_matmul_bwd, :254-257).
 //
 // The combined scale differs for each of a lane's four results of an MFMA (four consecutive n of one m), so the
-// fold is 4 multiplies + 4 FMAs per MFMA instead of 4 FMAs: a kernel of its own, kept simple (128x128 tile, four
-// waves of 64x64, the K block's two panels and two scale vectors copied global -> LDS by `buffer_load ... lds`,
-// double buffered, one barrier per K block), not the scheduled tile body of fp8_gemm_tile.h whose register budget
-// has no room for the per-column scales.  K % 128 == 0 (the callers contract over a padded token count).
+// fold is 4 multiplies + 4 FMAs per MFMA instead of 4 FMAs.  Two kernels: the scheduled tile body of fp8_gemm_tile.h in its
+// row-scaled-weight form (128x256 tiles; the 256x256 tile has no registers left for the per-column scales) for problems
+// that fill the CUs, and a plain loop (128x128 tile, four waves of 64x64, the K block's two panels and two scale vectors
+// copied global -> LDS by `buffer_load ... lds`, double buffered, one barrier per K block) for the rest.  K % 128 == 0 (the callers contract over a padded token count).
 #include "fp8_gemm_tile.h"
 
 namespace mdy {
@@ -117,6 +117,21 @@ __global__ __launch_bounds__(256) void fp8_gemm_rowscaled_kernel(
     }
 }
 
+// The scheduled tile body of fp8_gemm_tile.h in its row-scaled-weight form, 128x256 tiles (8 waves of 64x64, ring of three
+// K blocks): for problems that give every CU a tile.  Smaller problems run the plain kernel above, two workgroups per CU.
+template <typename OUT, int FMT>
+__global__ __launch_bounds__(512) void fp8_gemm_rowscaled_tile_kernel(
+    const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
+    const uint8_t* __restrict__ b, const float* __restrict__ b_s, int bs_rs, int bs_cs, uint32_t bs_bytes,
+    OUT* __restrict__ c, int M, int N, int K, int tiles_m, int tiles_n) {
+    __shared__ __attribute__((aligned(1024))) uint8_t pool[TileLds<128, 256, 8, 3>::bytes];
+    const int ntiles = tiles_m * tiles_n;
+    int tm, tn;
+    const Duty duty = tile_of(xcd_contiguous(blockIdx.x, ntiles), tiles_m, tiles_n, tm, tn);
+    fp8_gemm_tile<128, 256, 2, 4, 3, OUT, 0, 0, 0, FMT, true>(a, a_s, as_rs, as_cs, as_bytes, b, b_s, c, nullptr, tm * 128, M, M,
+                                                              tn * 256, N, K, N, duty, 0, K >> 7, pool, bs_rs, bs_cs, bs_bytes);
+}
+
 // returns hipError_t, or -1 when the operands do not qualify (K % 128 != 0, misaligned, scale extents >= 2^31 bytes)
 int launch_fp8_gemm_nt_rowscaled(const void* a, const float* a_s, int64_t as_rs, int64_t as_cs, const void* b,
                                  const float* b_s, int64_t bs_rs, int64_t bs_cs, void* c, int64_t M, int64_t N, int64_t K,
@@ -128,6 +143,19 @@ int launch_fp8_gemm_nt_rowscaled(const void* a, const float* a_s, int64_t as_rs,
         b_ext >= ((int64_t)1 << 31) || ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) != 0 ||
         128 * K >= ((int64_t)1 << 31))
         return -1;
+    // 128x256 tiles of the scheduled body once they fill the CUs (and K fits its weight-scale staging)
+    const int64_t big_m = (M + 127) / 128, big_n = (N + 255) / 256;
+    if (big_m * big_n >= 200 && K <= (1 << 16) && big_m * big_n <= 0x7FFFFFFF) {
+#define MDY_RST(OUT_T, FMT)                                                                                              \
+    hipLaunchKernelGGL((fp8_gemm_rowscaled_tile_kernel<OUT_T, FMT>), dim3((unsigned)(big_m * big_n)), dim3(512), 0, stream, \
+                       static_cast<const uint8_t*>(a), a_s, (int)as_rs, (int)as_cs, (uint32_t)a_ext,                      \
+                       static_cast<const uint8_t*>(b), b_s, (int)bs_rs, (int)bs_cs, (uint32_t)b_ext, static_cast<OUT_T*>(c), \
+                       (int)M, (int)N, (int)K, (int)big_m, (int)big_n)
+        if (out_dtype == 0) { if (fmt == 0) MDY_RST(uint16_t, 0); else MDY_RST(uint16_t, 1); }
+        else { if (fmt == 0) MDY_RST(float, 0); else MDY_RST(float, 1); }
+#undef MDY_RST
+        return (int)hipGetLastError();
+    }
     const int tiles_m = (int)((M + 127) / 128), tiles_n = (int)((N + 127) / 128);
     if ((int64_t)tiles_m * tiles_n > 0x7FFFFFFF) return kErrTooManyBlocks;
     dim3 grid((unsigned)(tiles_m * tiles_n)), block(256);

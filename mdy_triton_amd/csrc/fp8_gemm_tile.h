@@ -116,12 +116,17 @@ struct TileLds {
 //                  into buffer cur, one per GAP slots.
 // So the LDS latency after the barrier and the issue time of the copies sit in the shadow of the matrix
 // pipe instead of in front of the first MFMA of the next K block.
-template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT, int GAP_ = 0, int TD_ = 0, int ABL_ = 0, int FMT_ = 0>
+// BROW_: the weight operand carries one scale per ROW and K block (b_s[n * bs_rs + kb * bs_cs], bs_bytes long) instead of
+// one per 128x128 block: the scales of the tile's BN rows travel through LDS per K block like the activation scales
+// (copied by the waves behind the activation-scale waves), a lane keeps the four scales of its four columns of every
+// sub-tile, and the fold multiplies them in: 4 multiplies + 4 FMAs per MFMA instead of 4 FMAs.
+template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT, int GAP_ = 0, int TD_ = 0, int ABL_ = 0, int FMT_ = 0,
+          bool BROW_ = false>
 __device__ __forceinline__ void fp8_gemm_tile(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
     const uint16_t* __restrict__ bias, int m0, int m_end, int m_total, int n0, int N, int K, int ldc, const Duty duty,
-    int kb0, int kb1, uint8_t* __restrict__ pool) {
+    int kb0, int kb1, uint8_t* __restrict__ pool, int bs_rs = 0, int bs_cs = 0, uint32_t bs_bytes = 0) {
     // ABL_ switches parts of the K loop off for the timing probe (mdy_fp8_gemm_probe); the product uses 0.
     //   1: no global->LDS copies in the loop (the ring is filled once and replayed)   2: no LDS fragment / scale reads
     //   4: no FMA fold (the MFMAs accumulate in place, no block scales)                8: no pre-touches
@@ -185,13 +190,22 @@ __device__ __forceinline__ void fp8_gemm_tile(
     };
     const int prow = wave * 8 + (lane >> 3);                          // row inside a pass
     const int voff = prow * K + (((lane & 7) ^ swz(prow)) << 4);      // permuted chunk of that row
-    intx4 rs = make_rsrc(a_s, as_bytes);
-    if (wave >= S_WAVES) rs[2] = 0;                                   // these waves copy no scales: always out of range
+    // scale copies: waves 0 .. S_WAVES-1 copy 64 activation scales of the K block each; with BROW_ the next BN / 64 waves
+    // copy 64 weight-row scales each (into the area that otherwise holds the weight's block scales); the rest copy nothing
+    constexpr int SB_WAVES = BROW_ ? BN / 64 : 0;
+    static_assert(S_WAVES + SB_WAVES <= WAVES && (!BROW_ || STAGES * BN * 4 <= L::NBS * 512 * 4), "waves / LDS for the weight-row scales");
+    const bool sb_wave = BROW_ && wave >= S_WAVES && wave < S_WAVES + SB_WAVES;
+    float* lds_sbr = reinterpret_cast<float*>(pool + L::bs_off);     // BROW_: [STAGES][BN] weight-row scales
+    intx4 rs = sb_wave ? make_rsrc(b_s, bs_bytes) : make_rsrc(a_s, as_bytes);
+    if (wave >= S_WAVES && !sb_wave) rs[2] = 0;                       // these waves copy no scales: always out of range
+    const int sc_cs = sb_wave ? bs_cs : as_cs;
+    const uint32_t sc_bytes = sb_wave ? bs_bytes : as_bytes;
     const uint32_t ld_base = lds_addr(&lds_dummy[0]) + wave * 512;
     const uint32_t la_base = lds_addr(&lds_a[0][0]) + wave * 1024;
     const uint32_t lb_base = lds_addr(&lds_b[0][0]) + wave * 1024;
-    const uint32_t ls_base = wave < S_WAVES ? lds_addr(&lds_s[0][0]) + wave * 256 : ld_base;
-    const uint32_t ls_buf = wave < S_WAVES ? BM * 4 : 0;
+    const uint32_t ls_base = wave < S_WAVES ? lds_addr(&lds_s[0][0]) + wave * 256
+                             : sb_wave ? lds_addr(lds_sbr) + (wave - S_WAVES) * 256 : ld_base;
+    const uint32_t ls_buf = wave < S_WAVES ? BM * 4 : sb_wave ? BN * 4 : 0;
     // duty touch: the even waves load one dword of every line of this workgroup's share of the B panel (64
     // rows per wave), the odd waves of the A panel, TD K blocks ahead, into the dummy area: the lines are in L2
     // when this workgroup and its neighbours copy them.  Waves beyond the share run the same instruction on an
@@ -202,7 +216,8 @@ __device__ __forceinline__ void fp8_gemm_tile(
         TileAddr t;
         t.ra = make_rsrc(a + (size_t)tm0 * K, (uint32_t)min(BM, M - tm0) * (uint32_t)K);
         t.rb = make_rsrc(b + (size_t)tn0 * K, (uint32_t)min(BN, N - tn0) * (uint32_t)K);
-        t.s_voff = min(tm0 + (wave % S_WAVES) * 64 + lane, m_total - 1) * as_rs * 4;
+        t.s_voff = sb_wave ? min(tn0 + (wave - S_WAVES) * 64 + lane, N - 1) * bs_rs * 4
+                           : min(tm0 + (wave % S_WAVES) * 64 + lane, m_total - 1) * as_rs * 4;
         const int share = touch_b ? (BN >> d.b_sh) : (BM >> d.a_sh);      // rows of the share
         t.rt = touch_b ? t.rb : t.ra;
         // nobody to share with: touching one's own lines ahead of the copy only adds requests (measured)
@@ -218,7 +233,7 @@ __device__ __forceinline__ void fp8_gemm_tile(
     auto issue = [&](const TileAddr& t, int i, int kb, int buf) {
         const bool more = kb < kb1;
         if (i == 0)
-            dma4(rs, t.s_voff, more ? kb * as_cs * 4 : (int)as_bytes, ls_base + buf * ls_buf);
+            dma4(rs, t.s_voff, more ? kb * sc_cs * 4 : (int)sc_bytes, ls_base + buf * ls_buf);
         else if (i <= A_PASSES)
             dma16(t.ra, voff, (i - 1) * PASS_ROWS * K + (more ? kb * 128 : t.ra[2]), la_base + buf * (BM * 128) + (i - 1) * PASS_ROWS * 128);
         else
@@ -229,7 +244,7 @@ __device__ __forceinline__ void fp8_gemm_tile(
     // The start of a tile: its weight scales, then the copies in the order the K loop keeps up: for every K block its
     // first FIRST copies, the rest, one touch; K blocks 0 .. STAGES-2 whole and the first copies of block STAGES-1.
     auto prologue = [&](const TileAddr& t) {
-        if (wave < NBS) {
+        if (!BROW_ && wave < NBS) {
             const int nb = min((t.n0 >> 7) + wave, ((N + 127) >> 7) - 1);
             const intx4 rbs = make_rsrc(b_s + (size_t)nb * KB, (uint32_t)KB * 4u);
             for (int cc = 0; cc < KB; cc += 64) dma4(rbs, lane * 4, cc * 4, lds_addr(&lds_bs[wave][cc]));
@@ -282,10 +297,16 @@ __device__ __forceinline__ void fp8_gemm_tile(
     __syncthreads();
     intx8 fh[NH], fx[2];
     float sc[TI], sc_hi[STRADDLE ? TI : 1];
+    floatx4 sbv[BROW_ ? TJ : 1];                 // BROW_: the weight-row scales of this lane's four columns of every sub-tile
+    const float* sbr_lane = lds_sbr + wn * WN + 4 * fk;
+    if (BROW_) {
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) sbv[j] = *reinterpret_cast<const floatx4*>(sbr_lane + j * 16);
+    }
 #pragma unroll
     for (int h = 0; h < NH; ++h) fh[h] = read_frag(HOLD_A ? lds_a[0] : lds_b[0], h0, h1, h);
     {
-        const float sb = my_bs[kb0], sb_hi = my_bs_hi[kb0];
+        const float sb = BROW_ ? 1.0f : my_bs[kb0], sb_hi = BROW_ ? 1.0f : my_bs_hi[kb0];
 #pragma unroll
         for (int i = 0; i < TI; ++i) {
             const float sa = lds_s[0][s_rd + i * 16];
@@ -304,6 +325,7 @@ __device__ __forceinline__ void fp8_gemm_tile(
         const uint8_t* lx_n = HOLD_A ? lds_b[nxt] : lds_a[nxt];
         const float* ls_n = lds_s[nxt];
         float sc_n[TI], sc_hi_n[STRADDLE ? TI : 1];
+        floatx4 sbv_n[BROW_ ? TJ : 1];
         floatx4 p[DEPTH + 1];
 #pragma unroll
         for (int t = 0; t < NT + DEPTH; ++t) {
@@ -327,7 +349,11 @@ __device__ __forceinline__ void fp8_gemm_tile(
                     __syncthreads();
                     if (!NO_LDS) {
                         fx[0] = read_frag(lx_n, x0, x1, 0);      // queue slot 0 was last used by streamed fragment NS-2
-                        const float sb = my_bs[min(kb + 1, KB - 1)], sb_hi = my_bs_hi[min(kb + 1, KB - 1)];
+                        const float sb = BROW_ ? 1.0f : my_bs[min(kb + 1, KB - 1)], sb_hi = BROW_ ? 1.0f : my_bs_hi[min(kb + 1, KB - 1)];
+                        if (BROW_) {
+#pragma unroll
+                            for (int j = 0; j < TJ; ++j) sbv_n[j] = *reinterpret_cast<const floatx4*>(sbr_lane + nxt * BN + j * 16);
+                        }
 #pragma unroll
                         for (int i = 0; i < TI; ++i) {
                             const float sa = ls_n[s_rd + i * 16];
@@ -352,7 +378,14 @@ __device__ __forceinline__ void fp8_gemm_tile(
                 const int u = t - DEPTH, si = u / NH, h = u % NH;
                 const int i = HOLD_A ? h : si, j = HOLD_A ? si : h;
                 const floatx4 q = p[u % (DEPTH + 1)];
-                fold(acc[i][j], q, (STRADDLE && j >= jsplit) ? sc_hi[i] : sc[i]);
+                if (BROW_) {
+                    acc[i][j][0] = __builtin_fmaf(q[0], sc[i] * sbv[j][0], acc[i][j][0]);
+                    acc[i][j][1] = __builtin_fmaf(q[1], sc[i] * sbv[j][1], acc[i][j][1]);
+                    acc[i][j][2] = __builtin_fmaf(q[2], sc[i] * sbv[j][2], acc[i][j][2]);
+                    acc[i][j][3] = __builtin_fmaf(q[3], sc[i] * sbv[j][3], acc[i][j][3]);
+                } else {
+                    fold(acc[i][j], q, (STRADDLE && j >= jsplit) ? sc_hi[i] : sc[i]);
+                }
             }
             if (!NO_COPY) {
 #pragma unroll
@@ -369,6 +402,10 @@ __device__ __forceinline__ void fp8_gemm_tile(
         for (int i = 0; i < TI; ++i) {
             sc[i] = sc_n[i];
             if (STRADDLE) sc_hi[i] = sc_hi_n[i];
+        }
+        if (BROW_) {
+#pragma unroll
+            for (int j = 0; j < TJ; ++j) sbv[j] = sbv_n[j];
         }
         cur = nxt;
     }
