@@ -62,7 +62,8 @@ def test_act_quant_block_leading_dims_and_asserts():
         m.act_quant_block(x.to(DEV), dtype=torch.float16)
 
 
-@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (256, 384, 512), (130, 200, 384), (1000, 260, 1024), (64, 64, 2304)])
+@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (256, 384, 512), (130, 200, 384), (1000, 260, 1024), (64, 64, 2304),
+                                   (2048, 3328, 256), (1990, 3300, 384)])        # the last two: 128x256 tiles of the scheduled body
 def test_rowscaled_gemm_exact_integer(M, N, K):
     """Integer operands and power-of-two scales on both sides: every product and sum is exact, so the bf16 result must
     equal the float64 computation rounded once (catches swapped scale roles, K-block order, tile edges)."""
@@ -305,7 +306,7 @@ def test_e5m2_quantizers_bit_exact(dtype):
     assert wq4.dtype == FP8
 
 
-@pytest.mark.parametrize("M,N,K", [(128, 256, 256), (130, 200, 384), (256, 384, 1024)])
+@pytest.mark.parametrize("M,N,K", [(128, 256, 256), (130, 200, 384), (256, 384, 1024), (2048, 3328, 256)])
 def test_e5m2_gemms_exact_integer(M, N, K):
     """e5m2 operands through both GEMM forms of fp8_kernel.fp8_matmul (block-scaled weight: its scales expanded to one
     per row; row scales on both sides): integer operands and power-of-two scales are exact, so the result must equal
