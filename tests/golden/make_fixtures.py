@@ -21,6 +21,13 @@ weight_dequant_codes.npz
 gemm_exact.npz
     small-integer e4m3fn operands with power-of-two scales whose products and
     sums are exact in fp32 and in bf16; the expected output is computed in int64.
+act_quant_block_e5m2.npz
+    the same construction as act_quant_codes.npz for the e5m2 format (the default dtype of
+    deepseekv3/fp8_kernel.py's act_quant_block) in BOTH directions: x_bits uint16 [128, 256]
+    bfloat16 patterns; column c of the 128 rows holds every finite non-negative or non-positive
+    e5m2 value (codes 0x00..0x7B or 0x80..0xFB, 124 values, plus four more copies of 57344)
+    times 2**e(c), so the transposed quantization (along the rows) must return the codes
+    themselves: y_t uint8 [256, 128], s_t float32 [256, 1] = 2**e(c).
 """
 import os
 import sys
@@ -29,7 +36,7 @@ import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
-from oracle.fp8_format import decode_table, f32_to_bf16_bits_rne  # noqa: E402
+from oracle.fp8_format import decode_table, decode_table_e5m2, f32_to_bf16_bits_rne  # noqa: E402
 
 
 def bf16_bits_exact(x32: np.ndarray) -> np.ndarray:
@@ -104,7 +111,27 @@ def make_gemm_exact():
              bf16_exact=exact)
 
 
+def make_act_quant_block_e5m2():
+    tab = decode_table_e5m2()
+    rng = np.random.default_rng(77)
+    R, C = 128, 256
+    x_bits = np.zeros((R, C), np.uint16)
+    y_t = np.zeros((C, R), np.uint8)
+    s_t = np.zeros((C, 1), np.float32)
+    for c in range(C):
+        e = int(rng.integers(-20, 21))
+        base = 0x80 if c % 2 else 0x00
+        codes = np.concatenate([np.arange(base, base + 0x7C), [base + 0x7B] * 4]).astype(np.uint8)   # 124 finite codes + 57344 x 4
+        rng.shuffle(codes)
+        vals = tab[codes].astype(np.float64) * 2.0 ** e
+        x_bits[:, c] = bf16_bits_exact(vals.astype(np.float32))     # e5m2 values (2 mantissa bits) are exact in bfloat16
+        y_t[c] = codes
+        s_t[c, 0] = np.float32(2.0 ** e)
+    np.savez(os.path.join(HERE, "act_quant_block_e5m2.npz"), x_bits=x_bits, y_t=y_t, s_t=s_t)
+
+
 if __name__ == "__main__":
+    make_act_quant_block_e5m2()
     make_act_quant_codes()
     make_weight_dequant_codes()
     make_gemm_exact()

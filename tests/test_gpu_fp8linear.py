@@ -424,3 +424,14 @@ def test_e5m2_tile_kernels_exact_integer(M, N, K):
     # what the entry point does not take is refused, not mis-run
     assert L.mdy_fp8_gemm_nt_e5m2(a.data_ptr(), a_s.data_ptr(), KB, 1, b.data_ptr(), b_s.data_ptr(), out.data_ptr(), None, 64, N, K, 1,
                                   None) == -2
+
+
+def test_act_quant_block_e5m2_golden_codes_on_device():
+    """The closed-form e5m2 fixture on the device, both directions (the transposing kernel and the general row kernel)."""
+    import os
+    d = np.load(os.path.join(os.path.dirname(__file__), "golden", "act_quant_block_e5m2.npz"))
+    x = torch.from_numpy(d["x_bits"].view(np.int16)).view(torch.bfloat16).to(DEV)
+    y_t, s_t = m.act_quant_block(x, transpose=True)           # default dtype: float8_e5m2
+    assert np.array_equal(u8(y_t), d["y_t"]) and np.array_equal(s_t.cpu().numpy(), d["s_t"])
+    y, s = m.act_quant_block(x.t().contiguous())
+    assert np.array_equal(u8(y), d["y_t"]) and np.array_equal(s.cpu().numpy(), d["s_t"])

@@ -478,3 +478,15 @@ def test_fp8_linear_oracle_close_to_unquantized():
     assert dx.shape == x.shape and (dx.float() - dxr).abs().mean() < 0.06 * dxr.abs().mean()
     assert dw.shape == w.shape and (dw.float() - dwr).abs().mean() < 0.06 * dwr.abs().mean()
     assert torch.allclose(db.float(), dy.float().reshape(-1, 128).sum(0), rtol=1e-2, atol=1e-1)
+
+
+def test_act_quant_block_e5m2_golden_codes():
+    """The closed-form e5m2 fixture (tests/golden/make_fixtures.py, no oracle call): quantizing x along its rows must
+    return, for every column, exactly the e5m2 codes it was built from and the power-of-two scale."""
+    d = np.load(os.path.join(GOLD, "act_quant_block_e5m2.npz"))
+    x = torch.from_numpy(d["x_bits"].view(np.int16)).view(torch.bfloat16)
+    y_t, s_t = O.act_quant_block(x, transpose=True, dtype=torch.float8_e5m2)
+    assert np.array_equal(y_t.view(torch.uint8).numpy(), d["y_t"]) and np.array_equal(s_t.numpy(), d["s_t"])
+    # the row-wise direction of the transposed matrix is the same quantization
+    y, s = O.act_quant_block(x.t().contiguous(), dtype=torch.float8_e5m2)
+    assert np.array_equal(y.view(torch.uint8).numpy(), d["y_t"]) and np.array_equal(s.numpy(), d["s_t"])
