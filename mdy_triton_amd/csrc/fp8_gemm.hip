@@ -157,7 +157,7 @@ __global__ __launch_bounds__(512) void fp8_grouped_gemm_kernel(
 // ---------------------------------------------------------------------------
 constexpr int kSmWaves = 8;
 
-template <int MT, int NC, typename OUT>
+template <int MT, int NC, typename OUT, int FMT = 0>
 __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_kernel(const uint8_t* __restrict__ a,
                                                                           const float* __restrict__ a_s, int64_t as_rs,
                                                                           int64_t as_cs, const uint8_t* __restrict__ b,
@@ -234,7 +234,7 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_kernel(const ui
                 const intx8 fa = intx8{cur.alo[i][0], cur.alo[i][1], cur.alo[i][2], cur.alo[i][3],
                                        cur.ahi[i][0], cur.ahi[i][1], cur.ahi[i][2], cur.ahi[i][3]};
                 const float sc = cur.sa[i] * cur.sb[j];
-                const floatx4 p = mfma_block(fb, fa);
+                const floatx4 p = mfma_block<FMT>(fb, fa);
                 fold(acc[j][i], p, sc);
             }
         }
@@ -280,7 +280,7 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_kernel(const ui
 // ---------------------------------------------------------------------------
 constexpr int kStripKC = 4;   // K blocks per step
 
-template <int MT, typename OUT>
+template <int MT, typename OUT, int FMT = 0>
 __global__ __launch_bounds__(512) void fp8_gemm_strip_kernel(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
@@ -369,7 +369,7 @@ __global__ __launch_bounds__(512) void fp8_gemm_strip_kernel(
                     const intx4 hi = *reinterpret_cast<const intx4*>(la + a_rd1);
                     const intx8 fa = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                     const float sc = lds_sa[buf][kc][i * 16 + frow] * sb;
-                    const floatx4 p = mfma_block(fb, fa);
+                    const floatx4 p = mfma_block<FMT>(fb, fa);
                     fold(acc[i], p, sc);
                 }
             }
@@ -525,7 +525,7 @@ static int few_tiles_config(int M, int N, int K) {
     return 0;
 }
 
-template <typename OUT>
+template <typename OUT, int FMT = 0>
 static int launch_strip(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, uint32_t as_bytes,
                         const uint8_t* b, const float* b_s, OUT* c, const uint16_t* bias, const int64_t* m_splits, int G,
                         int max_rows, int N, int K, hipStream_t stream) {
@@ -540,7 +540,7 @@ static int launch_strip(const uint8_t* a, const float* a_s, int64_t as_rs, int64
     for (int g = G; g <= kMaxGroups; ++g) { tbl.row_start[g] = row; tbl.tile_start[g] = 0; }
     dim3 grid((unsigned)((N + 127) / 128), (unsigned)G), block(512);
 #define MDY_STRIP(MT)                                                                                              \
-    hipLaunchKernelGGL((fp8_gemm_strip_kernel<MT, OUT>), grid, block, 0, stream, a, a_s, (int)as_rs, (int)as_cs, as_bytes, b, \
+    hipLaunchKernelGGL((fp8_gemm_strip_kernel<MT, OUT, FMT>), grid, block, 0, stream, a, a_s, (int)as_rs, (int)as_cs, as_bytes, b, \
                        b_s, c, bias, N, K, tbl)
     if (max_rows <= 16) MDY_STRIP(1);
     else if (max_rows <= 32) MDY_STRIP(2);
@@ -553,6 +553,50 @@ static int launch_strip(const uint8_t* a, const float* a_s, int64_t as_rs, int64
 // few rows per group and enough 128-column strips to fill the CUs without splitting K (with a handful of rows the
 // 16-column kernel re-reads so little of a that it stays ahead)
 static bool strip_pays(int64_t max_rows, int64_t strips) { return max_rows > 4 && max_rows <= 64 && strips >= 200; }
+
+// Up to 64 rows (K % 128 == 0, aligned operands: the caller checks; big_ok: the scales also fit the tile kernels'
+// 32-bit addressing).  FMT: operand byte format, 0 e4m3fn, 1 e5m2.
+template <typename OUT, int FMT>
+static int dispatch_small(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, int64_t as_extent, bool big_ok,
+                          const uint8_t* b, const float* b_s, OUT* c, const uint16_t* bias, int M, int N, int K, hipStream_t stream) {
+    if (M <= 64 && big_ok && strip_pays(M, (N + 127) / 128)) {
+        const int64_t one = M;
+        return launch_strip<OUT, FMT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, &one, 1, M, N, K, stream);
+    }
+    // 32..64 rows against a wide weight: the kernel below re-reads the activation rows in every one of its
+    // N/16 workgroups, and from 32 rows on that traffic costs more than the empty rows of an MFMA tile.
+    // Measured (M=64): N=18432, K=7168 121 -> 64 us with 128x128 tiles; N=7168, K=16384 110 -> 80 us with 64x64.
+    if (M >= 32 && M <= 64 && big_ok && (N + 127) / 128 >= 128)
+        return launch_mfma<128, 128, 2, 2, 4, OUT, FMT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
+    if (M >= 32 && M <= 64 && big_ok && (N + 63) / 64 >= 100)
+        return launch_mfma<64, 64, 2, 2, 8, OUT, FMT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
+    if (M <= 64) {
+        // one workgroup streams 16 weight columns against MT row sub-tiles; every workgroup re-reads its rows of
+        // a, so with few column groups (N small) the rows are split over grid.y as well: more workgroups, less
+        // traffic through each CU's L1
+        const int sub = (M + 15) / 16;
+        int mt = sub;
+        if ((N + 15) / 16 < 200 && sub >= 2) mt = (sub + 1) / 2;
+        // two column groups per workgroup when that still leaves enough workgroups: the activation rows are
+        // fetched by half as many of them (measured: pays from 17 rows on with 288 workgroups, from 5 rows on with
+        // 512; M=31, N=18432, K=7168: 70 -> 59 us)
+        const long wgs32 = (N + 31) / 32;
+        const bool two = mt <= 2 && ((M > 16 && wgs32 >= 288) || (M > 4 && wgs32 >= 512));
+        dim3 grid((unsigned)(two ? (N + 31) / 32 : (N + 15) / 16), (unsigned)((sub + mt - 1) / mt));
+#define MDY_SM(MT, NC)                                                                                             \
+    hipLaunchKernelGGL((fp8_gemm_smallm_kernel<MT, NC, OUT, FMT>), grid, dim3(kSmWaves * 64), 0, stream, a, a_s, as_rs, as_cs, b, \
+                       b_s, c, bias, M, N, K)
+        if (two && mt == 1) MDY_SM(1, 2);
+        else if (two) MDY_SM(2, 2);
+        else if (mt == 1) MDY_SM(1, 1);
+        else if (mt == 2) MDY_SM(2, 1);
+        else if (mt == 3) MDY_SM(3, 1);
+        else MDY_SM(4, 1);
+#undef MDY_SM
+        return (int)hipGetLastError();
+    }
+    return -1;   // not reached: M <= 64 ends in the weight-streaming kernel above
+}
 
 // The MFMA tile kernels for more than 64 rows (K % 128 == 0, aligned operands, scales within 2^31 bytes: the caller
 // checks).  FMT: operand byte format, 0 e4m3fn, 1 e5m2.
@@ -606,42 +650,7 @@ static int dispatch(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t a
                            bias, M, N, K);
         return (int)hipGetLastError();
     }
-    if (M <= 64 && big_ok && strip_pays(M, (N + 127) / 128)) {
-        const int64_t one = M;
-        return launch_strip<OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, &one, 1, M, N, K, stream);
-    }
-    // 32..64 rows against a wide weight: the kernel below re-reads the activation rows in every one of its
-    // N/16 workgroups, and from 32 rows on that traffic costs more than the empty rows of an MFMA tile.
-    // Measured (M=64): N=18432, K=7168 121 -> 64 us with 128x128 tiles; N=7168, K=16384 110 -> 80 us with 64x64.
-    if (M >= 32 && M <= 64 && big_ok && (N + 127) / 128 >= 128)
-        return launch_mfma<128, 128, 2, 2, 4, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
-    if (M >= 32 && M <= 64 && big_ok && (N + 63) / 64 >= 100)
-        return launch_mfma<64, 64, 2, 2, 8, OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
-    if (M <= 64) {
-        // one workgroup streams 16 weight columns against MT row sub-tiles; every workgroup re-reads its rows of
-        // a, so with few column groups (N small) the rows are split over grid.y as well: more workgroups, less
-        // traffic through each CU's L1
-        const int sub = (M + 15) / 16;
-        int mt = sub;
-        if ((N + 15) / 16 < 200 && sub >= 2) mt = (sub + 1) / 2;
-        // two column groups per workgroup when that still leaves enough workgroups: the activation rows are
-        // fetched by half as many of them (measured: pays from 17 rows on with 288 workgroups, from 5 rows on with
-        // 512; M=31, N=18432, K=7168: 70 -> 59 us)
-        const long wgs32 = (N + 31) / 32;
-        const bool two = mt <= 2 && ((M > 16 && wgs32 >= 288) || (M > 4 && wgs32 >= 512));
-        dim3 grid((unsigned)(two ? (N + 31) / 32 : (N + 15) / 16), (unsigned)((sub + mt - 1) / mt));
-#define MDY_SM(MT, NC)                                                                                             \
-    hipLaunchKernelGGL((fp8_gemm_smallm_kernel<MT, NC, OUT>), grid, dim3(kSmWaves * 64), 0, stream, a, a_s, as_rs, as_cs, b, \
-                       b_s, c, bias, M, N, K)
-        if (two && mt == 1) MDY_SM(1, 2);
-        else if (two) MDY_SM(2, 2);
-        else if (mt == 1) MDY_SM(1, 1);
-        else if (mt == 2) MDY_SM(2, 1);
-        else if (mt == 3) MDY_SM(3, 1);
-        else MDY_SM(4, 1);
-#undef MDY_SM
-        return (int)hipGetLastError();
-    }
+    if (M <= 64) return dispatch_small<OUT, 0>(a, a_s, as_rs, as_cs, as_extent, big_ok, b, b_s, c, bias, M, N, K, stream);
     return dispatch_tiles<OUT, 0>(a, a_s, as_rs, as_cs, as_extent, b, b_s, c, bias, M, N, K, stream);
 }
 
@@ -844,21 +853,28 @@ int launch_fp8_gemm_nt_static(const void* a, const float* a_s, int64_t as_row_st
                                  kStaticScratchBytes, stream);
 }
 
-// The tile kernels on e5m2 operands (the tuned kernels for fewer than 65 rows, the K split and the grouped GEMM are
-// e4m3fn only).  Returns -1 when the operands do not qualify for the tile kernels.
+// The MFMA kernels on e5m2 operands: the tile, weight-streaming and strip kernels (the K split and the grouped GEMM are
+// e4m3fn only).  Returns -1 when the operands do not qualify (K % 128 != 0, K > 65536, unaligned, scales beyond 2^31 bytes).
 int launch_fp8_gemm_nt_e5m2(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,
                             const float* b_s, void* c, const void* bias, int64_t M, int64_t N, int64_t K, int out_dtype,
                             hipStream_t stream) {
     if (M == 0 || N == 0) return 0;
     const int64_t KB = K / 128;
     const int64_t as_extent = ((M - 1) * as_row_stride + (KB - 1) * as_col_stride + 1) * 4;
-    const bool ok = M > 64 && K % 128 == 0 && K <= (1 << 16) && as_row_stride >= 0 && as_col_stride >= 0 &&
+    const bool ok = K % 128 == 0 && K <= (1 << 16) && as_row_stride >= 0 && as_col_stride >= 0 &&
                     as_extent < ((int64_t)1 << 31) &&
                     ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) == 0;
     if (!ok) return -1;
     const uint8_t* ap = static_cast<const uint8_t*>(a);
     const uint8_t* bp = static_cast<const uint8_t*>(b);
     const uint16_t* biasp = static_cast<const uint16_t*>(bias);
+    if (M <= 64) {
+        if (out_dtype == 0)
+            return dispatch_small<uint16_t, 1>(ap, a_s, as_row_stride, as_col_stride, as_extent, true, bp, b_s, static_cast<uint16_t*>(c),
+                                               biasp, (int)M, (int)N, (int)K, stream);
+        return dispatch_small<float, 1>(ap, a_s, as_row_stride, as_col_stride, as_extent, true, bp, b_s, static_cast<float*>(c), biasp,
+                                        (int)M, (int)N, (int)K, stream);
+    }
     if (out_dtype == 0)
         return dispatch_tiles<uint16_t, 1>(ap, a_s, as_row_stride, as_col_stride, as_extent, bp, b_s, static_cast<uint16_t*>(c), biasp,
                                            (int)M, (int)N, (int)K, stream);
