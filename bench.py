@@ -34,7 +34,7 @@ Before the W warm-up steps the script runs the same step for 50 ms (set-up, unti
 GPU needs some 20 ms of work to reach its sustained clock, whatever W is.
 With --table a per-kernel table for every benchmark configuration and for the shapes the reference
 publishes numbers for goes to stderr; with --ablation the tile kernel is timed with parts of its K loop
-switched off (mdy_fp8_gemm_probe), power and clock beside each line (stdout, no JSON).
+switched off (mdy_fp8_gemm_probe of libmdyfp8_probe.so), power and clock beside each line (stdout, no JSON).
 """
 import argparse
 import json
@@ -552,11 +552,24 @@ def main():
     print(json.dumps(result))
 
 
+def load_probe_lib():
+    """libmdyfp8_probe.so: the timing probes (ablated tile kernels, copy-only and MFMA-only ceilings).  Not part of the
+    product library; only the diagnostic modes of this script load it."""
+    import ctypes
+    path = os.path.join(ROOT, "mdy_triton_amd", "csrc", "libmdyfp8_probe.so")
+    if not os.path.exists(path):
+        raise SystemExit("%s not found: build it with `python -m mdy_triton_amd.csrc.build`" % path)
+    L = ctypes.CDLL(path)
+    i64, p, i = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int
+    L.mdy_fp8_gemm_probe.argtypes = [i, i, p, p, i64, i64, p, p, p, i64, i64, i64, p]
+    L.mdy_fp8_gemm_probe.restype = i
+    return L
+
+
 def ablation(torch, m, dev):
     """The tile kernel with parts of its K loop switched off, each variant run back to back for ~1.5 s on the
     product's own operands; per launch: time, the rate the same FLOPs would mean, socket power, shader clock."""
-    from mdy_triton_amd import _lib
-    L = _lib.load()
+    L = load_probe_lib()
     names = {0: "full kernel, pre-touches on", 8: "full kernel, no pre-touches", 4: "no FMA fold (MFMAs accumulate in place)",
              2: "no LDS fragment reads", 1: "no global->LDS copies (ring replayed)", 5: "no copies, no fold",
              3: "no copies, no LDS reads", 7: "MFMA only (no copies, no LDS reads, no fold)"}
@@ -580,8 +593,10 @@ def ablation(torch, m, dev):
                                                                "constant" if const else "quantized N(0,1) x N(0,0.02)"))
             for abl in ((0, 8, 4, 2, 1, 5, 3, 7) if not const else (0, 7)):
                 def fn(abl=abl):
-                    _lib.check(L.mdy_fp8_gemm_probe(tile, abl, a_op.data_ptr(), xst.data_ptr(), 1, M, b_op.data_ptr(),
-                                                    ws.data_ptr(), c.data_ptr(), M, N, K, None), "probe")
+                    rc = L.mdy_fp8_gemm_probe(tile, abl, a_op.data_ptr(), xst.data_ptr(), 1, M, b_op.data_ptr(), ws.data_ptr(),
+                                              c.data_ptr(), M, N, K, None)
+                    if rc != 0:
+                        raise RuntimeError("mdy_fp8_gemm_probe(tile=%d, ablation=%d) returned %d" % (tile, abl, rc))
                 us, smi = sustained(torch, fn, seconds=1.5)
                 smi = smi or {}
                 print("  %-46s %8.1f us  %7.1f TFLOP/s-equivalent (%4.1f %% of peak)   %6s W   %5s MHz" % (

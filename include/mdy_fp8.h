@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define MDY_FP8_ABI_VERSION 14
+#define MDY_FP8_ABI_VERSION 15
 
 /* error codes (negative = argument rejected before any launch) */
 #define MDY_OK 0
@@ -227,10 +227,12 @@ int mdy_fp8_gemm_nt(const void* a, const float* a_s, int64_t as_row_stride, int6
                     const void* b, const float* b_s, void* c, const void* bias, int64_t M, int64_t N,
                     int64_t K, int out_dtype, void* stream);
 
-/* mdy_fp8_gemm_nt on float8_e5m2 operands (the default fp8 dtype of triton_kernels/deepseekv3/fp8_kernel.py): the MFMA tile
- * kernels with the instruction's operand format set to bf8.  Same arguments and formula; only problems with more than 64
- * rows, K % 128 == 0, K <= 65536 and 16-byte aligned a / b (MDY_E_SHAPE otherwise: run those through
- * mdy_fp8_gemm_nt_rowscaled with the weight's block scales expanded to one per row, as the Python wrapper does). */
+/* mdy_fp8_gemm_nt on float8_e5m2 operands (the default fp8 dtype of triton_kernels/deepseekv3/fp8_kernel.py:62,124,234):
+ * the MFMA kernels with the instruction's operand format set to bf8 - the tile kernels for more than 64 rows, the
+ * weight-streaming and strip kernels (or 128x128 / 64x64 tiles against a wide weight) for up to 64.  Same arguments and
+ * formula as mdy_fp8_gemm_nt; any M >= 1, but only K % 128 == 0, K <= 65536, 16-byte aligned a / b and activation scales
+ * that span less than 2^31 bytes (MDY_E_SHAPE otherwise: run those through mdy_fp8_gemm_nt_rowscaled with the weight's
+ * block scales expanded to one per row, as the Python wrapper does). */
 int mdy_fp8_gemm_nt_e5m2(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride, const void* b,
                          const float* b_s, void* c, const void* bias, int64_t M, int64_t N, int64_t K, int out_dtype,
                          void* stream);
@@ -252,20 +254,6 @@ int64_t mdy_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int mdy_fp8_gemm_nt_ws(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
                        const void* b, const float* b_s, void* c, const void* bias, int64_t M, int64_t N,
                        int64_t K, int out_dtype, void* workspace, int64_t workspace_bytes, void* stream);
-
-/* Diagnostic: one launch of the MFMA tile kernel of mdy_fp8_gemm_nt on a whole problem, optionally with parts of its
- * K loop switched off, for timing (and for reading power and clock while it runs).  No counterpart in the reference.
- *   tile      0: 256x256 tiles (what the large shapes run on)   1: 128x256 tiles
- *   ablation  0: the product's kernel, bf16 c as mdy_fp8_gemm_nt writes it (no bias).  Otherwise a set of
- *             1 no global->LDS copies inside the K loop (the LDS ring is filled once and replayed),
- *             2 no LDS fragment reads inside the loop, 4 no FMA fold of the block scales (the matrix cores
- *             accumulate in place), 8 no pre-touches of the shared panels; built: 0, 8, 1, 2, 4, 3, 5, 7.
- *             With 1, 2 or 4 in the set c is NOT the GEMM result.
- * K % 128 == 0, K <= 65536, N % 4 == 0, a / b / c 16-byte aligned; MDY_E_DTYPE for a combination that is not built.
- */
-int mdy_fp8_gemm_probe(int tile, int ablation, const void* a, const float* a_s, int64_t as_row_stride,
-                       int64_t as_col_stride, const void* b, const float* b_s, void* c, int64_t M, int64_t N,
-                       int64_t K, void* stream);
 
 /* Which kernel family mdy_fp8_gemm_nt (with_workspace = 0) or mdy_fp8_gemm_nt_ws with a sufficient workspace
  * (with_workspace = 1) runs for these operands; launches nothing, needs no GPU.  No counterpart in the reference

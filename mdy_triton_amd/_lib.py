@@ -10,7 +10,7 @@ import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libmdyfp8.so")
-ABI_VERSION = 14
+ABI_VERSION = 15
 
 _lock = threading.Lock()
 _lib = None
@@ -38,7 +38,6 @@ SIGNATURES = {
     "mdy_fp8_gemm_nt_e5m2": [_p, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p],
     "mdy_fp8_gemm_nt_ws": [_p, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p, _i64, _p],
     "mdy_fp8_gemm_workspace_bytes": [_i64, _i64, _i64],
-    "mdy_fp8_gemm_probe": [_int, _int, _p, _p, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _p],
     "mdy_fp8_gemm_path": [_p, _p, _i64, _i64, _i64, _i64, _i64, _int],
     "mdy_fp8_gemm_nt_static_ws": [_p, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p],
     "mdy_fp8_gemm_static_workspace_bytes": [],

@@ -24,10 +24,7 @@
 
 namespace mdy {
 
-#ifndef MDY_AQ_ROWS_PER_WAVE
-#define MDY_AQ_ROWS_PER_WAVE 2
-#endif
-constexpr int kAqRowsPerWave = MDY_AQ_ROWS_PER_WAVE;
+constexpr int kAqRowsPerWave = 2;
 constexpr int kAqWaves = 4;
 constexpr int kAqRowsPerBlock = kAqRowsPerWave * kAqWaves;  // 8 rows x 512 columns per block
 

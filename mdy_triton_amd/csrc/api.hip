@@ -263,7 +263,7 @@ int mdy_fp8_gemm_nt_e5m2(const void* a, const float* a_s, int64_t as_row_stride,
     const int rc = mdy::launch_fp8_gemm_nt_e5m2(a, a_s, as_row_stride, as_col_stride, b, b_s, c, bias, M, N, K, out_dtype,
                                                 static_cast<hipStream_t>(stream));
     if (rc == -1)
-        return fail(MDY_E_SHAPE, "fp8_gemm_nt_e5m2: needs more than 64 rows, K a multiple of 128 up to 65536, 16-byte aligned a and b "
+        return fail(MDY_E_SHAPE, "fp8_gemm_nt_e5m2: needs K a multiple of 128 up to 65536, 16-byte aligned a and b, activation scales within 2^31 bytes "
                     "(other e5m2 problems: mdy_fp8_gemm_nt_rowscaled with the weight scales expanded to one per row)");
     return launched(rc, "fp8_gemm_nt_e5m2");
 }
@@ -289,23 +289,6 @@ int mdy_fp8_gemm_nt_ws(const void* a, const float* a_s, int64_t as_row_stride, i
     return launched(mdy::launch_fp8_gemm_nt_ws(a, a_s, as_row_stride, as_col_stride, b, b_s, c, bias, M, N, K, out_dtype,
                                                workspace, workspace_bytes, static_cast<hipStream_t>(stream)),
                     "fp8_gemm_nt_ws");
-}
-
-int mdy_fp8_gemm_probe(int tile, int ablation, const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
-                       const void* b, const float* b_s, void* c, int64_t M, int64_t N, int64_t K, void* stream) {
-    if (M < 1 || N < 1 || K < 128 || K % 128 != 0 || K > 65536 || M > kMaxDim || N > kMaxDim)
-        return fail(MDY_E_SHAPE, "fp8_gemm_probe: needs M, N >= 1 and K a multiple of 128 up to 65536");
-    if (!a || !a_s || !b || !b_s || !c) return fail(MDY_E_NULL, "fp8_gemm_probe: null pointer");
-    if (!aligned(a, 16) || !aligned(b, 16) || !aligned(c, 16) || !aligned(a_s, 4) || !aligned(b_s, 4) || N % 4 != 0)
-        return fail(MDY_E_ALIGN, "fp8_gemm_probe: a, b, c must be 16-byte aligned and N a multiple of 4");
-    if (as_row_stride < 0 || as_col_stride < 0 ||
-        ((M - 1) * as_row_stride + (K / 128 - 1) * as_col_stride + 1) * 4 >= ((int64_t)1 << 31))
-        return fail(MDY_E_SHAPE, "fp8_gemm_probe: activation scales must span less than 2^31 bytes");
-    if (int e = check_device()) return e;
-    const int rc = mdy::launch_fp8_gemm_probe(tile, ablation, a, a_s, as_row_stride, as_col_stride, b, b_s, c, M, N, K,
-                                              static_cast<hipStream_t>(stream));
-    if (rc == -1) return fail(MDY_E_DTYPE, "fp8_gemm_probe: tile %d / ablation %d is not built", tile, ablation);
-    return launched(rc, "fp8_gemm_probe");
 }
 
 int mdy_fp8_gemm_path(const void* a, const void* b, int64_t as_row_stride, int64_t as_col_stride, int64_t M, int64_t N,

@@ -9,8 +9,12 @@ import sys
 from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SOURCES = ["api.hip", "act_quant.hip", "weight_quant.hip", "quant_transpose.hip", "swiglu.hip", "weight_dequant.hip", "fp8_gemm.hip", "gemm_probe.hip", "fp8_gemm_rowscaled.hip", "group_pad.hip", "add_bias.hip"]
+SOURCES = ["api.hip", "act_quant.hip", "weight_quant.hip", "quant_transpose.hip", "swiglu.hip", "weight_dequant.hip", "fp8_gemm.hip", "fp8_gemm_rowscaled.hip", "group_pad.hip", "add_bias.hip"]
 LIB = os.path.join(HERE, "libmdyfp8.so")
+# timing probes (ablated copies of the tile kernel, copy-only and MFMA-only ceilings): a library of its own that only
+# bench.py's diagnostic modes load
+PROBE_SOURCES = ["gemm_probe.hip"]
+PROBE_LIB = os.path.join(HERE, "libmdyfp8_probe.so")
 
 # -packed-fp32-ops: keep the compiler from forming v_pk_{add,mul,fma}_f32.
 # No fast-math: the quantizers rely on IEEE division and uncontracted FMAs.
@@ -44,18 +48,22 @@ def build(verbose: bool = False) -> str:
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
     objs = [os.path.join(objdir, s.replace(".hip", ".o")) for s in SOURCES]
+    probe_objs = [os.path.join(objdir, s.replace(".hip", ".o")) for s in PROBE_SOURCES]
 
     def compile_one(pair):
         src, obj = pair
         return _run([hipcc, *HIPCC_FLAGS, "-c", os.path.join(HERE, src), "-o", obj])
 
-    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
-        for out in ex.map(compile_one, zip(SOURCES, objs)):
+    with ThreadPoolExecutor(max_workers=8) as ex:
+        for out in ex.map(compile_one, zip(SOURCES + PROBE_SOURCES, objs + probe_objs)):
             if verbose and out.strip():
                 print(out)
     tmp = LIB + ".tmp"
     out = _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs])
     os.replace(tmp, LIB)
+    tmp = PROBE_LIB + ".tmp"
+    out += _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *probe_objs])
+    os.replace(tmp, PROBE_LIB)
     if verbose and out.strip():
         print(out)
     return LIB

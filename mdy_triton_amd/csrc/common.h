@@ -287,8 +287,6 @@ int64_t fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int launch_fp8_gemm_nt_ws(const void* a, const float* a_s, int64_t as_row_stride, int64_t as_col_stride,
                           const void* b, const float* b_s, void* c, const void* bias, int64_t M, int64_t N,
                           int64_t K, int out_dtype, void* workspace, int64_t workspace_bytes, hipStream_t stream);
-int launch_fp8_gemm_probe(int tile, int ablation, const void* a, const float* a_s, int64_t as_rs, int64_t as_cs,
-                          const void* b, const float* b_s, void* c, int64_t M, int64_t N, int64_t K, hipStream_t stream);
 int fp8_gemm_path(const void* a, const void* b, int64_t as_rs, int64_t as_cs, int64_t M, int64_t N, int64_t K,
                   int with_workspace);
 // static device scratch of the no-allocation GEMM entry point (defined in fp8_gemm.hip)

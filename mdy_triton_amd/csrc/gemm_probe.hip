@@ -2,7 +2,8 @@
 // It exists so that the cost of each part (global->LDS copies, LDS fragment reads, the FMA fold of the block
 // scales, the pre-touches) can be measured on the product's own code, with the product's own operands, and the
 // power / clock readings taken while it runs; the results of a probe with anything switched off are NOT a GEMM.
-// No counterpart in the reference.
+// No counterpart in the reference.  Built into libmdyfp8_probe.so, which only `bench.py --ablation` loads: it is not
+// part of libmdyfp8.so and has no declaration in include/mdy_fp8.h.
 #include "fp8_gemm_tile.h"
 
 namespace mdy {
@@ -21,7 +22,7 @@ static int probe_launch(const uint8_t* a, const float* a_s, int as_rs, int as_cs
 // tile: 0 = 256x256 (ring of 2 K blocks), 1 = 128x256 (ring of 3).  ablation: bit set of
 // 1 no copies in the loop, 2 no LDS reads, 4 no FMA fold, 8 no pre-touches; the combinations built are
 // 0, 8, 1, 2, 4, 3, 5, 7 (0 and 8 give the exact GEMM result).  Returns -1 for a combination that is not built.
-int launch_fp8_gemm_probe(int tile, int ablation, const void* a, const float* a_s, int64_t as_rs, int64_t as_cs,
+static int launch_fp8_gemm_probe(int tile, int ablation, const void* a, const float* a_s, int64_t as_rs, int64_t as_cs,
                           const void* b, const float* b_s, void* c, int64_t M, int64_t N, int64_t K, hipStream_t stream) {
     const int KB = (int)(K / 128);
     const int64_t as_extent = ((M - 1) * as_rs + (int64_t)(KB - 1) * as_cs + 1) * 4;
@@ -55,3 +56,17 @@ int launch_fp8_gemm_probe(int tile, int ablation, const void* a, const float* a_
 }
 
 }  // namespace mdy
+
+// Entry point of the probe library.  K % 128 == 0, K <= 65536, N % 4 == 0, a / b / c 16-byte aligned, activation scales
+// within 2^31 bytes; returns 0, a hipError_t, -1 for a tile / ablation pair that is not built, -2 for bad arguments.
+extern "C" int mdy_fp8_gemm_probe(int tile, int ablation, const void* a, const float* a_s, int64_t as_row_stride,
+                                  int64_t as_col_stride, const void* b, const float* b_s, void* c, int64_t M, int64_t N,
+                                  int64_t K, void* stream) {
+    if (M < 1 || N < 1 || K < 128 || K % 128 != 0 || K > 65536 || N % 4 != 0 || !a || !a_s || !b || !b_s || !c) return -2;
+    if (((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c)) & 15) != 0) return -2;
+    if (as_row_stride < 0 || as_col_stride < 0 ||
+        ((M - 1) * as_row_stride + (K / 128 - 1) * as_col_stride + 1) * 4 >= ((int64_t)1 << 31))
+        return -2;
+    return mdy::launch_fp8_gemm_probe(tile, ablation, a, a_s, as_row_stride, as_col_stride, b, b_s, c, M, N, K,
+                                      static_cast<hipStream_t>(stream));
+}

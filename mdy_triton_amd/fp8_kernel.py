@@ -237,17 +237,20 @@ def fp8_matmul(x: torch.Tensor, w: torch.Tensor, scale_x: torch.Tensor, scale_w:
             M, K = x2.shape
             N = w.size(0)
             x2c, wc = (x2 if x2.is_contiguous() else x2.contiguous()), (w if w.is_contiguous() else w.contiguous())
-            if M > 64 and K <= 65536 and x2c.data_ptr() % 16 == 0 and wc.data_ptr() % 16 == 0:
-                # e5m2 on the tuned tile kernels (the MFMA's operand format set to bf8)
+            sxc, swc = sx2.contiguous(), scale_w.contiguous()
+            scales_ok = M == 0 or ((M - 1) * sxc.stride(0) + K // 128) * 4 < (1 << 31)
+            if K <= 65536 and scales_ok and x2c.data_ptr() % 16 == 0 and wc.data_ptr() % 16 == 0:
+                # e5m2 on the MFMA kernels (operand format bf8): tile kernels, or the weight-streaming / strip kernels
+                # for up to 64 rows
                 fused = bias is not None and bias.dtype == torch.bfloat16
-                sxc, swc = sx2.contiguous(), scale_w.contiguous()
                 y = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
                 with on_device(dev):
                     check(lib().mdy_fp8_gemm_nt_e5m2(ptr(x2c), ptr(sxc), sxc.stride(0), 1, ptr(wc), ptr(swc), ptr(y),
                                                      ptr(bias.contiguous()) if fused else None, M, N, K, 0, stream_ptr(dev)),
                           "fp8_matmul")
             else:
-                # few rows: the GEMM with row scales on both operands, the weight's block scales expanded to one per row
+                # K beyond 65536, unaligned operands or scales spanning 2^31 bytes: the GEMM with row scales on both
+                # operands, the weight's block scales expanded to one per row
                 fused = False
                 sw_rows = scale_w.repeat_interleave(128, dim=0)[:N].contiguous()
                 y = _matmul_rowscaled(x2, sx2, w, sw_rows, M, N, K, dev, fmt)

@@ -107,8 +107,8 @@ def test_rowscaled_gemm_random_and_ragged_k():
     assert L.mdy_fp8_gemm_nt_rowscaled(p, p, -1, 1, p, p, 1, 1, p, 4, 4, 128, 0, 0, None) == -2
     assert L.mdy_fp8_gemm_nt_rowscaled(p, p, 1, 1, p, p, 1, 1, p, 4, 4, 128, 5, 0, None) == -4
     assert L.mdy_act_quant_transpose(p, 0, None, p, p, p, 4, 128, 128, 1, 128, 128, 0, None) == -1
-    assert L.mdy_act_quant_transpose(p, 7, p, p, p, p, 4, 128, 128, 1, 128, 128, 0, None)
-    assert L.mdy_act_quant_transpose(p, 0, p, p, p, p, 4, 128, 128, 1, 128, 128, 1, None) == -4 == -4
+    assert L.mdy_act_quant_transpose(p, 7, p, p, p, p, 4, 128, 128, 1, 128, 128, 0, None) == -4     # unknown x_dtype
+    assert L.mdy_act_quant_transpose(p, 0, p, p, p, p, 4, 128, 128, 1, 128, 128, 1, None) == -4     # mode 1 is not built
 
 
 @pytest.mark.parametrize("bias", [True, False])
@@ -421,9 +421,72 @@ def test_e5m2_tile_kernels_exact_integer(M, N, K):
     bias = torch.randint(-8, 9, (N,), generator=g).float().bfloat16()
     got = FK.fp8_matmul(a, b, a_s, b_s, bias.to(DEV))
     assert torch.equal(got.cpu().double(), (exact + bias.double()).to(torch.bfloat16).double())
-    # what the entry point does not take is refused, not mis-run
-    assert L.mdy_fp8_gemm_nt_e5m2(a.data_ptr(), a_s.data_ptr(), KB, 1, b.data_ptr(), b_s.data_ptr(), out.data_ptr(), None, 64, N, K, 1,
+    # what the entry point does not take is refused, not mis-run: K not a multiple of 128, an unaligned operand
+    assert L.mdy_fp8_gemm_nt_e5m2(a.data_ptr(), a_s.data_ptr(), KB, 1, b.data_ptr(), b_s.data_ptr(), out.data_ptr(), None, M, N, K - 64, 1,
                                   None) == -2
+    assert L.mdy_fp8_gemm_nt_e5m2(a.data_ptr() + 8, a_s.data_ptr(), KB, 1, b.data_ptr(), b_s.data_ptr(), out.data_ptr(), None, M - 1, N, K,
+                                  1, None) == -2
+
+
+# (M, N, K) -> the branch of the <= 64-row dispatch it lands in
+E5M2_SMALL = [(1, 512, 256), (5, 512, 384), (16, 520, 256), (17, 512, 256), (33, 512, 256), (64, 512, 256),      # weight streaming, one column group, rows split over grid.y from 17 on
+              (48, 3600, 256), (64, 3200, 128),                                                                  # weight streaming, 3 and 4 row sub-tiles per workgroup
+              (5, 16384, 256), (17, 9216, 256), (31, 9216, 128),                                                   # two column groups per workgroup
+              (5, 25600, 256), (16, 25600, 128), (33, 25616, 256), (64, 25600, 128),                               # strip kernel
+              (48, 16384, 256), (33, 16400, 128),                                                                  # 128x128 tiles
+              (48, 6400, 256), (64, 6404, 128)]                                                                    # 64x64 tiles
+
+
+@pytest.mark.parametrize("M,N,K", E5M2_SMALL)
+def test_e5m2_small_m_exact_integer(M, N, K):
+    """e5m2 operands, up to 64 rows: every branch of the small-M dispatch (weight streaming with one and two column
+    groups, the strip kernel, 128x128 and 64x64 tiles against a wide weight), exact on integer operands with power-of-two
+    scales; fp32 and bf16 output, bias in the epilogue, through the C entry point and through fp8_matmul."""
+    from mdy_triton_amd import _lib
+    g = torch.Generator().manual_seed(7 * M + N + K)
+    ai = torch.randint(-4, 5, (M, K), generator=g)
+    bi = torch.randint(-4, 5, (N, K), generator=g)
+    KB, NB = K // 128, (N + 127) // 128
+    ae = torch.randint(-2, 3, (M, KB), generator=g)
+    be = torch.randint(-2, 3, (NB, KB), generator=g)
+    exact = torch.zeros(M, N, dtype=torch.float64)
+    for kb in range(KB):
+        exact += (ai[:, kb * 128:(kb + 1) * 128].double() @ bi[:, kb * 128:(kb + 1) * 128].double().t()) * \
+            torch.exp2((ae[:, kb][:, None] + be[torch.arange(N) // 128, kb][None, :]).double())
+    a, b = ai.float().to(E5M2).to(DEV), bi.float().to(E5M2).to(DEV)
+    a_s, b_s = torch.exp2(ae.float()).to(DEV), torch.exp2(be.float()).to(DEV)
+    bias = torch.randint(-8, 9, (N,), generator=g).float().bfloat16()
+    L = _lib.load()
+    out = torch.full((M, N), float("nan"), device=DEV)
+    assert L.mdy_fp8_gemm_nt_e5m2(a.data_ptr(), a_s.data_ptr(), KB, 1, b.data_ptr(), b_s.data_ptr(), out.data_ptr(), None, M, N, K, 1,
+                                  None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu().double(), exact)
+    # column-major activation scales (the layout quant_input returns), fp32 out with the bias
+    a_st = a_s.t().contiguous()
+    out = torch.full((M, N), float("nan"), device=DEV)
+    bias_d = bias.to(DEV)
+    assert L.mdy_fp8_gemm_nt_e5m2(a.data_ptr(), a_st.data_ptr(), 1, M, b.data_ptr(), b_s.data_ptr(), out.data_ptr(), bias_d.data_ptr(), M,
+                                  N, K, 1, None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu().double(), exact + bias.double())
+    got = FK.fp8_matmul(a, b, a_s, b_s, bias_d)
+    assert got.dtype == torch.bfloat16 and torch.equal(got.cpu().double(), (exact + bias.double()).to(torch.bfloat16).double())
+    got = FK.fp8_matmul(a, b, a_s, b_s)
+    assert torch.equal(got.cpu().double(), exact.to(torch.bfloat16).double())
+
+
+def test_e5m2_small_m_realistic_against_oracle():
+    """Decode-sized e5m2 GEMMs on quantized Gaussian data against the oracle's dequantize-then-matmul (rtol = atol = 1e-2)."""
+    g = torch.Generator().manual_seed(99)
+    for M, N, K in [(1, 7168, 2048), (16, 2048, 7168), (64, 7168, 2048), (40, 25600, 512)]:
+        x = torch.randn(M, K, generator=g).bfloat16()
+        w = (torch.randn(N, K, generator=g) * 0.02).bfloat16()
+        xq, xs = O.act_quant_block(x, dtype=E5M2)
+        wq, ws = O.weight_quant_block(w, dtype=E5M2)
+        ref = O.fp8_gemm(xq, xs, wq, ws, dtype=torch.bfloat16)
+        got = FK.fp8_matmul(xq.to(DEV), wq.to(DEV), xs.to(DEV), ws.to(DEV))
+        assert close(got, ref), (M, N, K)
 
 
 def test_act_quant_block_e5m2_golden_codes_on_device():
