@@ -28,7 +28,9 @@
 //   * workgroup ids are remapped so that the 32 workgroups that share an XCD's L2
 //     cover a compact 4 x 8 block of tiles.
 // Tile sizes from 64x64 to 256x256 share that body; the host picks by tile count, and with a
-// workspace also splits K (fp8_gemm_splitk_kernel + splitk_reduce_kernel).
+// workspace also splits K (fp8_gemm_splitk_kernel + splitk_reduce_kernel).  The 128x192 tile (mid-size
+// shapes whose 128x256 tiles would leave a quarter of the CUs idle) runs a second body with producer and
+// consumer waves (fp8_gemm_tile_ws in fp8_gemm_tile.h).
 // Small-M kernel (M <= 64): weight streaming, one workgroup of 8 waves per 16 columns,
 // waves split K (next block prefetched) and reduce through LDS.  Strip kernel: 5..64 rows against
 // many 128-column strips.  Scalar kernel: any other shape/alignment.
@@ -502,7 +504,7 @@ static bool big_tiles_pay(int64_t M, int64_t N) {
 //   0: 128x128, 2 K blocks in LDS (two workgroups share a CU)   1: 128x128, 4 K blocks (one workgroup per CU)
 //   2: 128x64, 6 K blocks                                       3: 64x64, 8 K blocks
 //   4: 128x256, 3 K blocks, 8 waves                             5: 256x128, 3 K blocks, 8 waves
-//   6: 128x192, 3 K blocks, 8 waves (wave tile 64x48)
+//   6: 128x192, 4 consumer waves (wave tile 64x96) + 4 producer waves, 2 K blocks in flight
 // Measured rule: the smallest tile that still gives every workgroup a CU of its own (the time of these
 // shapes goes with the bytes each CU has to pull, not with its MFMAs), and the ring as deep as LDS allows.
 // Between 257 and 512 tiles of 128x128 that is a 128x256 tile (else, if those are too many, 256x128), one per CU,
@@ -518,7 +520,9 @@ static int few_tiles_config(int M, int N, int K) {
     if (K < 1024) return 0;    // a handful of K blocks: two short workgroups per CU hide each other's prologue and epilogue
     const long wide = rows128 * cols256, tall = rows256 * cols128;
     // more 128x256 tiles than 3/4 of the CUs and 128x192 tiles still one per CU: the smaller tile puts the idle CUs to
-    // work (4096x1536x7168: 256 tiles of 128x192 instead of 192 of 128x256)
+    // work (4096x1536x7168: 256 tiles of 128x192 instead of 192 of 128x256), and its wave tiles are small enough for
+    // the producer / consumer kernel (measured at that shape, same process, relaunched back to back: 59.5 -> 49.7 us
+    // with row-major scales, 54.8 -> 47.3 us with column-major ones; after a cache flush 61.7 -> 57.8 us)
     if (wide <= cus && rows128 * ((N + 191) / 192) <= cus && rows128 * ((N + 191) / 192) > wide) return 6;
     if (wide <= cus) return 4;    // also when it pads more than the tall tile: 12800x384x7168 82 against 95 us
     if (tall <= cus) return 5;
@@ -628,7 +632,13 @@ static int dispatch_tiles(const uint8_t* a, const float* a_s, int64_t as_rs, int
         case 3: MDY_FEW(64, 64, 2, 2, 8);
         case 4: MDY_FEW(128, 256, 2, 4, 3);
         case 5: MDY_FEW(256, 128, 2, 4, 3);
-        case 6: MDY_FEW(128, 192, 2, 4, 3);
+        case 6: {
+            const int tiles_m = (M + 127) / 128, tiles_n = (N + 191) / 192;
+            hipLaunchKernelGGL((fp8_gemm_ws_kernel<128, 192, 2, 2, 4, 4, OUT, FMT>), dim3((unsigned)(tiles_m * tiles_n)), dim3(512), 0,
+                               stream, a, a_s, (int)as_rs, (int)as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, tiles_m,
+                               tiles_n, pretouch_enabled() ? 1 : 0);
+            return (int)hipGetLastError();
+        }
         default: MDY_FEW(128, 128, 2, 2, 2);
     }
 #undef MDY_FEW

@@ -1,6 +1,7 @@
 // The MFMA tile body of the block-scaled FP8 GEMM and the kernel that walks tiles with it (gfx950 only).
 // Shared by fp8_gemm.hip (the product kernels) and gemm_probe.hip (the timing probe that switches parts of the
-// K loop off); the description of the kernel is at the top of fp8_gemm.hip.
+// K loop off); the description of the kernels is at the top of fp8_gemm.hip.  Two bodies: fp8_gemm_tile (every wave
+// does everything; the large tiles) and fp8_gemm_tile_ws (producer / consumer waves; 128x192 tiles).
 #pragma once
 #include "common.h"
 
@@ -94,6 +95,19 @@ struct TileLds {
     static constexpr int s_off = b_off + STAGES * BN * 128;
     static constexpr int bs_off = s_off + (STAGES * BM * 4 + 255) / 256 * 256;
     static constexpr int dummy_off = bs_off + NBS * 512 * 4;
+    static constexpr int bytes = dummy_off + WAVES * 512;
+};
+
+// LDS of a wave-specialized tile workgroup: separate ring depths for the a panels, the b panels and the activation scales.
+template <int BM, int BN, int WAVES, int SA, int SB, int SS>
+struct TileLdsWs {
+    static constexpr int NBS = (BN + 127) / 128;
+    static constexpr int BSROW = 512;
+    static constexpr int a_off = 0;
+    static constexpr int b_off = a_off + SA * BM * 128;
+    static constexpr int s_off = b_off + SB * BN * 128;
+    static constexpr int bs_off = s_off + (SS * BM * 4 + 255) / 256 * 256;
+    static constexpr int dummy_off = bs_off + NBS * BSROW * 4;
     static constexpr int bytes = dummy_off + WAVES * 512;
 };
 
@@ -450,6 +464,271 @@ __device__ __forceinline__ Duty tile_of(int local, int tiles_m, int tiles_n, int
     d.b_duty = in_group & ((1 << d.b_sh) - 1);
     d.a_duty = tn & ((1 << d.a_sh) - 1);
     return d;
+}
+
+// The tile with SPECIALIZED waves and the barrier of a K block EARLY in the block, for small wave tiles.
+// In fp8_gemm_tile every wave copies, reads fragments, issues MFMAs and folds, and the one barrier of a K block sits in
+// front of its last streamed fragment: behind it every wave reloads the held fragments, the first streamed fragment and the
+// scales of the next block from LDS with only NH MFMAs left to cover that latency, and every buffer_load ... lds stays at
+// the head of its (in-order) wave until the CU's address unit takes it, holding back the MFMAs queued behind it.  With a
+// 256x256 tile both are a small part of a K block; with 64x96 wave tiles on a 128x192 tile, in-kernel clocks at
+// 4096x1536x7168 showed 560-730 of ~1700 clocks per K block behind the barrier for 4 of 12 MFMAs, 40 clocks per MFMA slot
+// without a copy near it and 60 with one every second slot.  Here:
+//   * the first WGM x WGN waves ("consumers") run the MFMAs, the LDS reads and the fold and never touch global memory in the
+//     K loop; PW further waves ("producers") do nothing but the global->LDS copies and the pre-touches (small wave tiles
+//     leave registers for the second set of waves: all waves of a workgroup get the same allocation);
+//   * the barrier of block kb is at slot E, a few MFMAs into the block.  For a consumer it says "I have left block kb-1";
+//     a producer first waits for its own copies of block kb+1.  Behind it the consumers read block kb+1's held fragments,
+//     first streamed fragment and scales from LDS into a SECOND set of registers, spread over the slots (block kb+1 then
+//     starts on registers loaded a dozen slots earlier; the K loop is unrolled by two so that the sets swap without
+//     moves), and the producers copy block kb+STAGES-1 and touch the lines of a later block;
+//   * the held operand of block kb is read during block kb-1, the streamed operand during block kb itself: the held
+//     operand's buffer is free one block earlier, so its ring is one buffer shorter (STAGES-1) than the streamed operand's
+//     (STAGES) for the same STAGES-2 blocks in flight.  The activation scales follow the held operand;
+//   * on the 192-wide tile a wave's columns can straddle two 128-column blocks of weight scales: the combined scale is
+//     kept per row and 32-column group (multiplies once per block instead of a select per MFMA).
+// Swizzle, fragment layout, fold, epilogue and pre-touch shares are fp8_gemm_tile's.
+template <int BM, int BN, int WGM, int WGN, int PW, int STAGES, typename OUT, int FMT_ = 0, int E_ = 2>
+__device__ __forceinline__ void fp8_gemm_tile_ws(
+    const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
+    const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
+    const uint16_t* __restrict__ bias, int m0, int m_end, int m_total, int n0, int N, int K, int ldc, const Duty duty,
+    int kb0, int kb1, uint8_t* __restrict__ pool) {
+    constexpr int CW = WGM * WGN;                       // consumer waves
+    constexpr int WM = BM / WGM, WN = BN / WGN, TI = WM / 16, TJ = WN / 16;
+    constexpr int PASS_ROWS = PW * 8;                   // rows copied by one instruction of every producer
+    constexpr int A_PASSES = BM / PASS_ROWS, B_PASSES = BN / PASS_ROWS;
+    constexpr int S_WAVES = BM / 64;                    // producers that also copy the activation scales
+    constexpr int DEPTH = 4;
+    static_assert(BM % PASS_ROWS == 0 && BN % PASS_ROWS == 0 && PASS_ROWS % 16 == 0, "tile/threads mismatch");
+    constexpr bool STRADDLE = (128 % WN) != 0;
+    static_assert(WN <= 128 && (!STRADDLE || BN == 192) && S_WAVES <= PW && PW >= 2, "weight-scale blocks per wave column");
+    constexpr bool HOLD_A = TI <= TJ;
+    constexpr int NH = HOLD_A ? TI : TJ, NS = HOLD_A ? TJ : TI;
+    constexpr int NT = TI * TJ;
+    constexpr int SC = 1;                               // scale copies per K block and producer
+    constexpr int NDMA = SC + A_PASSES + B_PASSES;
+    constexpr int E = E_;
+    constexpr int TDA = 2;
+    static_assert(STAGES >= 4 && (STAGES - 2) * (NDMA + 1) + 1 <= 63, "streamed ring of at least 4 K blocks; vmcnt is a 6-bit counter");
+    constexpr int SA = HOLD_A ? STAGES - 1 : STAGES, SB = HOLD_A ? STAGES : STAGES - 1;   // ring depths of a and b
+    constexpr int SS = STAGES - 1;                                                        // ring depth of the activation scales
+    // loads younger than the last copy of block kb+1 at the barrier of block kb: the touch behind those copies and the
+    // copies + touches of blocks kb+2 .. kb+STAGES-2
+    constexpr int YOUNGER = (STAGES - 3) * (NDMA + 1) + 1;
+    static_assert(NS % 2 == 0 && NS >= 2, "the first streamed fragment of the next K block reuses queue slot 0");
+    constexpr int PWIN = NT - 2 - (E + 1);
+    static_assert(E >= 0 && E < NT - NH && PWIN >= NH, "barrier slot");
+
+    using L = TileLdsWs<BM, BN, CW + PW, SA, SB, SS>;
+    constexpr int NBS = L::NBS;
+    uint8_t(*lds_a)[BM * 128] = reinterpret_cast<uint8_t(*)[BM * 128]>(pool + L::a_off);
+    uint8_t(*lds_b)[BN * 128] = reinterpret_cast<uint8_t(*)[BN * 128]>(pool + L::b_off);
+    float(*lds_s)[BM] = reinterpret_cast<float(*)[BM]>(pool + L::s_off);
+    float(*lds_bs)[L::BSROW] = reinterpret_cast<float(*)[L::BSROW]>(pool + L::bs_off);
+    uint8_t* lds_dummy = pool + L::dummy_off;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int M = m_end;
+    const int KB = K >> 7;
+
+    if (wave >= CW) {
+        // ------------------------------------------------------------------ producer
+        const int pw = wave - CW;
+        const int prow = pw * 8 + (lane >> 3);
+        const int voff = prow * K + (((lane & 7) ^ swz(prow)) << 4);
+        intx4 rs = make_rsrc(a_s, as_bytes);
+        if (pw >= S_WAVES) rs[2] = 0;
+        const uint32_t ld_base = lds_addr(&lds_dummy[0]) + wave * 512;
+        const uint32_t la_base = lds_addr(&lds_a[0][0]) + pw * 1024;
+        const uint32_t lb_base = lds_addr(&lds_b[0][0]) + pw * 1024;
+        const uint32_t ls_base = pw < S_WAVES ? lds_addr(&lds_s[0][0]) + pw * 256 : ld_base;
+        const uint32_t ls_buf = pw < S_WAVES ? BM * 4 : 0;
+        const intx4 ra = make_rsrc(a + (size_t)m0 * K, (uint32_t)min(BM, M - m0) * (uint32_t)K);
+        const intx4 rb = make_rsrc(b + (size_t)n0 * K, (uint32_t)min(BN, N - n0) * (uint32_t)K);
+        const int s_voff = min(m0 + (pw % S_WAVES) * 64 + lane, m_total - 1) * as_rs * 4;
+        const bool touch_b = (pw & 1) == 0;
+        const int t_idx = (pw >> 1) * 64 + lane;
+        const int share = touch_b ? (BN >> duty.b_sh) : (BM >> duty.a_sh);
+        intx4 rt = touch_b ? rb : ra;
+        if ((pw >> 1) * 64 >= share || (touch_b ? duty.b_sh : duty.a_sh) == 0) rt[2] = 0;
+        const int touch_off = ((touch_b ? duty.b_duty : duty.a_duty) * share + t_idx % share) * K;
+        auto issue = [&](int i, int kb, int bufa, int bufb, int bufs) {
+            const bool more = kb < kb1;
+            if (i < SC)
+                dma4(rs, s_voff, more ? kb * as_cs * 4 : (int)as_bytes, ls_base + bufs * ls_buf);
+            else if (i < SC + A_PASSES)
+                dma16(ra, voff, (i - SC) * PASS_ROWS * K + (more ? kb * 128 : ra[2]), la_base + bufa * (BM * 128) + (i - SC) * PASS_ROWS * 128);
+            else
+                dma16(rb, voff, (i - SC - A_PASSES) * PASS_ROWS * K + (more ? kb * 128 : rb[2]),
+                      lb_base + bufb * (BN * 128) + (i - SC - A_PASSES) * PASS_ROWS * 128);
+        };
+        auto touch = [&](int kb) { dma4(rt, touch_off, kb < kb1 ? kb * 128 : rt[2], ld_base + 256); };
+
+        if (pw < NBS) {
+            const int nb = min((n0 >> 7) + pw, ((N + 127) >> 7) - 1);
+            const intx4 rbs = make_rsrc(b_s + (size_t)nb * KB, (uint32_t)KB * 4u);
+            for (int cc = 0; cc < KB; cc += 64) dma4(rbs, lane * 4, cc * 4, lds_addr(&lds_bs[pw][cc]));
+        }
+#pragma unroll
+        for (int blk = 0; blk < STAGES - 1; ++blk) {
+#pragma unroll
+            for (int i = 0; i < NDMA; ++i) issue(i, kb0 + blk, blk % SA, blk % SB, blk % SS);
+            touch(kb0 + blk + TDA);
+        }
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 2) * (NDMA + 1) + 1) : "memory");    // block kb0 has landed
+        __syncthreads();
+        // buffers of block kb+STAGES-1 in the three rings (kb = kb0: block index STAGES-1)
+        int fa = (STAGES - 1) % SA, fb = (STAGES - 1) % SB, fs = (STAGES - 1) % SS;
+        for (int kb = kb0; kb < kb1; ++kb) {
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(YOUNGER) : "memory");   // this wave's copies of block kb+1 have landed
+            __syncthreads();                                                   // every consumer has left block kb-1
+#pragma unroll
+            for (int i = 0; i < NDMA; ++i) issue(i, kb + STAGES - 1, fa, fb, fs);
+            touch(kb + STAGES - 1 + TDA);
+            fa = fa + 1 == SA ? 0 : fa + 1;
+            fb = fb + 1 == SB ? 0 : fb + 1;
+            fs = fs + 1 == SS ? 0 : fs + 1;
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing may still be writing LDS when the wave ends
+        return;
+    }
+
+    // ---------------------------------------------------------------------- consumer
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int frow = lane & 15, fk = lane >> 4;
+    const int a_rd0 = (wm * WM + frow) * 128 + (((2 * fk) ^ swz(frow)) << 4);
+    const int a_rd1 = (wm * WM + frow) * 128 + (((2 * fk + 1) ^ swz(frow)) << 4);
+    const int b_rd0 = (wn * WN + frow) * 128 + (((2 * fk) ^ swz(frow)) << 4);
+    const int b_rd1 = (wn * WN + frow) * 128 + (((2 * fk + 1) ^ swz(frow)) << 4);
+    const int h0 = HOLD_A ? a_rd0 : b_rd0, h1 = HOLD_A ? a_rd1 : b_rd1;
+    const int x0 = HOLD_A ? b_rd0 : a_rd0, x1 = HOLD_A ? b_rd1 : a_rd1;
+    const int s_rd = wm * WM + frow;
+    const int bs_col = (n0 & 127) + wn * WN;
+    // A wave's columns lie in one 128-column block of weight scales, except on the 192-wide tile (WN = 96 or 48): there
+    // every group of GW columns does (GW = 32 or 16 divides the possible offsets), so the combined scale is kept per row
+    // and column group: NG multiplies per row and K block instead of one select per MFMA.
+    constexpr int GW = STRADDLE ? ((WN % 32 == 0) ? 32 : 16) : WN, NG = WN / GW, JPG = GW / 16;
+    const float* my_bs[NG];
+#pragma unroll
+    for (int g = 0; g < NG; ++g) my_bs[g] = lds_bs[(bs_col + g * GW) >> 7];
+
+    floatx4 acc[TI][TJ];
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    auto read_frag = [&](const uint8_t* base, int rd0, int rd1, int idx) {
+        const intx4 lo = *reinterpret_cast<const intx4*>(base + rd0 + idx * 2048);
+        const intx4 hi = *reinterpret_cast<const intx4*>(base + rd1 + idx * 2048);
+        return intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    };
+
+    __syncthreads();                                     // block kb0, the weight scales have landed
+    intx8 fh_a[NH], fh_b[NH], fx[2];
+    float sc_a[TI][NG], sc_b[TI][NG];
+#pragma unroll
+    for (int h = 0; h < NH; ++h) fh_a[h] = read_frag(HOLD_A ? lds_a[0] : lds_b[0], h0, h1, h);
+#pragma unroll
+    for (int i = 0; i < TI; ++i) {
+        const float sa = lds_s[0][s_rd + i * 16];
+#pragma unroll
+        for (int g = 0; g < NG; ++g) sc_a[i][g] = sa * my_bs[g][kb0];
+    }
+    fx[0] = read_frag(HOLD_A ? lds_b[0] : lds_a[0], x0, x1, 0);
+
+    // buffers of K block kb in the ring of the held operand (and of the scales) / of the streamed operand
+    int ch = 0, cx = 0;
+    auto block = [&](intx8(&fh)[NH], intx8(&fhn)[NH], float(&sc)[TI][NG], float(&scn)[TI][NG], int kb) {
+        const int nh = ch + 1 == STAGES - 1 ? 0 : ch + 1;     // block kb+1, held ring
+        const int nx = cx + 1 == STAGES ? 0 : cx + 1;         // block kb+1, streamed ring
+        const uint8_t* lx = HOLD_A ? lds_b[cx] : lds_a[cx];
+        const uint8_t* lh_n = HOLD_A ? lds_a[nh] : lds_b[nh];
+        const uint8_t* lx_n = HOLD_A ? lds_b[nx] : lds_a[nx];
+        const float* ls_n = lds_s[nh];
+        floatx4 p[DEPTH + 1];
+#pragma unroll
+        for (int t = 0; t < NT + DEPTH; ++t) {
+            if (t < NT) {
+                const int si = t / NH, h = t % NH;
+                if (h == 0 && si + 1 < NS) fx[(si + 1) & 1] = read_frag(lx, x0, x1, si + 1);
+                if (h == 0 && si + 1 == NS) fx[0] = read_frag(lx_n, x0, x1, 0);      // first streamed fragment of block kb+1
+                const intx8 fa_ = HOLD_A ? fh[h] : fx[si & 1];
+                const intx8 fb_ = HOLD_A ? fx[si & 1] : fh[h];
+                p[t % (DEPTH + 1)] = mfma_block<FMT_>(fb_, fa_);
+                if (t == E) __syncthreads();
+                if (t == E + 1) {
+                    float sbg[NG];
+#pragma unroll
+                    for (int g = 0; g < NG; ++g) sbg[g] = my_bs[g][min(kb + 1, KB - 1)];
+#pragma unroll
+                    for (int i = 0; i < TI; ++i) {
+                        const float sa = ls_n[s_rd + i * 16];
+#pragma unroll
+                        for (int g = 0; g < NG; ++g) scn[i][g] = sa * sbg[g];
+                    }
+                }
+#pragma unroll
+                for (int hh = 0; hh < NH; ++hh)
+                    if (t == E + 1 + (hh * PWIN) / NH) fhn[hh] = read_frag(lh_n, h0, h1, hh);
+            }
+            if (t >= DEPTH) {
+                const int u = t - DEPTH, si = u / NH, h = u % NH;
+                const int i = HOLD_A ? h : si, j = HOLD_A ? si : h;
+                fold(acc[i][j], p[u % (DEPTH + 1)], sc[i][j / JPG]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        ch = nh;
+        cx = nx;
+    };
+    {
+        int kb = kb0;
+        for (; kb + 1 < kb1; kb += 2) {
+            block(fh_a, fh_b, sc_a, sc_b, kb);
+            block(fh_b, fh_a, sc_b, sc_a, kb + 1);
+        }
+        if (kb < kb1) block(fh_a, fh_b, sc_a, sc_b, kb);     // odd number of K blocks
+    }
+
+    const bool vec_ok = (ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
+#pragma unroll
+    for (int i = 0; i < TI; ++i) {
+        const int m = m0 + wm * WM + i * 16 + frow;
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+            const int n = n0 + wn * WN + j * 16 + 4 * fk;
+            float v[4] = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+            if (bias != nullptr) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (n + e < N) v[e] += bf16_one(bias[n + e]);
+            }
+            store4<OUT>(c, ldc, m, n, M, N, v, vec_ok);
+        }
+    }
+}
+
+// the wave-specialized tile as a kernel: one workgroup of WGM*WGN + PW waves per tile (or per several, walked in turn)
+template <int BM, int BN, int WGM, int WGN, int PW, int STAGES, typename OUT, int FMT_ = 0, int E_ = 2>
+__global__ __launch_bounds__((WGM * WGN + PW) * 64) void fp8_gemm_ws_kernel(
+    const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
+    const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
+    const uint16_t* __restrict__ bias, int M, int N, int K, int ldc, int tiles_m, int tiles_n, int pretouch) {
+    constexpr bool HOLD_A = BM / WGM <= BN / WGN;
+    __shared__ __attribute__((aligned(1024)))
+    uint8_t pool[TileLdsWs<BM, BN, WGM * WGN + PW, HOLD_A ? STAGES - 1 : STAGES, HOLD_A ? STAGES : STAGES - 1, STAGES - 1>::bytes];
+    const int ntiles = tiles_m * tiles_n;
+    for (int pid = blockIdx.x; pid < ntiles; pid += gridDim.x) {
+        int tm, tn;
+        Duty duty = tile_of(xcd_contiguous(pid, ntiles), tiles_m, tiles_n, tm, tn);
+        if (!pretouch) duty.a_sh = duty.b_sh = 0;
+        fp8_gemm_tile_ws<BM, BN, WGM, WGN, PW, STAGES, OUT, FMT_, E_>(a, a_s, as_rs, as_cs, as_bytes, b, b_s, c, bias, tm * BM, M, M,
+                                                                            tn * BN, N, K, ldc, duty, 0, K >> 7, pool);
+        __syncthreads();
+    }
 }
 
 template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT, int GAP_ = 0, int TD_ = 0, int ABL_ = 0, int FMT_ = 0>

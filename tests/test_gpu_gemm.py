@@ -89,6 +89,34 @@ def test_gemm_exact_integer_few_tiles_configs(M, N, K):
     test_gemm_exact_integer_cases_all_kernels(M, N, K)
 
 
+@pytest.mark.parametrize("M,N,K", [(4096, 1536, 7168), (4000, 1531, 1152), (2048, 3000, 1408), (3900, 1345, 1024)])
+def test_gemm_exact_integer_producer_consumer_tiles(M, N, K):
+    """The 128x192 producer / consumer kernel through the C entry point: column-major activation scales (the layout
+    quant_input returns), a bias in the epilogue, bf16 and fp32 output, ragged M, N not a multiple of 4 (scalar stores),
+    odd and even numbers of K blocks.  Exact on integer operands with power-of-two scales."""
+    g = torch.Generator().manual_seed(M + N + K)
+    ai = torch.randint(-4, 5, (M, K), generator=g)
+    bi = torch.randint(-4, 5, (N, K), generator=g)
+    KB, NB = K // 128, (N + 127) // 128
+    ae = torch.randint(-2, 3, (M, KB), generator=g)
+    be = torch.randint(-2, 3, (NB, KB), generator=g)
+    exact = torch.zeros(M, N, dtype=torch.float64)
+    for kb in range(KB):
+        exact += (ai[:, kb * 128:(kb + 1) * 128].double() @ bi[:, kb * 128:(kb + 1) * 128].double().t()) * \
+            torch.exp2((ae[:, kb][:, None] + be[torch.arange(N) // 128, kb][None, :]).double())
+    bias = torch.randint(-8, 9, (N,), generator=g).float().bfloat16()
+    a, b = ai.float().to(FP8).to(DEV), bi.float().to(FP8).to(DEV)
+    a_st, b_s, bias_d = torch.exp2(ae.float()).t().contiguous().to(DEV), torch.exp2(be.float()).to(DEV), bias.to(DEV)
+    lib = _lib.load()
+    assert lib.mdy_fp8_gemm_path(a.data_ptr(), b.data_ptr(), 1, M, M, N, K, 0) == 3
+    for dtype, code in ((torch.float32, 1), (torch.bfloat16, 0)):
+        out = torch.full((M, N), float("nan"), device=DEV, dtype=dtype)
+        assert lib.mdy_fp8_gemm_nt(a.data_ptr(), a_st.data_ptr(), 1, M, b.data_ptr(), b_s.data_ptr(), out.data_ptr(), bias_d.data_ptr(),
+                                   M, N, K, code, None) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(out.cpu().double(), (exact + bias.double()).to(dtype).double())
+
+
 SPLIT_SHAPES = [(128, 1536, 4096), (100, 777, 4224), (64, 2048, 4352), (40, 300, 8192), (256, 4096, 4096),
                 (130, 1100, 5120), (33, 130, 4096)]
 
