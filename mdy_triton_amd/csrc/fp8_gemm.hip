@@ -501,10 +501,14 @@ static bool big_tiles_pay(int64_t M, int64_t N) {
 }
 
 // Tile and ring depth for the shapes that do not take 256x256 tiles:
-//   0: 128x128, 2 K blocks in LDS (two workgroups share a CU)   1: 128x128, 4 K blocks (one workgroup per CU)
-//   2: 128x64, 6 K blocks                                       3: 64x64, 8 K blocks
+//   0: 128x128, 2 K blocks in LDS (two workgroups share a CU)   3: 64x64, 8 K blocks
 //   4: 128x256, 3 K blocks, 8 waves                             5: 256x128, 3 K blocks, 8 waves
-//   6: 128x192, 4 consumer waves (wave tile 64x96) + 4 producer waves, 2 K blocks in flight
+//   1: 128x128, 2: 128x64, 6: 128x192 - one workgroup per CU of 4 consumer + 4 producer waves (fp8_gemm_tile_ws), 2 or 3
+//      K blocks in flight.  Against the same tiles on the one-body kernel (4 waves, ring of 4 / 6; 8 waves, ring of 3),
+//      relaunched back to back / after a cache flush, row-major scales: 2048x2048x7168 46.6 -> 38.5 / 56.5 -> 53.0 us,
+//      2048x2048x256 8.0 -> 7.2 / 11.0 -> 10.4 us, 2048x1024x7168 34.3 -> 29.7 / 47.2 -> 44.2 us, 1000x1090x1664
+//      13.0 -> 10.2 / 18.0 -> 16.2 us, 4096x1536x7168 59.5 -> 49.7 / 63.6 -> 63.2 us (column-major scales 54.8 -> 47.3 /
+//      61.7 -> 57.8 us).
 // Measured rule: the smallest tile that still gives every workgroup a CU of its own (the time of these
 // shapes goes with the bytes each CU has to pull, not with its MFMAs), and the ring as deep as LDS allows.
 // Between 257 and 512 tiles of 128x128 that is a 128x256 tile (else, if those are too many, 256x128), one per CU,
@@ -627,18 +631,21 @@ static int dispatch_tiles(const uint8_t* a, const float* a_s, int64_t as_rs, int
 #define MDY_FEW(BM_, BN_, WGM_, WGN_, ST_)                                                                            \
     return launch_mfma<BM_, BN_, WGM_, WGN_, ST_, OUT, FMT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream)
     switch (few_tiles_config(M, N, K)) {
-        case 1: MDY_FEW(128, 128, 2, 2, 4);
-        case 2: MDY_FEW(128, 64, 2, 2, 6);
+#define MDY_WS(BM_, BN_, ST_)                                                                                          \
+    {                                                                                                                  \
+        const int tiles_m = (M + BM_ - 1) / BM_, tiles_n = (N + BN_ - 1) / BN_;                                        \
+        hipLaunchKernelGGL((fp8_gemm_ws_kernel<BM_, BN_, 2, 2, 4, ST_, OUT, FMT>), dim3((unsigned)(tiles_m * tiles_n)), dim3(512), 0, \
+                           stream, a, a_s, (int)as_rs, (int)as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, tiles_m, \
+                           tiles_n, pretouch_enabled() ? 1 : 0);                                                       \
+        return (int)hipGetLastError();                                                                                 \
+    }
+        case 1: MDY_WS(128, 128, 4)
+        case 2: MDY_WS(128, 64, 5)
+        case 6: MDY_WS(128, 192, 4)
+#undef MDY_WS
         case 3: MDY_FEW(64, 64, 2, 2, 8);
         case 4: MDY_FEW(128, 256, 2, 4, 3);
         case 5: MDY_FEW(256, 128, 2, 4, 3);
-        case 6: {
-            const int tiles_m = (M + 127) / 128, tiles_n = (N + 191) / 192;
-            hipLaunchKernelGGL((fp8_gemm_ws_kernel<128, 192, 2, 2, 4, 4, OUT, FMT>), dim3((unsigned)(tiles_m * tiles_n)), dim3(512), 0,
-                               stream, a, a_s, (int)as_rs, (int)as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, tiles_m,
-                               tiles_n, pretouch_enabled() ? 1 : 0);
-            return (int)hipGetLastError();
-        }
         default: MDY_FEW(128, 128, 2, 2, 2);
     }
 #undef MDY_FEW
