@@ -272,6 +272,136 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_kernel(const ui
 }
 
 // ---------------------------------------------------------------------------
+// Row-vector kernel: M <= 4 rows (single-token decode).  No matrix cores: a weight row against one activation row is a
+// dot product, and what bounds it is how many weight bytes every CU has in flight.  A wave owns R weight rows and
+// issues all of their loads up front (16 bytes per lane, 1 KB per load and row: K = 7168 -> 7 KB per row in flight), a
+// workgroup of 8 waves covers 8 R consecutive rows, so N = 2048 still gives 256 workgroups where the 16-column MFMA
+// kernel gives 128 (M = 1, N = 2048, K = 7168: 6.9 -> 4.9 us per call in a replayed graph).  The activation rows and
+// their scales are staged in LDS once per workgroup.  Per 16-byte piece a lane converts its bytes to fp32, takes the
+// dot product with the matching activation bytes and folds it with a_s[m,kb] * b_s[n/128,kb] (the piece lies in one K
+// block); the 64 partial sums of a row are added across the wave at the end.  The sum of a K block is thus formed
+// in eight scaled parts instead of one - the same value in exact arithmetic, another rounding (as with the K split).
+// ---------------------------------------------------------------------------
+constexpr int kGemvMaxK = 16384;     // MR rows x K bytes of activations in LDS
+constexpr int kGemvPieces = 8;       // 16-byte pieces per lane and batch over the wave's R rows (R x JB = 8: 8 KB in flight)
+
+template <int FMT>
+__device__ __forceinline__ void fp8x4_to_f32(uint32_t w, float (&f)[4]) {
+    floatx2 lo, hi;
+    if (FMT == 0) {
+        lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
+        hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);
+    } else {
+        lo = __builtin_amdgcn_cvt_pk_f32_bf8((int)w, false);
+        hi = __builtin_amdgcn_cvt_pk_f32_bf8((int)w, true);
+    }
+    f[0] = lo.x; f[1] = lo.y; f[2] = hi.x; f[3] = hi.y;
+}
+
+template <int MR, int R, typename OUT, int FMT>
+__global__ __launch_bounds__(512) void fp8_gemv_kernel(const uint8_t* __restrict__ a, const float* __restrict__ a_s, int64_t as_rs,
+                                                        int64_t as_cs, const uint8_t* __restrict__ b, const float* __restrict__ b_s,
+                                                        OUT* __restrict__ c, const uint16_t* __restrict__ bias, int N, int K) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds_x[MR * kGemvMaxK];
+    __shared__ float lds_sa[MR * (kGemvMaxK / 128)];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int KB = K >> 7, NB = (N + 127) >> 7;
+    // the activation rows (16 bytes per thread and step) and their scales
+    for (int m = 0; m < MR; ++m) {
+        for (int off = tid * 16; off < K; off += 512 * 16)
+            *reinterpret_cast<uint4*>(lds_x + m * K + off) = *reinterpret_cast<const uint4*>(a + (int64_t)m * K + off);
+        for (int kb = tid; kb < KB; kb += 512) lds_sa[m * KB + kb] = a_s[(int64_t)m * as_rs + (int64_t)kb * as_cs];
+    }
+    const int n0 = (blockIdx.x * 8 + wave) * R;
+    float acc[MR][R];
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[m][r] = 0.0f;
+    const int pieces = K >> 4;                       // 16-byte pieces of a row; piece p of this lane: p = j * 64 + lane
+    bool staged = false;
+    constexpr int JB = kGemvPieces / R;
+    for (int j0 = 0; j0 * 64 < pieces; j0 += JB) {
+        uint4 w[R][JB];
+        float sb[R][JB];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int n = min(n0 + r, N - 1);
+            const uint8_t* row = b + (int64_t)n * K;
+            const float* srow = b_s + (int64_t)min(n >> 7, NB - 1) * KB;
+#pragma unroll
+            for (int j = 0; j < JB; ++j) {
+                const int p = (j0 + j) * 64 + lane;
+                const bool ok = p < pieces;
+                w[r][j] = ok ? load_nt16(row + (int64_t)p * 16) : make_uint4(0u, 0u, 0u, 0u);
+                sb[r][j] = ok ? srow[p >> 3] : 0.0f;
+            }
+        }
+        if (!staged) {      // the weight loads are in flight: now wait for the activation rows
+            __syncthreads();
+            staged = true;
+        }
+#pragma unroll
+        for (int j = 0; j < JB; ++j) {
+            const int p = (j0 + j) * 64 + lane;
+            if (p < pieces) {
+                const int kb = p >> 3;
+                float wf[R][16];
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const uint32_t ww[4] = {w[r][j].x, w[r][j].y, w[r][j].z, w[r][j].w};
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        float f4[4];
+                        fp8x4_to_f32<FMT>(ww[q], f4);
+                        wf[r][4 * q] = f4[0]; wf[r][4 * q + 1] = f4[1]; wf[r][4 * q + 2] = f4[2]; wf[r][4 * q + 3] = f4[3];
+                    }
+                }
+#pragma unroll
+                for (int m = 0; m < MR; ++m) {
+                    const uint4 xv = *reinterpret_cast<const uint4*>(lds_x + m * K + p * 16);
+                    const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+                    float xf[16];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        float f4[4];
+                        fp8x4_to_f32<FMT>(xw[q], f4);
+                        xf[4 * q] = f4[0]; xf[4 * q + 1] = f4[1]; xf[4 * q + 2] = f4[2]; xf[4 * q + 3] = f4[3];
+                    }
+                    const float sa = lds_sa[m * KB + kb];
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        float d = 0.0f;
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) d = __builtin_fmaf(wf[r][e], xf[e], d);
+                        acc[m][r] = __builtin_fmaf(d, sa * sb[r][j], acc[m][r]);
+                    }
+                }
+            }
+        }
+    }
+    if (!staged) __syncthreads();
+    // add the 64 partial sums of every (m, r) across the wave; lane 0 stores
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            float v = acc[m][r];
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+            const int n = n0 + r;
+            if (lane == 0 && n < N) {
+                if (bias != nullptr) v += bf16_one(bias[n]);
+                if (sizeof(OUT) == 2)
+                    reinterpret_cast<uint16_t*>(c)[(int64_t)m * N + n] = (uint16_t)(pack2_bf16(v, 0.0f) & 0xFFFFu);
+                else
+                    reinterpret_cast<float*>(c)[(int64_t)m * N + n] = v;
+            }
+        }
+}
+
+// ---------------------------------------------------------------------------
 // Strip kernel: few rows (<= 16*MT <= 64 per group) against a weight that is wide enough to give every CU
 // work without splitting K (many column strips: a vocabulary-sized N, or many experts).  One workgroup = 8
 // waves = 128 weight columns of one group, wave w streams rows n0+16w .. +15 of the weight straight from
@@ -558,6 +688,10 @@ static int launch_strip(const uint8_t* a, const float* a_s, int64_t as_rs, int64
     return (int)hipGetLastError();
 }
 
+// up to 4 rows whose activations fit the row-vector kernel's LDS staging (K % 128 == 0, 16-byte aligned operands: the
+// caller checks)
+static bool gemv_pays(int64_t M, int64_t K) { return M <= 4 && K <= kGemvMaxK; }
+
 // few rows per group and enough 128-column strips to fill the CUs without splitting K (with a handful of rows the
 // 16-column kernel re-reads so little of a that it stays ahead)
 static bool strip_pays(int64_t max_rows, int64_t strips) { return max_rows > 4 && max_rows <= 64 && strips >= 200; }
@@ -567,6 +701,28 @@ static bool strip_pays(int64_t max_rows, int64_t strips) { return max_rows > 4 &
 template <typename OUT, int FMT>
 static int dispatch_small(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, int64_t as_extent, bool big_ok,
                           const uint8_t* b, const float* b_s, OUT* c, const uint16_t* bias, int M, int N, int K, hipStream_t stream) {
+    if (gemv_pays(M, K)) {
+        // rows per wave: 8 KB of weight bytes in flight per wave (4 rows of up to 2 KB, 2 of up to 4 KB, else 1), fewer
+        // when that would leave less than ~220 workgroups
+        int r = K <= 2048 ? 4 : K <= 4096 ? 2 : 1;
+        while (r > 1 && (int64_t)N / (8 * r) < 220) r >>= 1;
+        dim3 grid((unsigned)((N + 8 * r - 1) / (8 * r))), block(512);
+#define MDY_GEMV(MR, R)                                                                                               \
+    hipLaunchKernelGGL((fp8_gemv_kernel<MR, R, OUT, FMT>), grid, block, 0, stream, a, a_s, as_rs, as_cs, b, b_s, c, bias, N, K)
+#define MDY_GEMV_R(MR)                              \
+    do {                                            \
+        if (r == 1) MDY_GEMV(MR, 1);                \
+        else if (r == 2) MDY_GEMV(MR, 2);           \
+        else MDY_GEMV(MR, 4);                       \
+    } while (0)
+        if (M == 1) MDY_GEMV_R(1);
+        else if (M == 2) MDY_GEMV_R(2);
+        else if (M == 3) MDY_GEMV_R(3);
+        else MDY_GEMV_R(4);
+#undef MDY_GEMV_R
+#undef MDY_GEMV
+        return (int)hipGetLastError();
+    }
     if (M <= 64 && big_ok && strip_pays(M, (N + 127) / 128)) {
         const int64_t one = M;
         return launch_strip<OUT, FMT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, &one, 1, M, N, K, stream);

@@ -298,6 +298,68 @@ def test_gemm_small_m_exact(M):
     test_gemm_exact_integer_cases_all_kernels(M, 272, 384)
 
 
+@pytest.mark.parametrize("fmt", ["e4m3fn", "e5m2"])
+@pytest.mark.parametrize("M,N,K", [(1, 2048, 7168), (1, 7168, 2048), (2, 1000, 4096), (3, 259, 128), (4, 7001, 1024), (4, 520, 16384),
+                                   (1, 33, 1664), (2, 4096, 3072)])
+def test_gemm_row_vector_kernel_exact_integer(M, N, K, fmt):
+    """Up to 4 rows run on the row-vector kernel (no matrix cores; 1, 2 or 4 weight rows per wave by K and N): exact on
+    integer operands with power-of-two scales through the C entry points, row- and column-major activation scales, bias,
+    fp32 and bf16 output, N not a multiple of the rows per workgroup, both fp8 formats; K beyond its LDS staging
+    (16384) goes to the MFMA weight-streaming kernel and gives the same exact result."""
+    dt = FP8 if fmt == "e4m3fn" else torch.float8_e5m2
+    lib = _lib.load()
+    entry = lib.mdy_fp8_gemm_nt if fmt == "e4m3fn" else lib.mdy_fp8_gemm_nt_e5m2
+    g = torch.Generator().manual_seed(M + N + K)
+    ai = torch.randint(-4, 5, (M, K), generator=g)
+    bi = torch.randint(-4, 5, (N, K), generator=g)
+    KB, NB = K // 128, (N + 127) // 128
+    ae = torch.randint(-2, 3, (M, KB), generator=g)
+    be = torch.randint(-2, 3, (NB, KB), generator=g)
+    exact = torch.zeros(M, N, dtype=torch.float64)
+    for kb in range(KB):
+        exact += (ai[:, kb * 128:(kb + 1) * 128].double() @ bi[:, kb * 128:(kb + 1) * 128].double().t()) * \
+            torch.exp2((ae[:, kb][:, None] + be[torch.arange(N) // 128, kb][None, :]).double())
+    bias = torch.randint(-8, 9, (N,), generator=g).float().bfloat16()
+    a, b = ai.float().to(dt).to(DEV), bi.float().to(dt).to(DEV)
+    a_s, b_s, bias_d = torch.exp2(ae.float()).to(DEV), torch.exp2(be.float()).to(DEV), bias.to(DEV)
+    a_st = a_s.t().contiguous()
+    for dtype, code in ((torch.float32, 1), (torch.bfloat16, 0)):
+        for scales, rs, cs in ((a_s, KB, 1), (a_st, 1, M)):
+            for bp, want in ((None, exact), (bias_d, exact + bias.double())):
+                out = torch.full((M, N), float("nan"), device=DEV, dtype=dtype)
+                assert entry(a.data_ptr(), scales.data_ptr(), rs, cs, b.data_ptr(), b_s.data_ptr(), out.data_ptr(),
+                             bp.data_ptr() if bp is not None else None, M, N, K, code, None) == 0
+                torch.cuda.synchronize()
+                assert torch.equal(out.cpu().double(), want.to(dtype).double())
+    if fmt == "e4m3fn":       # a longer K than the kernel stages: the MFMA kernel, same exact result
+        K2 = 16384 + 128
+        a2 = torch.zeros(M, K2, dtype=torch.uint8, device=DEV).view(dt)
+        b2 = torch.zeros(N, K2, dtype=torch.uint8, device=DEV).view(dt)
+        a2[:, :K] = a
+        b2[:, :K] = b
+        a2_s = torch.ones(M, K2 // 128, device=DEV)
+        b2_s = torch.ones(NB, K2 // 128, device=DEV)
+        a2_s[:, :KB] = a_s
+        b2_s[:, :KB] = b_s
+        out = torch.full((M, N), float("nan"), device=DEV)
+        assert entry(a2.data_ptr(), a2_s.data_ptr(), K2 // 128, 1, b2.data_ptr(), b2_s.data_ptr(), out.data_ptr(), None, M, N, K2, 1,
+                     None) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(out.cpu().double(), exact)
+
+
+def test_gemm_row_vector_kernel_against_oracle():
+    """The row-vector kernel on quantized Gaussian data: within rtol = atol = 1e-2 of the oracle (it adds a K block in
+    eight scaled parts, another rounding than the MFMA kernels), and within 2^-8 of the float64 truth's scale."""
+    for M, N, K in [(1, 2048, 7168), (1, 7168, 2048), (4, 1536, 4096)]:
+        a, a_s, wq, ws = quantized_problem("normal", M, N, K, seed=M + K)
+        ref = O.fp8_gemm(a, a_s, wq, ws, dtype=torch.float32)
+        got = m.fp8_gemm(a.to(DEV), a_s.to(DEV), wq.to(DEV), ws.to(DEV), out_dtype=torch.float32)
+        assert close(got, ref)
+        truth = O.fp8_gemm_f64(a, a_s, wq, ws)
+        assert (got.cpu().double() - truth).abs().max() <= 2 ** -12 * truth.abs().max() + 1e-6
+
+
 def test_gemm_one_hot_and_scale_block_perturbation():
     N, K = 512, 512
     g = torch.Generator().manual_seed(2)
