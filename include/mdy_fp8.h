@@ -96,10 +96,11 @@ int mdy_act_quant_typed(const void* x, int x_dtype, int block_size, void* y, flo
  * mode = MDY_QUANT_OFFICIAL.
  *
  *   w   bf16 [N, K], element (n, k) at w[n * w_row_stride + k * w_col_stride]
- *   y   e4m3fn [PN, PK] row-major, PN % 128 == 0, PK % 128 == 0, padding reads as 0
- *   s   fp32 [PN/128, PK/128] row-major
+ *   y   e4m3fn [PN, PK] row-major, PN % 128 == 0, PK % 128 == 0, padding reads as 0; or NULL when only the
+ *       transposed copy is wanted (per_block_cast_to_fp8(output_normal=False), megatron_patchs/fp8_matmul.py:334-392)
+ *   s   fp32 [PN/128, PK/128] row-major or NULL (must be given iff y is)
  *   y_t e4m3fn [PK, PN] row-major (transposed copy) or NULL
- *   s_t fp32 [PK/128, PN/128] row-major or NULL (must be given iff y_t is)
+ *   s_t fp32 [PK/128, PN/128] row-major or NULL (must be given iff y_t is); at least one of y / y_t
  */
 int mdy_weight_quant(const void* w, void* y, float* s, void* y_t, float* s_t, int64_t N, int64_t K,
                      int64_t w_row_stride, int64_t w_col_stride, int64_t PN, int64_t PK, int mode,

@@ -105,9 +105,10 @@ int mdy_weight_quant_typed(const void* w, int w_dtype, void* y, float* s, void* 
         return fail(MDY_E_SHAPE, "weight_quant: need 0 <= N <= PN, 0 <= K <= PK");
     if (PN % 128 != 0 || PK % 128 != 0) return fail(MDY_E_SHAPE, "weight_quant: PN=%lld, PK=%lld must be multiples of 128", (long long)PN, (long long)PK);
     if ((y_t == nullptr) != (s_t == nullptr)) return fail(MDY_E_NULL, "weight_quant: y_t and s_t must be given together");
+    if ((y == nullptr) != (s == nullptr)) return fail(MDY_E_NULL, "weight_quant: y and s must be given together");
     if (PN == 0 || PK == 0) return 0;
-    if (!y || !s || (!w && N > 0 && K > 0)) return fail(MDY_E_NULL, "weight_quant: null pointer");
-    if (!aligned(y, 8) || (y_t && !aligned(y_t, 8))) return fail(MDY_E_ALIGN, "weight_quant: y / y_t must be 8-byte aligned");
+    if ((!y && !y_t) || (!w && N > 0 && K > 0)) return fail(MDY_E_NULL, "weight_quant: null pointer");
+    if ((y && !aligned(y, 8)) || (y_t && !aligned(y_t, 8))) return fail(MDY_E_ALIGN, "weight_quant: y / y_t must be 8-byte aligned");
     if (int e = check_device()) return e;
     return launched(mdy::launch_weight_quant(w, w_dtype, y, s, y_t, s_t, N, K, w_row_stride, w_col_stride, PN, PK, mode,
                                              static_cast<hipStream_t>(stream)),

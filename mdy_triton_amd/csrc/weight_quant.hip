@@ -61,7 +61,7 @@ __global__ __launch_bounds__(512) void weight_quant_kernel(const void* __restric
     const bool fast = XT == 0 && group_is_fast<MODE>(amax);
     const float r = 1.0f / sc;
     if (t == 0) {
-        s[(int64_t)bn * (PK >> 7) + bk] = sc;
+        if (s) s[(int64_t)bn * (PK >> 7) + bk] = sc;
         if (s_t) s_t[(int64_t)bk * (PN >> 7) + bn] = sc;
     }
     uint32_t qlo[RPT], qhi[RPT];   // row i of the quantized bytes: columns 0..3 | 4..7
@@ -69,7 +69,7 @@ __global__ __launch_bounds__(512) void weight_quant_kernel(const void* __restric
     for (int i = 0; i < RPT; ++i) {
         const uint2 o = quantize8_scaled<MODE>(f[i], sc, r, fast);
         const int row = rbase + i;  // < PN because PN % 128 == 0
-        store_nt8(y + (int64_t)row * PK + c0, o);
+        if (y) store_nt8(y + (int64_t)row * PK + c0, o);      // NULL: only the transposed copy is wanted
         qlo[i] = o.x;
         qhi[i] = o.y;
     }

@@ -96,15 +96,18 @@ def per_block_cast_to_fp8(x, output_normal: bool = True, output_transpose: bool 
     BA, BB = (256 if output_transpose else 128), (256 if output_normal else 128)
     PM, PN = _cdiv(M, BA) * BA, _cdiv(N, BB) * BB
     A, B = PM // 128, PN // 128
-    # the kernel always writes the normal copy; without output_normal it goes to a scratch tensor
-    y = torch.empty(G, PM, PN, device=dev, dtype=FP8)
-    s = torch.empty(G, A, B, device=dev, dtype=torch.float32)
+    if not (output_normal or output_transpose):
+        return ()
+    # a copy that is not asked for is neither allocated nor written (the kernel takes NULL for it)
+    y = torch.empty(G, PM, PN, device=dev, dtype=FP8) if output_normal else None
+    s = torch.empty(G, A, B, device=dev, dtype=torch.float32) if output_normal else None
     y_t = torch.empty(G, PN, PM, device=dev, dtype=FP8) if output_transpose else None
     s_t = torch.empty(G, B, A, device=dev, dtype=torch.float32) if output_transpose else None
     if PM * PN > 0:
         with on_device(dev):
             for g, w in enumerate(xs):
-                check(lib().mdy_weight_quant_typed(ptr(w), xt, ptr(y[g]), ptr(s[g]), ptr(y_t[g]) if output_transpose else None,
+                check(lib().mdy_weight_quant_typed(ptr(w), xt, ptr(y[g]) if output_normal else None, ptr(s[g]) if output_normal else None,
+                                             ptr(y_t[g]) if output_transpose else None,
                                              ptr(s_t[g]) if output_transpose else None, M, N, w.stride(0), w.stride(1), PM, PN, 1,
                                              stream_ptr(dev)), "per_block_cast_to_fp8")
     post = (lambda t: t.squeeze(0)) if G == 1 else (lambda t: t)
