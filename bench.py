@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the block-wise FP8 linear path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3] [--table] [--ablation]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3] [--table] [--ablation] [--ceilings] [--energy]
 
 One "step" is one pass of the hot path over one batch of synthetic input that is
 already resident in HBM: act_quant(X) followed by fp8_gemm(Xq, Xs, Wq, Ws) -> bf16,
@@ -24,7 +24,8 @@ Prints ONE JSON line on stdout:
                each timed alone, cold cache (a 512 MiB buffer is rewritten before every launch),
                and per launch of several back-to-back launches on uncached buffers (us_streamed);
                the same three kernels at the other large configurations (C2, C4; cold, one
-               event pair per launch); the six decode shapes (C5) as the per-call time of a
+               event pair per launch; the GEMM also as the headline GEMM is timed: bracketed by
+               events inside a loop of act_quant + fp8_gemm, `us_in_loop`); the six decode shapes (C5) as the per-call time of a
                replayed HIP graph of 20 calls (the Python call is not in the number)
   power        socket power and shader clock while the GEMM runs back to back for about a
                second (amd-smi readings), next to the board's power cap
@@ -34,7 +35,8 @@ Before the W warm-up steps the script runs the same step for 50 ms (set-up, unti
 GPU needs some 20 ms of work to reach its sustained clock, whatever W is.
 With --table a per-kernel table for every benchmark configuration and for the shapes the reference
 publishes numbers for goes to stderr; with --ablation the tile kernel is timed with parts of its K loop
-switched off (mdy_fp8_gemm_probe of libmdyfp8_probe.so), power and clock beside each line (stdout, no JSON).
+switched off (mdy_fp8_gemm_probe of libmdyfp8_probe.so), power and clock beside each line (stdout, no JSON); with
+--ceilings the copy-only twins of the quantizers, a register-resident MFMA loop and the launch floor (same library).
 """
 import argparse
 import json
@@ -72,6 +74,12 @@ def parse_args():
     ap.add_argument("--table", action="store_true", help="also print a per-kernel table for all configurations to stderr")
     ap.add_argument("--ablation", action="store_true",
                     help="time the tile kernel with parts of its K loop switched off, with power and clock (no JSON)")
+    ap.add_argument("--energy", action="store_true",
+                    help="energy per call of the headline GEMM's main launch for other XCD tile-block shapes (no JSON)")
+    ap.add_argument("--energy-launches", type=int, default=0,
+                    help="with --energy: launch every variant only this many times (for a rocprofv3 --pmc run)")
+    ap.add_argument("--ceilings", action="store_true",
+                    help="copy-only twins of the quantizers, the MFMA-only register loop and the launch floor (no JSON)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload (skip C2, C4, C5 and the power loop)")
     ap.add_argument("--only-decode", action="store_true",
@@ -352,6 +360,19 @@ def kernel_entries(torch, m, timer, x, wq, ws, reps=12):
     aq_us, _ = timer.run(lambda: m.act_quant(x), reps)
     wd_us, _ = timer.run(lambda: m.weight_dequant(wq, ws, out_dtype=torch.bfloat16), reps)
     g_us, _ = timer.run(lambda: m.fp8_gemm(xq, xs, wq, ws, out_dtype=torch.bfloat16), reps)
+    # the same GEMM in the loop the headline value is measured in: act_quant + fp8_gemm back to back, the GEMM bracketed by
+    # events (its operands come from the caches the way they do between the layers of a model)
+    for _ in range(5):
+        a_, s_ = m.act_quant(x)
+        m.fp8_gemm(a_, s_, wq, ws, out_dtype=torch.bfloat16)
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(20)]
+    for e0, e1 in ev:
+        a_, s_ = m.act_quant(x)
+        e0.record()
+        m.fp8_gemm(a_, s_, wq, ws, out_dtype=torch.bfloat16)
+        e1.record()
+    torch.cuda.synchronize()
+    loop_us = sorted(e0.elapsed_time(e1) * 1e3 for e0, e1 in ev)[len(ev) // 2]
     aq_b = 3.03125 * M * K
     wd_b = 3.0 * N * K + 4.0 * ((N + 127) // 128) * (K // 128)
     fl = 2.0 * M * N * K
@@ -361,7 +382,8 @@ def kernel_entries(torch, m, timer, x, wq, ws, reps=12):
         "weight_dequant": {"us": round(wd_us, 2), "GB/s": round(wd_b / wd_us / 1e3, 1),
                            "frac_hbm_peak": round(wd_b / wd_us / 1e3 / PEAK_HBM_GBS, 4)},
         "fp8_gemm": {"us": round(g_us, 2), "TFLOP/s": round(fl / g_us / 1e6, 1),
-                     "frac_mfma_peak": round(fl / g_us / 1e6 / PEAK_FP8_TFLOPS, 4)},
+                     "frac_mfma_peak": round(fl / g_us / 1e6 / PEAK_FP8_TFLOPS, 4),
+                     "us_in_loop": round(loop_us, 2), "frac_mfma_peak_in_loop": round(fl / loop_us / 1e6 / PEAK_FP8_TFLOPS, 4)},
     }
 
 
@@ -404,6 +426,12 @@ def main():
     torch.cuda.set_device(dev)
     if args.ablation:
         ablation(torch, m, dev)
+        return
+    if args.ceilings:
+        ceilings(torch, m, ColdTimer(torch, dev), dev)
+        return
+    if args.energy:
+        energy(torch, m, dev, args.energy_launches)
         return
     if args.only_decode:
         print(json.dumps({"C5_graph_replay": decode_entries(torch, m, dev, eager_calls=200)}))
@@ -562,8 +590,133 @@ def load_probe_lib():
     L = ctypes.CDLL(path)
     i64, p, i = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int
     L.mdy_fp8_gemm_probe.argtypes = [i, i, p, p, i64, i64, p, p, p, i64, i64, i64, p]
-    L.mdy_fp8_gemm_probe.restype = i
+    L.mdy_fp8_gemm_order_probe.argtypes = [i, i, p, p, i64, i64, p, p, p, i64, i64, i64, p]
+    L.mdy_fp8_gemm_order_probe.restype = i
+    L.mdy_probe_copy_aq.argtypes = [p, p, p, i64, i64, p]
+    L.mdy_probe_copy_wd.argtypes = [p, p, p, i64, i64, p]
+    L.mdy_probe_mfma_loop.argtypes = [i, p, p, i, i, p]
+    L.mdy_probe_empty.argtypes = [p]
+    for f in (L.mdy_fp8_gemm_probe, L.mdy_probe_copy_aq, L.mdy_probe_copy_wd, L.mdy_probe_mfma_loop, L.mdy_probe_empty):
+        f.restype = i
     return L
+
+
+def energy(torch, m, dev, launches=0):
+    """Energy per call of the headline GEMM's main launch (1024 tiles of 256x256: C3's first 16384 columns) for the shapes
+    of the block of tiles that an XCD runs at a time (2x16, 4x8 = product, 8x4) with the pre-touches on and off: each
+    variant relaunched for ~1.5 s, time per launch x socket power.  With launches > 0 every variant is only launched that
+    many times (the run that rocprofv3 --pmc FETCH_SIZE counts)."""
+    L = load_probe_lib()
+    seed, kind, M, N, K, _ = WORKLOADS["C3"]
+    N = 16384
+    x, w = make_inputs(torch, kind, M, N, K, seed, dev)
+    wq, ws = quantize_weight(torch, w, dev)
+    xq, xs = m.act_quant(x)
+    xst = xs.t().contiguous()
+    c = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    ref = None
+    idle = SmiSampler.read()
+    print("M=%d N=%d K=%d, 1024 tiles of 256x256; power cap %s W; idle reading %s" % (M, N, K, power_cap_w(), idle))
+    print("%-34s %9s %8s %7s %9s %s" % ("tiles per XCD at a time / touches", "us", "W", "MHz", "mJ/call", "same bits"))
+    for gm in (4, 2, 8):
+        for touch in (1, 0):
+            def fn(gm=gm, touch=touch):
+                rc = L.mdy_fp8_gemm_order_probe(gm, touch, xq.data_ptr(), xst.data_ptr(), 1, M, wq.data_ptr(), ws.data_ptr(), c.data_ptr(),
+                                                M, N, K, None)
+                if rc != 0:
+                    raise RuntimeError("mdy_fp8_gemm_order_probe(%d, %d) returned %d" % (gm, touch, rc))
+            fn()
+            torch.cuda.synchronize()
+            if ref is None:
+                ref = c.clone()
+            same = bool(torch.equal(c, ref))
+            if launches > 0:
+                for _ in range(launches):
+                    fn()
+                torch.cuda.synchronize()
+                print("%-34s launched %d times, same bits %s" % ("%dx%d, pre-touches %s" % (gm, 32 // gm, "on" if touch else "off"), launches, same))
+                continue
+            us, smi = sustained(torch, fn, seconds=1.5)
+            smi = smi or {}
+            pw = smi.get("socket_power_w")
+            print("%-34s %9.1f %8s %7s %9s %s" % ("%dx%d, pre-touches %s" % (gm, 32 // gm, "on" if touch else "off"), us, pw,
+                                                 smi.get("gfx_clock_mhz"), "%.1f" % (us * pw * 1e-3) if pw else "-", same), flush=True)
+
+
+def ceilings(torch, m, timer, dev):
+    """What the memory system and the matrix cores give this library's access patterns with the arithmetic taken out
+    (libmdyfp8_probe.so), next to the product kernels under the same timing protocols (stdout, no JSON):
+    copy-only twins of act_quant and weight_dequant; a register-resident MFMA loop with and without the fp32 fold of the
+    block-scaled GEMM, on hashed and on constant operand bytes, with socket power and shader clock; an empty kernel
+    and the M = 1 GEMM in a replayed graph."""
+    L = load_probe_lib()
+    from mdy_triton_amd._torch_glue import stream_ptr
+
+    def ok(rc, what):
+        if rc != 0:
+            raise RuntimeError("%s returned %d" % (what, rc))
+
+    print("== HBM streams: copy-only twin against the product kernel (us; cold = one launch after a 512 MiB flush incl. ~3 us "
+          "of event overhead; streamed = per launch of back-to-back launches on uncached buffers)")
+    for M, K in ((4096, 7168), (4096, 18432), (16384, 4096)):
+        n = max(2, int(6e8 // (2 * M * K)) + 1)
+        xs = [torch.randn(M, K, device=dev).bfloat16() for _ in range(n)]
+        ys = [torch.empty(M, K, dtype=torch.uint8, device=dev) for _ in range(n)]
+        ss = [torch.empty(M, K // 128, device=dev) for _ in range(n)]
+        twin = [(lambda i=i: ok(L.mdy_probe_copy_aq(xs[i].data_ptr(), ys[i].data_ptr(), ss[i].data_ptr(), M, K, stream_ptr(dev)), "copy_aq"))
+                for i in range(n)]
+        prod = [(lambda i=i: m.act_quant(xs[i])) for i in range(n)]
+        b = 3.03125 * M * K
+        tc, _ = timer.run(twin[0], 20)
+        pc, _ = timer.run(prod[0], 20)
+        ts, ps = streamed_us(torch, timer, twin, 10), streamed_us(torch, timer, prod, 10)
+        print("act_quant %5dx%-5d  copy-only cold %6.2f streamed %6.2f (%4.1f %% of 8 TB/s) | product cold %6.2f streamed %6.2f (%4.1f %%) "
+              "| product / copy-only %5.3f" % (M, K, tc, ts, b / ts / 1e3 / 80, pc, ps, b / ps / 1e3 / 80, ts / ps), flush=True)
+        del xs, ys, ss
+    for N, K in ((18432, 7168), (7168, 18432)):
+        n = max(2, int(4e8 // (N * K)) + 1)
+        ws = torch.rand((N + 127) // 128, K // 128, device=dev) + 0.5
+        xq = [torch.randint(0, 120, (N, K), dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn) for _ in range(n)]
+        ys = [torch.empty(N, K, dtype=torch.bfloat16, device=dev) for _ in range(n)]
+        twin = [(lambda i=i: ok(L.mdy_probe_copy_wd(xq[i].data_ptr(), ws.data_ptr(), ys[i].data_ptr(), N, K, stream_ptr(dev)), "copy_wd"))
+                for i in range(n)]
+        prod = [(lambda i=i: m.weight_dequant(xq[i], ws, out_dtype=torch.bfloat16)) for i in range(n)]
+        b = 3.0 * N * K + 4.0 * ws.numel()
+        tc, _ = timer.run(twin[0], 20)
+        pc, _ = timer.run(prod[0], 20)
+        ts, ps = streamed_us(torch, timer, twin, 10), streamed_us(torch, timer, prod, 10)
+        print("weight_dequant %5dx%-5d  copy-only cold %6.2f streamed %6.2f (%4.1f %% of 8 TB/s) | product cold %6.2f streamed %6.2f "
+              "(%4.1f %%) | product / copy-only %5.3f" % (N, K, tc, ts, b / ts / 1e3 / 80, pc, ps, b / ps / 1e3 / 80, ts / ps), flush=True)
+        del xq, ys
+
+    print("== matrix cores alone: 8 waves per CU, 32 v_mfma_f32_16x16x128_f8f6f4 per iteration from registers, relaunched for "
+          "~1.5 s; power cap %s W" % power_cap_w())
+    out = torch.empty(256 * 512, device=dev)
+    g = torch.Generator().manual_seed(7)
+    seeds = {"hashed operand bytes": torch.randint(1, 2 ** 31 - 1, (64,), generator=g, dtype=torch.int64).to(torch.int32).to(dev),
+             "constant operand bytes (0x38)": torch.zeros(64, dtype=torch.int32, device=dev)}
+    iters = 1000
+    flop = 256.0 * 8 * iters * 32 * 65536
+    for fold, label in ((0, "MFMA only, accumulating in place"), (1, "each MFMA from zero + 4 v_fma_f32 (the block-scale fold)")):
+        for sname, seed in seeds.items():
+            def fn(fold=fold, seed=seed):
+                ok(L.mdy_probe_mfma_loop(fold, seed.data_ptr(), out.data_ptr(), 256, iters, stream_ptr(dev)), "mfma_loop")
+            us, smi = sustained(torch, fn, seconds=1.5)
+            smi = smi or {}
+            print("  %-58s %-30s %8.1f us  %6.2f PFLOP/s (%4.1f %% of 5.0)  %6s W  %5s MHz" % (
+                label, sname, us, flop / us / 1e9, flop / us / 1e9 / 5.0 * 100, smi.get("socket_power_w"), smi.get("gfx_clock_mhz")), flush=True)
+
+    print("== launch floor: per call inside a replayed HIP graph of 20 calls")
+    e_us = graph_replay_us(torch, lambda: ok(L.mdy_probe_empty(stream_ptr(dev)), "empty"))
+    print("  empty kernel                         %5.2f us" % e_us)
+    for (M, N, K) in ((1, 7168, 2048), (1, 2048, 7168)):
+        x = torch.randn(M, K, device=dev).bfloat16()
+        w = torch.randn(N, K, device=dev).mul_(0.02).bfloat16()
+        wq, wsc = quantize_weight(torch, w, dev)
+        xq, xsc = m.act_quant(x)
+        us = graph_replay_us(torch, lambda: m.fp8_gemm(xq, xsc, wq, wsc, out_dtype=torch.bfloat16))
+        print("  fp8_gemm M=%d N=%d K=%d              %5.2f us  (%.1f MB of weights: %.2f TB/s over the empty kernel's time)" % (
+            M, N, K, us, N * K / 1e6, N * K / (us - e_us) / 1e6))
 
 
 def ablation(torch, m, dev):

@@ -13,7 +13,7 @@ SOURCES = ["api.hip", "act_quant.hip", "weight_quant.hip", "quant_transpose.hip"
 LIB = os.path.join(HERE, "libmdyfp8.so")
 # timing probes (ablated copies of the tile kernel, copy-only and MFMA-only ceilings): a library of its own that only
 # bench.py's diagnostic modes load
-PROBE_SOURCES = ["gemm_probe.hip"]
+PROBE_SOURCES = ["gemm_probe.hip", "ceiling_probe.hip"]
 PROBE_LIB = os.path.join(HERE, "libmdyfp8_probe.so")
 
 # -packed-fp32-ops: keep the compiler from forming v_pk_{add,mul,fma}_f32.

@@ -449,18 +449,21 @@ __device__ __forceinline__ void fp8_gemm_tile(
 __device__ __forceinline__ int xcd_contiguous(int pid, int ntiles) {
     return (ntiles % 8 == 0) ? (pid & 7) * (ntiles >> 3) + (pid >> 3) : pid;
 }
+// GM: tile rows per group; the 32 workgroups that an XCD runs at a time then cover a GM x (32 / GM) block of tiles
+// (4 x 8 in the product; the probe library also builds 2 x 16 and 8 x 4 to measure their fabric traffic and energy).
+template <int GM = 4>
 __device__ __forceinline__ Duty tile_of(int local, int tiles_m, int tiles_n, int& tm, int& tn) {
-    constexpr int GM = 4;
     const int group = local / (GM * tiles_n);
     const int first_m = group * GM;
     const int gsz = min(tiles_m - first_m, GM);
     const int in_group = (local % (GM * tiles_n)) % gsz;
     tm = first_m + in_group;
     tn = (local % (GM * tiles_n)) / gsz;
-    // the workgroups of an XCD run a gsz x (up to 8) block of tiles at a time
+    // the workgroups of an XCD run a gsz x (up to 32 / GM) block of tiles at a time
     Duty d;
-    d.b_sh = gsz >= 4 ? 2 : gsz >= 2 ? 1 : 0;
-    d.a_sh = tiles_n >= 8 ? 3 : tiles_n >= 4 ? 2 : tiles_n >= 2 ? 1 : 0;
+    d.b_sh = gsz >= 8 ? 3 : gsz >= 4 ? 2 : gsz >= 2 ? 1 : 0;
+    constexpr int COLS = 32 / GM;
+    d.a_sh = (tiles_n >= 16 && COLS >= 16) ? 4 : (tiles_n >= 8 && COLS >= 8) ? 3 : (tiles_n >= 4 && COLS >= 4) ? 2 : tiles_n >= 2 ? 1 : 0;
     d.b_duty = in_group & ((1 << d.b_sh) - 1);
     d.a_duty = tn & ((1 << d.a_sh) - 1);
     return d;
@@ -731,7 +734,7 @@ __global__ __launch_bounds__((WGM * WGN + PW) * 64) void fp8_gemm_ws_kernel(
     }
 }
 
-template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT, int GAP_ = 0, int TD_ = 0, int ABL_ = 0, int FMT_ = 0>
+template <int BM, int BN, int WGM, int WGN, int STAGES, typename OUT, int GAP_ = 0, int TD_ = 0, int ABL_ = 0, int FMT_ = 0, int GM_ = 4>
 __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
@@ -744,7 +747,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void fp8_gemm_mfma_kernel(
     const int ntiles = tiles_m * tiles_n;
     for (int pid = blockIdx.x; pid < ntiles; pid += gridDim.x) {
         int tm, tn;
-        Duty duty = tile_of(xcd_contiguous(pid, ntiles), tiles_m, tiles_n, tm, tn);
+        Duty duty = tile_of<GM_>(xcd_contiguous(pid, ntiles), tiles_m, tiles_n, tm, tn);
         if (!pretouch) duty.a_sh = duty.b_sh = 0;
         fp8_gemm_tile<BM, BN, WGM, WGN, STAGES, OUT, GAP_, TD_, ABL_, FMT_>(a, a_s, as_rs, as_cs, as_bytes, b, b_s, c, bias, tm * BM, M,
                                                                             M, tn * BN, N, K, ldc, duty, 0, K >> 7, pool);

@@ -55,10 +55,48 @@ static int launch_fp8_gemm_probe(int tile, int ablation, const void* a, const fl
     return -1;
 }
 
+// The product's 256x256 kernel with another shape of the block of tiles that an XCD runs at a time (GM tile rows x
+// 32 / GM tile columns; the product uses 4 x 8) and the pre-touches on or off: the exact GEMM result every time.
+static int launch_fp8_gemm_order_probe(int gm, int pretouch, const void* a, const float* a_s, int64_t as_rs, int64_t as_cs,
+                                       const void* b, const float* b_s, void* c, int64_t M, int64_t N, int64_t K, hipStream_t stream) {
+    const int KB = (int)(K / 128);
+    const int64_t as_extent = ((M - 1) * as_rs + (int64_t)(KB - 1) * as_cs + 1) * 4;
+    int cus = 256, dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus = n;
+    }
+    const int tiles_m = (int)((M + 255) / 256), tiles_n = (int)((N + 255) / 256);
+    const int wgs = tiles_m * tiles_n > cus ? cus : tiles_m * tiles_n;
+#define MDY_ORDER(GM)                                                                                                   \
+    hipLaunchKernelGGL((fp8_gemm_mfma_kernel<256, 256, 2, 4, 2, uint16_t, 0, 0, 0, 0, GM>), dim3((unsigned)wgs), dim3(512), 0, stream, \
+                       static_cast<const uint8_t*>(a), a_s, (int)as_rs, (int)as_cs, (uint32_t)as_extent,                  \
+                       static_cast<const uint8_t*>(b), b_s, static_cast<uint16_t*>(c), static_cast<const uint16_t*>(nullptr), \
+                       (int)M, (int)N, (int)K, (int)N, tiles_m, tiles_n, pretouch)
+    if (gm == 2) MDY_ORDER(2);
+    else if (gm == 4) MDY_ORDER(4);
+    else if (gm == 8) MDY_ORDER(8);
+    else return -1;
+#undef MDY_ORDER
+    return (int)hipGetLastError();
+}
+
 }  // namespace mdy
 
 // Entry point of the probe library.  K % 128 == 0, K <= 65536, N % 4 == 0, a / b / c 16-byte aligned, activation scales
 // within 2^31 bytes; returns 0, a hipError_t, -1 for a tile / ablation pair that is not built, -2 for bad arguments.
+extern "C" int mdy_fp8_gemm_order_probe(int gm, int pretouch, const void* a, const float* a_s, int64_t as_row_stride,
+                                        int64_t as_col_stride, const void* b, const float* b_s, void* c, int64_t M, int64_t N,
+                                        int64_t K, void* stream) {
+    if (M < 1 || N < 1 || K < 128 || K % 128 != 0 || K > 65536 || N % 4 != 0 || !a || !a_s || !b || !b_s || !c) return -2;
+    if (((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c)) & 15) != 0) return -2;
+    if (as_row_stride < 0 || as_col_stride < 0 ||
+        ((M - 1) * as_row_stride + (K / 128 - 1) * as_col_stride + 1) * 4 >= ((int64_t)1 << 31))
+        return -2;
+    return mdy::launch_fp8_gemm_order_probe(gm, pretouch, a, a_s, as_row_stride, as_col_stride, b, b_s, c, M, N, K,
+                                            static_cast<hipStream_t>(stream));
+}
+
 extern "C" int mdy_fp8_gemm_probe(int tile, int ablation, const void* a, const float* a_s, int64_t as_row_stride,
                                   int64_t as_col_stride, const void* b, const float* b_s, void* c, int64_t M, int64_t N,
                                   int64_t K, void* stream) {
