@@ -117,6 +117,24 @@ def test_gemm_exact_integer_producer_consumer_tiles(M, N, K):
         assert torch.equal(out.cpu().double(), (exact + bias.double()).to(dtype).double())
 
 
+def _random_mid_shapes():
+    g = torch.Generator().manual_seed(20250101)
+    out = []
+    for _ in range(28):
+        M = int(torch.randint(65, 4200, (1,), generator=g))
+        N = int(torch.randint(8, 3200, (1,), generator=g))
+        K = 128 * int(torch.randint(1, 17, (1,), generator=g))
+        out.append((M, N, K))
+    return out
+
+
+@pytest.mark.parametrize("M,N,K", _random_mid_shapes())
+def test_gemm_exact_integer_random_mid_shapes(M, N, K):
+    """Randomly drawn (seeded) shapes in the range where the dispatch picks among the few-tile configurations (one-body and
+    producer / consumer kernels, every ring depth, ragged M and N, 1 to 16 K blocks): exact on integer operands."""
+    test_gemm_exact_integer_cases_all_kernels(M, N, K)
+
+
 SPLIT_SHAPES = [(128, 1536, 4096), (100, 777, 4224), (64, 2048, 4352), (40, 300, 8192), (256, 4096, 4096),
                 (130, 1100, 5120), (33, 130, 4096)]
 
