@@ -81,6 +81,19 @@ __device__ __forceinline__ void dma4(const intx4& rsrc, int voff, int soff, uint
 
 // Shares of the panel pre-touches: the A panel of a tile row is cut into 2^a_sh shares among the tiles of
 // that row that run side by side, the B panel of a tile column into 2^b_sh shares among its tile rows.
+// In the producer/consumer kernel a touch covers kTouchBurst CONSECUTIVE lines (K blocks) of a row at a time: a K
+// block's copy needs one 128-byte line from each of a panel's rows, rows that lie K bytes apart - for memory that is
+// one isolated line per DRAM page and K block.  Touching 4 lines (512 contiguous bytes) of a row every 4th K block
+// instead of one line every K block asks memory for the same bytes in a quarter of the places.  Measured one launch
+// after a cache flush (operands cold, caches full of dirty lines), same process, row-major scales: 4096x1536x7168
+// 63.5 -> 57.2 us, 2048x2048x7168 52.7 -> 44.2 us, 2048x1024x7168 44.6 -> 34.4 us, 1024x4096x7168 54.0 -> 44.8 us;
+// bursts of 2 / 8 / 16 lines are 1.5 / 1.4 / 4.3 us slower than 4 at the first shape; touching single lines further
+// ahead (5 or 8 K blocks instead of 2) changes nothing; relaunched back to back (operands in the caches) all tie.
+// The one-body kernel (hundreds of tiles, many workgroups on every panel) keeps single-line touches: bursts made
+// 4096x18432x7168 472 -> 491 us and 4096x7168x18432 455 -> 468 us back to back.
+constexpr int kTouchBurstLog = 2, kTouchBurst = 1 << kTouchBurstLog;
+// a byte offset beyond every descriptor of these kernels (their ranges stay below 2^31): such a lane accesses nothing
+constexpr int kOutOfRange = 0x7ffffff0;
 struct Duty {
     int a_duty, a_sh, b_duty, b_sh;
 };
@@ -555,8 +568,9 @@ __device__ __forceinline__ void fp8_gemm_tile_ws(
         const int t_idx = (pw >> 1) * 64 + lane;
         const int share = touch_b ? (BN >> duty.b_sh) : (BM >> duty.a_sh);
         intx4 rt = touch_b ? rb : ra;
-        if ((pw >> 1) * 64 >= share || (touch_b ? duty.b_sh : duty.a_sh) == 0) rt[2] = 0;
-        const int touch_off = ((touch_b ? duty.b_duty : duty.a_duty) * share + t_idx % share) * K;
+        if ((touch_b ? duty.b_sh : duty.a_sh) == 0) rt[2] = 0;
+        const int touch_row0 = (touch_b ? duty.b_duty : duty.a_duty) * share;
+        constexpr int TOUCH_LANES = (PW / 2) * 64;
         auto issue = [&](int i, int kb, int bufa, int bufb, int bufs) {
             const bool more = kb < kb1;
             if (i < SC)
@@ -567,7 +581,12 @@ __device__ __forceinline__ void fp8_gemm_tile_ws(
                 dma16(rb, voff, (i - SC - A_PASSES) * PASS_ROWS * K + (more ? kb * 128 : rb[2]),
                       lb_base + bufb * (BN * 128) + (i - SC - A_PASSES) * PASS_ROWS * 128);
         };
-        auto touch = [&](int kb) { dma4(rt, touch_off, kb < kb1 ? kb * 128 : rt[2], ld_base + 256); };
+        auto touch = [&](int kbp) {      // kTouchBurst consecutive lines of a row at a time (see kTouchBurst)
+            const int j = kbp & (kTouchBurst - 1), base = kbp - j;
+            const int q = j * TOUCH_LANES + t_idx, row = q >> kTouchBurstLog, line = q & (kTouchBurst - 1);
+            const bool ok = row < share && base + line < kb1;
+            dma4(rt, ok ? (touch_row0 + row) * K + (base + line) * 128 : kOutOfRange, 0, ld_base + 256);
+        };
 
         if (pw < NBS) {
             const int nb = min((n0 >> 7) + pw, ((N + 127) >> 7) - 1);
@@ -578,7 +597,7 @@ __device__ __forceinline__ void fp8_gemm_tile_ws(
         for (int blk = 0; blk < STAGES - 1; ++blk) {
 #pragma unroll
             for (int i = 0; i < NDMA; ++i) issue(i, kb0 + blk, blk % SA, blk % SB, blk % SS);
-            touch(kb0 + blk + TDA);
+            touch(kb0 + blk);                  // groups 0 .. STAGES-2 of the first burst
         }
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 2) * (NDMA + 1) + 1) : "memory");    // block kb0 has landed
         __syncthreads();
