@@ -697,7 +697,8 @@ def ceilings(torch, m, timer, dev):
              "constant operand bytes (0x38)": torch.zeros(64, dtype=torch.int32, device=dev)}
     iters = 1000
     flop = 256.0 * 8 * iters * 32 * 65536
-    for fold, label in ((0, "MFMA only, accumulating in place"), (1, "each MFMA from zero + 4 v_fma_f32 (the block-scale fold)")):
+    for fold, label in ((0, "MFMA only, accumulating in place"), (1, "each MFMA from zero + 4 v_fma_f32 (the block-scale fold)"),
+                        (2, "32x32x64 MFMAs, accumulating in place"), (3, "32x32x64 MFMAs in pairs from zero + 16 v_fma_f32 a pair")):
         for sname, seed in seeds.items():
             def fn(fold=fold, seed=seed):
                 ok(L.mdy_probe_mfma_loop(fold, seed.data_ptr(), out.data_ptr(), 256, iters, stream_ptr(dev)), "mfma_loop")

@@ -127,6 +127,63 @@ __global__ __launch_bounds__(512) void mfma_loop_kernel(const uint32_t* __restri
     out[blockIdx.x * 512 + threadIdx.x] = r;
 }
 
+// The same work per iteration (32 x 16x16x128 = 16 x 32x32x64) with v_mfma_f32_32x32x64_f8f6f4, which reads half the operand
+// bytes from the register file per multiply-add: 2 x 2 output tiles of 32x32, each with operands for 128 of K (two MFMAs),
+// two passes over them per iteration.  FOLD: the first MFMA of a pair starts from zero, the second accumulates onto it, and
+// 16 v_fma_f32 fold the pair's results (4 per 32768 multiply-adds, as with the 16x16x128 form).
+typedef float probe_floatx16 __attribute__((ext_vector_type(16)));
+template <bool FOLD>
+__global__ __launch_bounds__(512) void mfma32_loop_kernel(const uint32_t* __restrict__ seed, float* __restrict__ out, int iters, float sc) {
+    probe_intx8 fa[2][2], fb[2][2];
+    const uint32_t s0 = seed[threadIdx.x & 63];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            fa[i >> 1][i & 1][e] = s0 == 0 ? 0x38383838 : (int)(((s0 + (uint32_t)(i * 8 + e) * 2654435761u) * 2246822519u) & 0xBFBFBFBFu);
+            fb[i >> 1][i & 1][e] = s0 == 0 ? 0x38383838 : (int)(((s0 * 40503u + (uint32_t)(i * 8 + e) * 2246822519u) * 2654435761u) & 0xBFBFBFBFu);
+        }
+    probe_floatx16 acc[2][2], zero;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) zero[e] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = zero;
+    for (int it = 0; it < iters; ++it) {
+        probe_floatx16 p[2];
+#pragma unroll
+        for (int t = 0; t < 8 + 1; ++t) {
+            if (t < 8) {
+                const int i = (t >> 1) & 1, j = t & 1;
+                asm volatile("" : "+v"(fb[j][0]));      // the second pass is not the first one's common subexpression
+                if (FOLD) {
+                    p[t % 2] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[j][0], fa[i][0], zero, 0, 0, 0, 0, 0, 0);
+                    p[t % 2] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[j][1], fa[i][1], p[t % 2], 0, 0, 0, 0, 0, 0);
+                } else {
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[j][0], fa[i][0], acc[i][j], 0, 0, 0, 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[j][1], fa[i][1], acc[i][j], 0, 0, 0, 0, 0, 0);
+                }
+            }
+            if (FOLD && t >= 1) {
+                const int u = t - 1, i = (u >> 1) & 1, j = u & 1;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][j][e] = __builtin_fmaf(p[u % 2][e], sc, acc[i][j][e]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        asm volatile("" : "+v"(fa[0][0]));
+    }
+    float r = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) r += acc[i][j][e];
+    out[blockIdx.x * 512 + threadIdx.x] = r;
+}
+
 __global__ void empty_kernel() {}
 
 }  // namespace mdy
@@ -149,10 +206,18 @@ extern "C" int mdy_probe_copy_wd(const void* x, const float* s, void* y, int64_t
     return (int)hipGetLastError();
 }
 
+// fold: bit 0 = fold every MFMA's result with v_fma_f32, bit 1 = 32x32x64 instead of 16x16x128 MFMAs
 // seed: 64 uint32 (all zero: constant operand bytes 0x38 = 1.0; otherwise per-lane hash seeds); out: workgroups * 512 floats
 extern "C" int mdy_probe_mfma_loop(int fold, const void* seed, float* out, int workgroups, int iters, void* stream) {
-    if (!seed || !out || workgroups < 1 || iters < 1) return -2;
-    if (fold)
+    if (!seed || !out || workgroups < 1 || iters < 1 || fold < 0 || fold > 3) return -2;
+    if (fold & 2) {
+        if (fold & 1)
+            hipLaunchKernelGGL(mdy::mfma32_loop_kernel<true>, dim3((unsigned)workgroups), dim3(512), 0, static_cast<hipStream_t>(stream),
+                               static_cast<const uint32_t*>(seed), out, iters, 1.0f);
+        else
+            hipLaunchKernelGGL(mdy::mfma32_loop_kernel<false>, dim3((unsigned)workgroups), dim3(512), 0, static_cast<hipStream_t>(stream),
+                               static_cast<const uint32_t*>(seed), out, iters, 1.0f);
+    } else if (fold)
         hipLaunchKernelGGL(mdy::mfma_loop_kernel<true>, dim3((unsigned)workgroups), dim3(512), 0, static_cast<hipStream_t>(stream),
                            static_cast<const uint32_t*>(seed), out, iters, 1.0f);
     else

@@ -272,6 +272,146 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_kernel(const ui
 }
 
 // ---------------------------------------------------------------------------
+// Small-M kernel with whole-line loads (up to 16*MT rows).  The kernel above loads MFMA fragments straight from global
+// memory: per instruction 16 rows x 4 pieces of 16 bytes, 64 of every 128-byte line, the line's other half by the
+// next instruction.  Measured on loads alone (M=16, N=2048, K=7168, replayed graph): 8.5 us per call that way, 3.4 us
+// when every load instruction covers whole lines (8 rows x the 128 bytes of one K block: lane l has piece l & 7 of
+// row l >> 3).  So here a wave loads its K blocks that way, UF blocks before the first use, and turns a block into
+// fragments through LDS that only this wave touches - two 16-byte writes and two 16-byte reads per 16 rows, pieces
+// XOR-swizzled by the row so that both fall on all banks - which needs no barrier: every wave runs on as its own
+// loads arrive, block u+1 on its way through LDS while the MFMAs of block u run.  Wave w owns the K blocks
+// [w per, (w+1) per), per = ceil(KB / 8): no branch depends on the block, so the waits the compiler places count
+// exactly; a block beyond the wave's range is a re-read of the last valid one whose product is replaced by zero.
+// ---------------------------------------------------------------------------
+template <int MT, int NC, int UF, typename OUT, int FMT>
+__global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_lines_kernel(const uint8_t* __restrict__ a, const float* __restrict__ a_s,
+                                                                               int64_t as_rs, int64_t as_cs, const uint8_t* __restrict__ b,
+                                                                               const float* __restrict__ b_s, OUT* __restrict__ c,
+                                                                               const uint16_t* __restrict__ bias, int M, int N, int K) {
+    constexpr int SUB = NC * MT, TILES = NC + MT;      // (column group, row sub-tile) pairs; 16-row operand tiles per K block
+    static_assert(SUB <= kSmWaves, "one wave reduces one (column group, row sub-tile) pair");
+    constexpr int SV = (UF + 3) / 4;                    // activation-scale loads per row sub-tile and pass
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kSmWaves][2][TILES * 2048];
+    __shared__ float red[kSmWaves][SUB][64][4];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int frow = lane & 15, fk = lane >> 4;
+    const int r8 = lane >> 3, pc = lane & 7;
+    const int n0 = blockIdx.x * (16 * NC);
+    const int KB = K >> 7, NB = (N + 127) >> 7;
+    const int per = (KB + kSmWaves - 1) / kSmWaves;
+    const int k_begin = min(wave * per, KB), k_end = min(k_begin + per, KB);      // this wave's K blocks
+    // global: lane l loads piece l & 7 of row 8 t + (l >> 3) for t = 0, 1 of every 16-row tile
+    const uint8_t* bld[2 * NC];
+    const uint8_t* ald[2 * MT];
+#pragma unroll
+    for (int t = 0; t < 2 * NC; ++t) bld[t] = b + (int64_t)min(n0 + 8 * t + r8, N - 1) * K + pc * 16;
+#pragma unroll
+    for (int t = 0; t < 2 * MT; ++t) ald[t] = a + (int64_t)min(8 * t + r8, M - 1) * K + pc * 16;
+    const float* bsp[NC];
+    const float* asp[MT];
+#pragma unroll
+    for (int j = 0; j < NC; ++j) bsp[j] = b_s + (int64_t)min((n0 + 16 * j) >> 7, NB - 1) * KB;
+#pragma unroll
+    for (int i = 0; i < MT; ++i) asp[i] = a_s + (int64_t)min(i * 16 + frow, M - 1) * as_rs;
+    // LDS: piece p of row r of a tile at r * 128 + ((p ^ (r & 7)) * 16)
+    const int wr_off = r8 * 128 + ((pc ^ r8) << 4);                                 // + 1024 for the rows 8 .. 15
+    const int rd_lo = frow * 128 + (((2 * fk) ^ (frow & 7)) << 4), rd_hi = frow * 128 + (((2 * fk + 1) ^ (frow & 7)) << 4);
+
+    floatx4 acc[NC][MT];
+#pragma unroll
+    for (int j = 0; j < NC; ++j)
+#pragma unroll
+        for (int i = 0; i < MT; ++i) acc[j][i] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    for (int kp = k_begin; kp < k_end; kp += UF) {      // uniform in the wave
+        intx4 vb[UF][2 * NC], va[UF][2 * MT];      // plain vectors: a struct type here ends up in scratch memory
+        float sb[UF][NC], sraw[SV][MT];
+#pragma unroll
+        for (int u = 0; u < UF; ++u) {
+            const int kb = min(kp + u, k_end - 1);
+#pragma unroll
+            for (int t = 0; t < 2 * NC; ++t) vb[u][t] = __builtin_nontemporal_load(reinterpret_cast<const intx4*>(bld[t] + (int64_t)kb * 128));
+#pragma unroll
+            for (int t = 0; t < 2 * MT; ++t) va[u][t] = *reinterpret_cast<const intx4*>(ald[t] + (int64_t)kb * 128);
+#pragma unroll
+            for (int j = 0; j < NC; ++j) sb[u][j] = bsp[j][kb];
+        }
+        // the activation scales: one load per lane and K block of its row touches 16 lines for 64 bytes (UF of them cost
+        // 1.5 us per call), so the 4 lanes of a row each load another block's scale and hand it over when it is needed
+#pragma unroll
+        for (int v = 0; v < SV; ++v) {
+            const int kb = min(kp + fk + 4 * v, k_end - 1);
+#pragma unroll
+            for (int i = 0; i < MT; ++i) sraw[v][i] = asp[i][(int64_t)kb * as_cs];
+        }
+        intx8 fa[2][MT], fb[2][NC];
+        auto through_lds = [&](int u) {      // block u of the pass: registers -> this wave's LDS -> fragments
+            uint8_t* buf = lds[wave][u & 1];
+#pragma unroll
+            for (int t = 0; t < 2 * NC; ++t) *reinterpret_cast<intx4*>(buf + t * 1024 + wr_off) = vb[u][t];
+#pragma unroll
+            for (int t = 0; t < 2 * MT; ++t) *reinterpret_cast<intx4*>(buf + (2 * NC + t) * 1024 + wr_off) = va[u][t];
+#pragma unroll
+            for (int j = 0; j < NC; ++j) {
+                const intx4 lo = *reinterpret_cast<const intx4*>(buf + j * 2048 + rd_lo), hi = *reinterpret_cast<const intx4*>(buf + j * 2048 + rd_hi);
+                fb[u & 1][j] = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            }
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                const uint8_t* src = buf + (NC + i) * 2048;
+                const intx4 lo = *reinterpret_cast<const intx4*>(src + rd_lo), hi = *reinterpret_cast<const intx4*>(src + rd_hi);
+                fa[u & 1][i] = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            }
+        };
+        through_lds(0);
+#pragma unroll
+        for (int u = 0; u < UF; ++u) {
+            if (u + 1 < UF) through_lds(u + 1);
+            const bool valid = kp + u < k_end;      // uniform in the wave
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                const float sa = __int_as_float(__builtin_amdgcn_ds_bpermute((frow + 16 * (u & 3)) << 2, __float_as_int(sraw[u >> 2][i])));
+#pragma unroll
+                for (int j = 0; j < NC; ++j) {
+                    floatx4 p = mfma_block<FMT>(fb[u & 1][j], fa[u & 1][i]);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) p[e] = valid ? p[e] : 0.0f;
+                    fold(acc[j][i], p, sa * sb[u][j]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < NC; ++j)
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) red[wave][j * MT + i][lane][e] = acc[j][i][e];
+    __syncthreads();
+    if (wave < SUB) {
+        // wave (j, i) reduces column group j, row sub-tile i (fixed order, so results do not depend on timing)
+        const int j = wave / MT, i = wave % MT;
+        const bool vec_ok = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float t = 0.0f;
+#pragma unroll
+            for (int w = 0; w < kSmWaves; ++w) t += red[w][wave][lane][e];
+            v[e] = t;
+        }
+        const int m = i * 16 + frow, n = n0 + 16 * j + 4 * fk;
+        if (bias != nullptr) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (n + e < N) v[e] += bf16_one(bias[n + e]);
+        }
+        store4<OUT>(c, N, m, n, M, N, v, vec_ok);
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Row-vector kernel: M <= 4 rows (single-token decode).  No matrix cores: a weight row against one activation row is a
 // dot product, and what bounds it is how many weight bytes every CU has in flight.  A wave owns R weight rows and
 // issues all of their loads up front (16 bytes per lane, 1 KB per load and row: K = 7168 -> 7 KB per row in flight), a
@@ -734,6 +874,37 @@ static int dispatch_small(const uint8_t* a, const float* a_s, int64_t as_rs, int
         return launch_mfma<128, 128, 2, 2, 4, OUT, FMT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
     if (M >= 32 && M <= 64 && big_ok && (N + 63) / 64 >= 100)
         return launch_mfma<64, 64, 2, 2, 8, OUT, FMT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
+    if (M <= 16) {
+        // 32 columns per workgroup when that still leaves ~200 workgroups (loads alone, M=16: N=7168, K=2048 2.9 -> 2.5 us
+        // per call; N=2048, K=7168 3.4 -> 4.1 us); the K blocks of a wave in passes of up to 8
+        const bool wide = (N + 31) / 32 >= 200;
+        const int per = (K / 128 + kSmWaves - 1) / kSmWaves;
+        int uf = per;
+        if (per > 8) uf = per % 8 == 0 ? 8 : per % 7 == 0 ? 7 : per % 6 == 0 ? 6 : per % 5 == 0 ? 5 : 8;
+        dim3 grid((unsigned)(wide ? (N + 31) / 32 : (N + 15) / 16));
+#define MDY_LINES(NC, UF)                                                                                                          \
+    hipLaunchKernelGGL((fp8_gemm_smallm_lines_kernel<1, NC, UF, OUT, FMT>), grid, dim3(kSmWaves * 64), 0, stream, a, a_s, as_rs, as_cs, b, \
+                       b_s, c, bias, M, N, K)
+#define MDY_LINES_UF(NC)                          \
+    switch (uf) {                                 \
+        case 1: MDY_LINES(NC, 1); break;          \
+        case 2: MDY_LINES(NC, 2); break;          \
+        case 3: MDY_LINES(NC, 3); break;          \
+        case 4: MDY_LINES(NC, 4); break;          \
+        case 5: MDY_LINES(NC, 5); break;          \
+        case 6: MDY_LINES(NC, 6); break;          \
+        case 7: MDY_LINES(NC, 7); break;          \
+        default: MDY_LINES(NC, 8); break;         \
+    }
+        if (wide) {
+            MDY_LINES_UF(2)
+        } else {
+            MDY_LINES_UF(1)
+        }
+#undef MDY_LINES_UF
+#undef MDY_LINES
+        return (int)hipGetLastError();
+    }
     if (M <= 64) {
         // one workgroup streams 16 weight columns against MT row sub-tiles; every workgroup re-reads its rows of
         // a, so with few column groups (N small) the rows are split over grid.y as well: more workgroups, less
