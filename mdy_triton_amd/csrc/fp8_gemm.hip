@@ -863,9 +863,57 @@ static int dispatch_small(const uint8_t* a, const float* a_s, int64_t as_rs, int
 #undef MDY_GEMV
         return (int)hipGetLastError();
     }
-    if (M <= 64 && big_ok && strip_pays(M, (N + 127) / 128)) {
+    // up to 24 rows, and up to 32 unless the weight is very wide, run the whole-line kernel (measured, K=7168: M=32 N=16384
+    // 31.3 us there, 34.9 us on 128x128 tiles; N=18432 42.0 against 34.8 us; M=32 N=129280 240 against 206 us on strips;
+    // M=16 N=129280 161 against 182 us on strips; M=24 N=25600 K=4096 28.3 against 34.6 us)
+    const bool lines = M <= 24 || (M <= 32 && (N + 127) / 128 < 136);
+    if (!lines && M <= 64 && big_ok && strip_pays(M, (N + 127) / 128)) {
         const int64_t one = M;
         return launch_strip<OUT, FMT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, &one, 1, M, N, K, stream);
+    }
+    if (lines) {
+        // 32 columns per workgroup when that still leaves ~200 workgroups (loads alone, M=16: N=7168, K=2048 2.9 -> 2.5 us
+        // per call; N=2048, K=7168 3.4 -> 4.1 us); the K blocks of a wave in passes of up to 8 (up to 16 rows) or 4
+        const bool wide = (N + 31) / 32 >= 200;
+        const int per = (K / 128 + kSmWaves - 1) / kSmWaves, cap = M <= 16 ? 8 : 4;
+        int uf = per;
+        if (per > cap) {
+            uf = cap;
+            for (int d = cap; d > cap / 2; --d)
+                if (per % d == 0) { uf = d; break; }
+        }
+        dim3 grid((unsigned)(wide ? (N + 31) / 32 : (N + 15) / 16));
+#define MDY_LINES(MT, NC, UF)                                                                                                       \
+    hipLaunchKernelGGL((fp8_gemm_smallm_lines_kernel<MT, NC, UF, OUT, FMT>), grid, dim3(kSmWaves * 64), 0, stream, a, a_s, as_rs, as_cs, b, \
+                       b_s, c, bias, M, N, K)
+#define MDY_LINES_UF4(MT, NC)                         \
+    switch (uf) {                                     \
+        case 1: MDY_LINES(MT, NC, 1); break;          \
+        case 2: MDY_LINES(MT, NC, 2); break;          \
+        case 3: MDY_LINES(MT, NC, 3); break;          \
+        default: MDY_LINES(MT, NC, 4); break;         \
+    }
+#define MDY_LINES_UF8(MT, NC)                         \
+    switch (uf) {                                     \
+        case 5: MDY_LINES(MT, NC, 5); break;          \
+        case 6: MDY_LINES(MT, NC, 6); break;          \
+        case 7: MDY_LINES(MT, NC, 7); break;          \
+        case 8: MDY_LINES(MT, NC, 8); break;          \
+        default: MDY_LINES_UF4(MT, NC)                \
+    }
+        if (M <= 16 && wide) {
+            MDY_LINES_UF8(1, 2)
+        } else if (M <= 16) {
+            MDY_LINES_UF8(1, 1)
+        } else if (wide) {
+            MDY_LINES_UF4(2, 2)
+        } else {
+            MDY_LINES_UF4(2, 1)
+        }
+#undef MDY_LINES_UF8
+#undef MDY_LINES_UF4
+#undef MDY_LINES
+        return (int)hipGetLastError();
     }
     // 32..64 rows against a wide weight: the kernel below re-reads the activation rows in every one of its
     // N/16 workgroups, and from 32 rows on that traffic costs more than the empty rows of an MFMA tile.
@@ -874,37 +922,6 @@ static int dispatch_small(const uint8_t* a, const float* a_s, int64_t as_rs, int
         return launch_mfma<128, 128, 2, 2, 4, OUT, FMT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
     if (M >= 32 && M <= 64 && big_ok && (N + 63) / 64 >= 100)
         return launch_mfma<64, 64, 2, 2, 8, OUT, FMT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
-    if (M <= 16) {
-        // 32 columns per workgroup when that still leaves ~200 workgroups (loads alone, M=16: N=7168, K=2048 2.9 -> 2.5 us
-        // per call; N=2048, K=7168 3.4 -> 4.1 us); the K blocks of a wave in passes of up to 8
-        const bool wide = (N + 31) / 32 >= 200;
-        const int per = (K / 128 + kSmWaves - 1) / kSmWaves;
-        int uf = per;
-        if (per > 8) uf = per % 8 == 0 ? 8 : per % 7 == 0 ? 7 : per % 6 == 0 ? 6 : per % 5 == 0 ? 5 : 8;
-        dim3 grid((unsigned)(wide ? (N + 31) / 32 : (N + 15) / 16));
-#define MDY_LINES(NC, UF)                                                                                                          \
-    hipLaunchKernelGGL((fp8_gemm_smallm_lines_kernel<1, NC, UF, OUT, FMT>), grid, dim3(kSmWaves * 64), 0, stream, a, a_s, as_rs, as_cs, b, \
-                       b_s, c, bias, M, N, K)
-#define MDY_LINES_UF(NC)                          \
-    switch (uf) {                                 \
-        case 1: MDY_LINES(NC, 1); break;          \
-        case 2: MDY_LINES(NC, 2); break;          \
-        case 3: MDY_LINES(NC, 3); break;          \
-        case 4: MDY_LINES(NC, 4); break;          \
-        case 5: MDY_LINES(NC, 5); break;          \
-        case 6: MDY_LINES(NC, 6); break;          \
-        case 7: MDY_LINES(NC, 7); break;          \
-        default: MDY_LINES(NC, 8); break;         \
-    }
-        if (wide) {
-            MDY_LINES_UF(2)
-        } else {
-            MDY_LINES_UF(1)
-        }
-#undef MDY_LINES_UF
-#undef MDY_LINES
-        return (int)hipGetLastError();
-    }
     if (M <= 64) {
         // one workgroup streams 16 weight columns against MT row sub-tiles; every workgroup re-reads its rows of
         // a, so with few column groups (N small) the rows are split over grid.y as well: more workgroups, less
@@ -1148,6 +1165,7 @@ int fp8_gemm_path(const void* a, const void* b, int64_t as_rs, int64_t as_cs, in
     const bool big_ok = mfma_ok && K <= (1 << 16) && as_rs >= 0 && as_cs >= 0 && as_extent < ((int64_t)1 << 31);
     if (with_workspace && big_ok && plan_split(M, N, K).ksplit > 1) return 4;
     if (!mfma_ok || (M > 64 && !big_ok)) return 0;
+    if (M <= 24 || (M <= 32 && (N + 127) / 128 < 136)) return 1;
     if (M <= 64 && big_ok && strip_pays(M, (N + 127) / 128)) return 2;
     if (M >= 32 && M <= 64 && big_ok && ((N + 127) / 128 >= 128 || (N + 63) / 64 >= 100)) return 3;
     if (M <= 64) return 1;

@@ -324,6 +324,24 @@ def test_gemm_row_vector_kernel_exact_integer(M, N, K, fmt):
     integer operands with power-of-two scales through the C entry points, row- and column-major activation scales, bias,
     fp32 and bf16 output, N not a multiple of the rows per workgroup, both fp8 formats; K beyond its LDS staging
     (16384) goes to the MFMA weight-streaming kernel and gives the same exact result."""
+    _small_m_exact_through_c_abi(M, N, K, fmt, longer_k=(fmt == "e4m3fn"))
+
+
+@pytest.mark.parametrize("fmt", ["e4m3fn", "e5m2"])
+@pytest.mark.parametrize("M,N,K", [(16, 2048, 7168), (16, 7168, 2048), (5, 272, 128), (8, 1000, 1024), (9, 6401, 3072),
+                                   (12, 1536, 1536), (16, 530, 4096), (13, 6500, 5120), (7, 333, 6144), (16, 4096, 8192),
+                                   (11, 520, 16384), (16, 300, 18432), (6, 290, 9344), (15, 7000, 2176),
+                                   (17, 2048, 7168), (32, 7168, 2048), (24, 777, 1024), (31, 6410, 2176), (20, 515, 3072),
+                                   (32, 1000, 4096), (25, 300, 16384), (32, 290, 9344)])
+def test_gemm_whole_line_kernel_exact_integer(M, N, K, fmt):
+    """5..32 rows run on the whole-line kernel (one or two 16-row activation tiles, 16 or 32 weight columns per workgroup
+    by N, 1..8 K blocks per wave and pass by K, several passes for long K, K-block counts that are no multiple of the 8
+    waves so that some waves get fewer blocks or none): exact on integer operands with power-of-two scales through the C
+    entry points, row- and column-major activation scales, bias, fp32 and bf16 output, ragged N, both fp8 formats."""
+    _small_m_exact_through_c_abi(M, N, K, fmt, longer_k=False)
+
+
+def _small_m_exact_through_c_abi(M, N, K, fmt, longer_k):
     dt = FP8 if fmt == "e4m3fn" else torch.float8_e5m2
     lib = _lib.load()
     entry = lib.mdy_fp8_gemm_nt if fmt == "e4m3fn" else lib.mdy_fp8_gemm_nt_e5m2
@@ -349,7 +367,7 @@ def test_gemm_row_vector_kernel_exact_integer(M, N, K, fmt):
                              bp.data_ptr() if bp is not None else None, M, N, K, code, None) == 0
                 torch.cuda.synchronize()
                 assert torch.equal(out.cpu().double(), want.to(dtype).double())
-    if fmt == "e4m3fn":       # a longer K than the kernel stages: the MFMA kernel, same exact result
+    if longer_k:              # a longer K than the kernel stages: the MFMA kernel, same exact result
         K2 = 16384 + 128
         a2 = torch.zeros(M, K2, dtype=torch.uint8, device=DEV).view(dt)
         b2 = torch.zeros(N, K2, dtype=torch.uint8, device=DEV).view(dt)
