@@ -291,7 +291,8 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_lines_kernel(co
     constexpr int SUB = NC * MT, TILES = NC + MT;      // (column group, row sub-tile) pairs; 16-row operand tiles per K block
     static_assert(SUB <= kSmWaves, "one wave reduces one (column group, row sub-tile) pair");
     constexpr int SV = (UF + 3) / 4;                    // activation-scale loads per row sub-tile and pass
-    __shared__ __attribute__((aligned(16))) uint8_t lds[kSmWaves][2][TILES * 2048];
+    constexpr int NBUF = MT < 4 ? 2 : 1;               // LDS regions and fragment sets per wave (64 rows: no room for two)
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kSmWaves][NBUF][TILES * 2048];
     __shared__ float red[kSmWaves][SUB][64][4];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -345,9 +346,9 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_lines_kernel(co
 #pragma unroll
             for (int i = 0; i < MT; ++i) sraw[v][i] = asp[i][(int64_t)kb * as_cs];
         }
-        intx8 fa[2][MT], fb[2][NC];
+        intx8 fa[NBUF][MT], fb[NBUF][NC];
         auto through_lds = [&](int u) {      // block u of the pass: registers -> this wave's LDS -> fragments
-            uint8_t* buf = lds[wave][u & 1];
+            uint8_t* buf = lds[wave][u % NBUF];
 #pragma unroll
             for (int t = 0; t < 2 * NC; ++t) *reinterpret_cast<intx4*>(buf + t * 1024 + wr_off) = vb[u][t];
 #pragma unroll
@@ -355,26 +356,27 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_lines_kernel(co
 #pragma unroll
             for (int j = 0; j < NC; ++j) {
                 const intx4 lo = *reinterpret_cast<const intx4*>(buf + j * 2048 + rd_lo), hi = *reinterpret_cast<const intx4*>(buf + j * 2048 + rd_hi);
-                fb[u & 1][j] = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                fb[u % NBUF][j] = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             }
 #pragma unroll
             for (int i = 0; i < MT; ++i) {
                 const uint8_t* src = buf + (NC + i) * 2048;
                 const intx4 lo = *reinterpret_cast<const intx4*>(src + rd_lo), hi = *reinterpret_cast<const intx4*>(src + rd_hi);
-                fa[u & 1][i] = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                fa[u % NBUF][i] = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             }
         };
-        through_lds(0);
+        if (NBUF == 2) through_lds(0);
 #pragma unroll
         for (int u = 0; u < UF; ++u) {
-            if (u + 1 < UF) through_lds(u + 1);
+            if (NBUF == 1) through_lds(u);
+            else if (u + 1 < UF) through_lds(u + 1);
             const bool valid = kp + u < k_end;      // uniform in the wave
 #pragma unroll
             for (int i = 0; i < MT; ++i) {
                 const float sa = __int_as_float(__builtin_amdgcn_ds_bpermute((frow + 16 * (u & 3)) << 2, __float_as_int(sraw[u >> 2][i])));
 #pragma unroll
                 for (int j = 0; j < NC; ++j) {
-                    floatx4 p = mfma_block<FMT>(fb[u & 1][j], fa[u & 1][i]);
+                    floatx4 p = mfma_block<FMT>(fb[u % NBUF][j], fa[u % NBUF][i]);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) p[e] = valid ? p[e] : 0.0f;
                     fold(acc[j][i], p, sa * sb[u][j]);
@@ -834,6 +836,17 @@ static bool gemv_pays(int64_t M, int64_t K) { return M <= 4 && K <= kGemvMaxK; }
 
 // few rows per group and enough 128-column strips to fill the CUs without splitting K (with a handful of rows the
 // 16-column kernel re-reads so little of a that it stays ahead)
+// The whole-line small-M kernel (5 or more rows; K % 128 == 0, 16-byte aligned operands: the caller checks): up to 24
+// rows always, up to 32 unless the weight is very wide, up to 64 for a middling N.  Measured per call in a replayed graph,
+// K=7168 unless noted: M=32 N=16384 31.3 us there, 34.9 us on 128x128 tiles; N=18432 42.0 against 34.8 us; M=32 N=129280
+// 240 against 206 us on strips; M=16 N=129280 161 against 182 us on strips; M=24 N=25600 K=4096 28.3 against 34.6 us;
+// M=64 N=7168 K=2048 6.6 against 8.7 us on 64x64 tiles, N=12800 K=2048 11.7 against 8.9 us, N=4096 17.1 against 24.8 us on
+// the fragment-loading kernel, N=2048 16.2 against 15.5 us.
+static bool lines_pays(int64_t M, int64_t N) {
+    const int64_t strips = (N + 127) / 128;
+    return M > 4 && (M <= 24 || (M <= 32 && strips < 136) || (M <= 64 && N >= 3200 && strips < 100));
+}
+
 static bool strip_pays(int64_t max_rows, int64_t strips) { return max_rows > 4 && max_rows <= 64 && strips >= 200; }
 
 // Up to 64 rows (K % 128 == 0, aligned operands: the caller checks; big_ok: the scales also fit the tile kernels'
@@ -866,7 +879,7 @@ static int dispatch_small(const uint8_t* a, const float* a_s, int64_t as_rs, int
     // up to 24 rows, and up to 32 unless the weight is very wide, run the whole-line kernel (measured, K=7168: M=32 N=16384
     // 31.3 us there, 34.9 us on 128x128 tiles; N=18432 42.0 against 34.8 us; M=32 N=129280 240 against 206 us on strips;
     // M=16 N=129280 161 against 182 us on strips; M=24 N=25600 K=4096 28.3 against 34.6 us)
-    const bool lines = M <= 24 || (M <= 32 && (N + 127) / 128 < 136);
+    const bool lines = lines_pays(M, N);
     if (!lines && M <= 64 && big_ok && strip_pays(M, (N + 127) / 128)) {
         const int64_t one = M;
         return launch_strip<OUT, FMT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, &one, 1, M, N, K, stream);
@@ -875,7 +888,7 @@ static int dispatch_small(const uint8_t* a, const float* a_s, int64_t as_rs, int
         // 32 columns per workgroup when that still leaves ~200 workgroups (loads alone, M=16: N=7168, K=2048 2.9 -> 2.5 us
         // per call; N=2048, K=7168 3.4 -> 4.1 us); the K blocks of a wave in passes of up to 8 (up to 16 rows) or 4
         const bool wide = (N + 31) / 32 >= 200;
-        const int per = (K / 128 + kSmWaves - 1) / kSmWaves, cap = M <= 16 ? 8 : 4;
+        const int per = (K / 128 + kSmWaves - 1) / kSmWaves, cap = M <= 16 ? 8 : M <= 32 ? 4 : 2;
         int uf = per;
         if (per > cap) {
             uf = cap;
@@ -905,10 +918,16 @@ static int dispatch_small(const uint8_t* a, const float* a_s, int64_t as_rs, int
             MDY_LINES_UF8(1, 2)
         } else if (M <= 16) {
             MDY_LINES_UF8(1, 1)
-        } else if (wide) {
+        } else if (M <= 32 && wide) {
             MDY_LINES_UF4(2, 2)
-        } else {
+        } else if (M <= 32) {
             MDY_LINES_UF4(2, 1)
+        } else if (wide) {
+            if (uf == 1) MDY_LINES(4, 2, 1);
+            else MDY_LINES(4, 2, 2);
+        } else {
+            if (uf == 1) MDY_LINES(4, 1, 1);
+            else MDY_LINES(4, 1, 2);
         }
 #undef MDY_LINES_UF8
 #undef MDY_LINES_UF4
@@ -1031,6 +1050,8 @@ static SplitPlan plan_split(int64_t M, int64_t N, int64_t K) {
     const int KB = (int)(K / 128);
     if (big_tiles_pay(M, N) || KB < 32) return p;
     if (M <= 64 && strip_pays(M, (N + 127) / 128)) return p;
+    // up to 32 K blocks the whole-line kernel is as fast without the second pass (M=64 N=6400 K=4096: 10.6 against 12.9 us)
+    if (lines_pays(M, N) && KB <= 32) return p;
     // the largest tile that, cut into slabs of at least 8 K blocks, still yields a workgroup for most CUs
     const long rows128 = (M + 127) / 128, rows64 = (M + 63) / 64;
     const long cols128 = (N + 127) / 128, cols64 = (N + 63) / 64;
@@ -1165,7 +1186,7 @@ int fp8_gemm_path(const void* a, const void* b, int64_t as_rs, int64_t as_cs, in
     const bool big_ok = mfma_ok && K <= (1 << 16) && as_rs >= 0 && as_cs >= 0 && as_extent < ((int64_t)1 << 31);
     if (with_workspace && big_ok && plan_split(M, N, K).ksplit > 1) return 4;
     if (!mfma_ok || (M > 64 && !big_ok)) return 0;
-    if (M <= 24 || (M <= 32 && (N + 127) / 128 < 136)) return 1;
+    if (lines_pays(M, N)) return 1;
     if (M <= 64 && big_ok && strip_pays(M, (N + 127) / 128)) return 2;
     if (M >= 32 && M <= 64 && big_ok && ((N + 127) / 128 >= 128 || (N + 63) / 64 >= 100)) return 3;
     if (M <= 64) return 1;

@@ -332,12 +332,14 @@ def test_gemm_row_vector_kernel_exact_integer(M, N, K, fmt):
                                    (12, 1536, 1536), (16, 530, 4096), (13, 6500, 5120), (7, 333, 6144), (16, 4096, 8192),
                                    (11, 520, 16384), (16, 300, 18432), (6, 290, 9344), (15, 7000, 2176),
                                    (17, 2048, 7168), (32, 7168, 2048), (24, 777, 1024), (31, 6410, 2176), (20, 515, 3072),
-                                   (32, 1000, 4096), (25, 300, 16384), (32, 290, 9344)])
+                                   (32, 1000, 4096), (25, 300, 16384), (32, 290, 9344),
+                                   (64, 7168, 2048), (33, 3201, 1024), (48, 6402, 4096), (64, 3300, 2176), (50, 4099, 128)])
 def test_gemm_whole_line_kernel_exact_integer(M, N, K, fmt):
-    """5..32 rows run on the whole-line kernel (one or two 16-row activation tiles, 16 or 32 weight columns per workgroup
-    by N, 1..8 K blocks per wave and pass by K, several passes for long K, K-block counts that are no multiple of the 8
-    waves so that some waves get fewer blocks or none): exact on integer operands with power-of-two scales through the C
-    entry points, row- and column-major activation scales, bias, fp32 and bf16 output, ragged N, both fp8 formats."""
+    """5..32 rows, and up to 64 against a middling N, run on the whole-line kernel (one, two or four 16-row activation
+    tiles, 16 or 32 weight columns per workgroup by N, 1..8 K blocks per wave and pass by K, several passes for long K,
+    K-block counts that are no multiple of the 8 waves so that some waves get fewer blocks or none): exact on integer
+    operands with power-of-two scales through the C entry points, row- and column-major activation scales, bias, fp32
+    and bf16 output, ragged N, both fp8 formats."""
     _small_m_exact_through_c_abi(M, N, K, fmt, longer_k=False)
 
 
