@@ -414,7 +414,8 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_lines_kernel(co
 }
 
 // ---------------------------------------------------------------------------
-// Row-vector kernel: M <= 4 rows (single-token decode).  No matrix cores: a weight row against one activation row is a
+// Row-vector kernel: written for up to 4 rows, used for one (single-token decode against a long K: see gemv_pays).  No
+// matrix cores: a weight row against one activation row is a
 // dot product, and what bounds it is how many weight bytes every CU has in flight.  A wave owns R weight rows and
 // issues all of their loads up front (16 bytes per lane, 1 KB per load and row: K = 7168 -> 7 KB per row in flight), a
 // workgroup of 8 waves covers 8 R consecutive rows, so N = 2048 still gives 256 workgroups where the 16-column MFMA
@@ -830,9 +831,11 @@ static int launch_strip(const uint8_t* a, const float* a_s, int64_t as_rs, int64
     return (int)hipGetLastError();
 }
 
-// up to 4 rows whose activations fit the row-vector kernel's LDS staging (K % 128 == 0, 16-byte aligned operands: the
-// caller checks)
-static bool gemv_pays(int64_t M, int64_t K) { return M <= 4 && K <= kGemvMaxK; }
+// The row-vector kernel: one row against a long K that fits its LDS staging (K % 128 == 0, 16-byte aligned operands: the
+// caller checks).  With 2..4 rows, and with one row and a K of up to 4096, the whole-line MFMA kernel is ahead (per call
+// in a replayed graph: M=4 N=2048 K=7168 9.3 us here, 5.5 there; M=2 N=7168 K=2048 7.3 against 3.9; M=1 N=7168 K=2048
+// 5.4 against 3.8; M=1 N=4096 K=4096 5.0 against 4.4; but M=1 N=2048 K=7168 4.0 against 5.0, N=18432 24.5 against 26.6).
+static bool gemv_pays(int64_t M, int64_t K) { return M == 1 && K > 4096 && K <= kGemvMaxK; }
 
 // few rows per group and enough 128-column strips to fill the CUs without splitting K (with a handful of rows the
 // 16-column kernel re-reads so little of a that it stays ahead)
@@ -844,7 +847,7 @@ static bool gemv_pays(int64_t M, int64_t K) { return M <= 4 && K <= kGemvMaxK; }
 // the fragment-loading kernel, N=2048 16.2 against 15.5 us.
 static bool lines_pays(int64_t M, int64_t N) {
     const int64_t strips = (N + 127) / 128;
-    return M > 4 && (M <= 24 || (M <= 32 && strips < 136) || (M <= 64 && N >= 3200 && strips < 100));
+    return (M <= 24 || (M <= 32 && strips < 136) || (M <= 64 && N >= 3200 && strips < 100));
 }
 
 static bool strip_pays(int64_t max_rows, int64_t strips) { return max_rows > 4 && max_rows <= 64 && strips >= 200; }
@@ -855,25 +858,8 @@ template <typename OUT, int FMT>
 static int dispatch_small(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, int64_t as_extent, bool big_ok,
                           const uint8_t* b, const float* b_s, OUT* c, const uint16_t* bias, int M, int N, int K, hipStream_t stream) {
     if (gemv_pays(M, K)) {
-        // rows per wave: 8 KB of weight bytes in flight per wave (4 rows of up to 2 KB, 2 of up to 4 KB, else 1), fewer
-        // when that would leave less than ~220 workgroups
-        int r = K <= 2048 ? 4 : K <= 4096 ? 2 : 1;
-        while (r > 1 && (int64_t)N / (8 * r) < 220) r >>= 1;
-        dim3 grid((unsigned)((N + 8 * r - 1) / (8 * r))), block(512);
-#define MDY_GEMV(MR, R)                                                                                               \
-    hipLaunchKernelGGL((fp8_gemv_kernel<MR, R, OUT, FMT>), grid, block, 0, stream, a, a_s, as_rs, as_cs, b, b_s, c, bias, N, K)
-#define MDY_GEMV_R(MR)                              \
-    do {                                            \
-        if (r == 1) MDY_GEMV(MR, 1);                \
-        else if (r == 2) MDY_GEMV(MR, 2);           \
-        else MDY_GEMV(MR, 4);                       \
-    } while (0)
-        if (M == 1) MDY_GEMV_R(1);
-        else if (M == 2) MDY_GEMV_R(2);
-        else if (M == 3) MDY_GEMV_R(3);
-        else MDY_GEMV_R(4);
-#undef MDY_GEMV_R
-#undef MDY_GEMV
+        dim3 grid((unsigned)((N + 7) / 8)), block(512);      // one weight row per wave
+        hipLaunchKernelGGL((fp8_gemv_kernel<1, 1, OUT, FMT>), grid, block, 0, stream, a, a_s, as_rs, as_cs, b, b_s, c, bias, N, K);
         return (int)hipGetLastError();
     }
     // up to 24 rows, and up to 32 unless the weight is very wide, run the whole-line kernel (measured, K=7168: M=32 N=16384

@@ -318,12 +318,13 @@ def test_gemm_small_m_exact(M):
 
 @pytest.mark.parametrize("fmt", ["e4m3fn", "e5m2"])
 @pytest.mark.parametrize("M,N,K", [(1, 2048, 7168), (1, 7168, 2048), (2, 1000, 4096), (3, 259, 128), (4, 7001, 1024), (4, 520, 16384),
-                                   (1, 33, 1664), (2, 4096, 3072)])
+                                   (1, 33, 1664), (2, 4096, 3072), (1, 777, 8192), (1, 1000, 16384), (1, 2050, 4224)])
 def test_gemm_row_vector_kernel_exact_integer(M, N, K, fmt):
-    """Up to 4 rows run on the row-vector kernel (no matrix cores; 1, 2 or 4 weight rows per wave by K and N): exact on
+    """One row against a K of 4224..16384 runs on the row-vector kernel (no matrix cores, one weight row per wave); the
+    other shapes here (2..4 rows, short K) run on the whole-line MFMA kernel with a mostly empty row tile: exact on
     integer operands with power-of-two scales through the C entry points, row- and column-major activation scales, bias,
-    fp32 and bf16 output, N not a multiple of the rows per workgroup, both fp8 formats; K beyond its LDS staging
-    (16384) goes to the MFMA weight-streaming kernel and gives the same exact result."""
+    fp32 and bf16 output, N not a multiple of the rows per workgroup, both fp8 formats; K beyond the row-vector kernel's
+    LDS staging (16384) goes to an MFMA kernel and gives the same exact result."""
     _small_m_exact_through_c_abi(M, N, K, fmt, longer_k=(fmt == "e4m3fn"))
 
 
