@@ -284,10 +284,9 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_kernel(const ui
 // exactly; a block beyond the wave's range is a re-read of the last valid one whose product is replaced by zero.
 // ---------------------------------------------------------------------------
 template <int MT, int NC, int UF, typename OUT, int FMT>
-__global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_lines_kernel(const uint8_t* __restrict__ a, const float* __restrict__ a_s,
-                                                                               int64_t as_rs, int64_t as_cs, const uint8_t* __restrict__ b,
-                                                                               const float* __restrict__ b_s, OUT* __restrict__ c,
-                                                                               const uint16_t* __restrict__ bias, int M, int N, int K) {
+__device__ __forceinline__ void smallm_lines_body(const uint8_t* __restrict__ a, const float* __restrict__ a_s, int64_t as_rs, int64_t as_cs,
+                                                  const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
+                                                  const uint16_t* __restrict__ bias, int M, int N, int K) {
     constexpr int SUB = NC * MT, TILES = NC + MT;      // (column group, row sub-tile) pairs; 16-row operand tiles per K block
     static_assert(SUB <= kSmWaves, "one wave reduces one (column group, row sub-tile) pair");
     constexpr int SV = (UF + 3) / 4;                    // activation-scale loads per row sub-tile and pass
@@ -411,6 +410,35 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_lines_kernel(co
         }
         store4<OUT>(c, N, m, n, M, N, v, vec_ok);
     }
+}
+
+template <int MT, int NC, int UF, typename OUT, int FMT>
+__global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_lines_kernel(const uint8_t* __restrict__ a, const float* __restrict__ a_s,
+                                                                               int64_t as_rs, int64_t as_cs, const uint8_t* __restrict__ b,
+                                                                               const float* __restrict__ b_s, OUT* __restrict__ c,
+                                                                               const uint16_t* __restrict__ bias, int M, int N, int K) {
+    smallm_lines_body<MT, NC, UF, OUT, FMT>(a, a_s, as_rs, as_cs, b, b_s, c, bias, M, N, K);
+}
+
+// The same for a grouped GEMM whose groups have at most 16*MT rows each (routed experts at decode): blockIdx.y is the group,
+// its rows, weight, weight scales, bias and output rows are the operands of an ordinary small-M GEMM.
+struct GroupRows {
+    int row_start[kMaxGroups + 1];   // first row of group g; [G] = total rows
+};
+
+template <int MT, int NC, int UF, typename OUT>
+__global__ __launch_bounds__(kSmWaves * 64) void fp8_grouped_lines_kernel(const uint8_t* __restrict__ a, const float* __restrict__ a_s,
+                                                                           int64_t as_rs, int64_t as_cs, const uint8_t* __restrict__ b,
+                                                                           const float* __restrict__ b_s, OUT* __restrict__ c,
+                                                                           const uint16_t* __restrict__ bias, int N, int K,
+                                                                           const GroupRows rows) {
+    const int g = blockIdx.y;
+    const int r0 = __builtin_amdgcn_readfirstlane(rows.row_start[g]);
+    const int M = __builtin_amdgcn_readfirstlane(rows.row_start[g + 1]) - r0;
+    if (M <= 0) return;      // uniform in the workgroup
+    const int KB = K >> 7, NB = (N + 127) >> 7;
+    smallm_lines_body<MT, NC, UF, OUT, 0>(a + (size_t)r0 * K, a_s + (int64_t)r0 * as_rs, as_rs, as_cs, b + (size_t)g * N * K,
+                                          b_s + (size_t)g * NB * KB, c + (size_t)r0 * N, bias ? bias + (size_t)g * N : nullptr, M, N, K);
 }
 
 // ---------------------------------------------------------------------------
@@ -1287,6 +1315,46 @@ static int launch_grouped(const uint8_t* a, const float* a_s, int64_t as_rs, int
     return (int)hipGetLastError();
 }
 
+// Groups of at most 64 rows each on the whole-line small-M kernel, one grid row per group (32 weight columns per workgroup).
+template <typename OUT>
+static int launch_grouped_lines(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, const uint8_t* b, const float* b_s,
+                                OUT* c, const uint16_t* bias, const int64_t* m_splits, int G, int max_rows, int N, int K,
+                                hipStream_t stream) {
+    GroupRows rows;
+    int row = 0;
+    for (int g = 0; g < G; ++g) {
+        rows.row_start[g] = row;
+        row += (int)m_splits[g];
+    }
+    for (int g = G; g <= kMaxGroups; ++g) rows.row_start[g] = row;
+    const int per = (K / 128 + kSmWaves - 1) / kSmWaves, cap = max_rows <= 16 ? 8 : max_rows <= 32 ? 4 : 2;
+    int uf = per;
+    if (per > cap) {
+        uf = cap;
+        for (int d = cap; d > cap / 2; --d)
+            if (per % d == 0) { uf = d; break; }
+    }
+    dim3 grid((unsigned)((N + 31) / 32), (unsigned)G), block(kSmWaves * 64);
+#define MDY_GL(MT, UF)                                                                                                             \
+    hipLaunchKernelGGL((fp8_grouped_lines_kernel<MT, 2, UF, OUT>), grid, block, 0, stream, a, a_s, as_rs, as_cs, b, b_s, c, bias, N, K, rows)
+    if (max_rows <= 16) {
+        if (uf <= 1) MDY_GL(1, 1);
+        else if (uf <= 2) MDY_GL(1, 2);
+        else if (uf <= 4) MDY_GL(1, 4);
+        else if (uf <= 7) MDY_GL(1, 7);
+        else MDY_GL(1, 8);
+    } else if (max_rows <= 32) {
+        if (uf <= 1) MDY_GL(2, 1);
+        else if (uf <= 2) MDY_GL(2, 2);
+        else MDY_GL(2, 4);
+    } else {
+        if (uf <= 1) MDY_GL(4, 1);
+        else MDY_GL(4, 2);
+    }
+#undef MDY_GL
+    return (int)hipGetLastError();
+}
+
 template <typename OUT>
 static int dispatch_grouped(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t as_cs, const uint8_t* b,
                             const float* b_s, OUT* c, const uint16_t* bias, const int64_t* m_splits, int G, int64_t M,
@@ -1299,7 +1367,15 @@ static int dispatch_grouped(const uint8_t* a, const float* a_s, int64_t as_rs, i
     if (tiled_ok) {
         int64_t max_rows = 0;
         for (int g = 0; g < G; ++g) max_rows = m_splits[g] > max_rows ? m_splits[g] : max_rows;
-        if (strip_pays(max_rows, (int64_t)G * ((N + 127) / 128)))
+        // few rows per group (routed experts at decode): the whole-line small-M kernel up to 24 rows, and up to 64 when
+        // there are too few strips for the strip kernel (per call in a replayed graph, old -> new: 32 groups x 16 rows,
+        // N=4096, K=7168 191 -> 173 us = 5.4 TB/s of weights; 64 x 2 rows 322 -> 276 us = 6.8 TB/s; 8 x 4 rows, N=2048 43 -> 21 us;
+        // 4 x 16 rows, N=2048 42 -> 13 us; 16 x 24 rows, N=1536, K=4096 28.7 -> 26.2 us; but 32 x 40 rows 215 us on strips,
+        // 288 us here, 32 x 64 rows 225 against 324 us)
+        const bool strips = strip_pays(max_rows, (int64_t)G * ((N + 127) / 128));
+        if (max_rows <= 24 || (max_rows <= 64 && !strips))
+            return launch_grouped_lines<OUT>(a, a_s, as_rs, as_cs, b, b_s, c, bias, m_splits, G, (int)max_rows, N, K, stream);
+        if (strips)
             return launch_strip<OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, m_splits, G, (int)max_rows, N, K,
                                      stream);
         return launch_grouped<OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, m_splits, G, N, K, stream);

@@ -84,12 +84,27 @@ def test_grouped_gemm_exact_integer(m_splits, N, K):
 
 
 @pytest.mark.parametrize("m_splits,N,K", [([1, 64, 0, 17, 33, 48, 16, 5], 3300, 896),    # ragged rows and columns, K tail step
-                                          ([16] * 40, 640, 128),                          # one K block
+                                          ([40] * 40, 640, 128),                          # one K block
                                           ([64] * 4, 6400, 1152)])
 def test_grouped_gemm_exact_integer_strip_kernel(m_splits, N, K):
-    """<= 64 rows per group and >= 200 strips of 128 columns: the weight-streaming strip kernel runs."""
-    assert max(m_splits) <= 64 and len(m_splits) * ((N + 127) // 128) >= 200
+    """25..64 rows in the largest group and >= 200 strips of 128 columns: the weight-streaming strip kernel runs."""
+    assert 24 < max(m_splits) <= 64 and len(m_splits) * ((N + 127) // 128) >= 200
     exact_grouped_case(m_splits, N, K, 3 * sum(m_splits) + N + K, call_f32)
+
+
+@pytest.mark.parametrize("m_splits,N,K", [([1, 16, 0, 7, 3, 24, 9, 2], 3300, 896),        # one or two row tiles, ragged N, 7 K blocks
+                                          ([16] * 40, 640, 128),                          # one K block: 7 of 8 waves idle
+                                          ([2] * 64, 1030, 7168),                         # routed experts at decode, 7 K blocks per wave
+                                          ([33, 64, 0, 40], 2050, 1152),                  # up to 64 rows, too few strips for the strip kernel
+                                          ([30, 17, 32], 1000, 2176),                     # 17 K blocks: uneven shares of the waves
+                                          ([5, 0, 0, 11], 290, 9344),                     # several passes over K
+                                          ([12] * 3, 515, 3072), ([20, 4], 777, 5120)])   # pass depths that round up (3 -> 4, 5 -> 7 blocks)
+def test_grouped_gemm_exact_integer_whole_line_kernel(m_splits, N, K):
+    """At most 24 rows in the largest group, or at most 64 with fewer than 200 strips: every group is a small-M GEMM of
+    the whole-line kernel (one grid row per group, empty groups return at once)."""
+    strips = len(m_splits) * ((N + 127) // 128)
+    assert max(m_splits) <= 24 or (max(m_splits) <= 64 and strips < 200)
+    exact_grouped_case(m_splits, N, K, 5 * sum(m_splits) + N + K, call_f32)
 
 
 def test_dense_wide_weight_exact_integer_strip_kernel():
@@ -121,7 +136,7 @@ def test_grouped_matmul_against_oracle_with_bias_and_column_major_scales():
     ref = O.fp8_grouped_matmul(ra[:M], rsa[:M], rb, rsb, m_splits)
     assert out.dtype == torch.bfloat16 and out.shape == (M, N)
     assert torch.allclose(out.float().cpu(), ref.float(), rtol=RTOL, atol=ATOL)
-    # decode-like split of the same rows (strip kernel): 8 experts would not fill it, 64 small ones do
+    # decode-like split of the same rows (64 groups of 16: the whole-line small-M kernel, one grid row per group)
     small = [16] * 64
     Ms = sum(small)
     qb64, sb64 = qb.repeat(11, 1, 1)[:64].contiguous(), sb.repeat(11, 1, 1)[:64].contiguous()
