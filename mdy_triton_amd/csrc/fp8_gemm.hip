@@ -575,11 +575,12 @@ __global__ __launch_bounds__(512) void fp8_gemv_kernel(const uint8_t* __restrict
 // ---------------------------------------------------------------------------
 // Strip kernel: few rows (<= 16*MT <= 64 per group) against a weight that is wide enough to give every CU
 // work without splitting K (many column strips: a vocabulary-sized N, or many experts).  One workgroup = 8
-// waves = 128 weight columns of one group, wave w streams rows n0+16w .. +15 of the weight straight from
-// global memory into MFMA fragments (each row is read once, 512 contiguous bytes per row and step), while
-// the activation rows of the step (<= 64 rows x 512 bytes) and their scales are copied into LDS ONCE per
-// workgroup and shared by the 8 waves - in the kernel above every 16 columns re-read them, which is what
-// bounds it as soon as there are 16 or more rows.  grid = (ceil(N/128), groups).
+// waves = 128 weight columns of one group, wave w streams rows n0+16w .. +15 of the weight (each row is read
+// once, in whole 128-byte lines: 8 rows x one K block per instruction, turned into MFMA fragments through a
+// 2 KB tile of LDS that only this wave touches, as in the whole-line small-M kernel; the loads of step s+1
+// are issued before the wait for step s), while the activation rows of the step (<= 64 rows x 512 bytes) and
+// their scales are copied into LDS ONCE per workgroup and shared by the 8 waves - in the small-M kernels every
+// 16 or 32 columns re-read them.  grid = (ceil(N/128), groups).
 // ---------------------------------------------------------------------------
 constexpr int kStripKC = 4;   // K blocks per step
 
@@ -593,6 +594,7 @@ __global__ __launch_bounds__(512) void fp8_gemm_strip_kernel(
     __shared__ __attribute__((aligned(256))) float lds_sa[2][KC][64];
     __shared__ __attribute__((aligned(256))) float lds_bs[512];
     __shared__ __attribute__((aligned(256))) uint8_t lds_dummy[8 * 1024];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_bt[8][2048];      // a wave's weight tile on its way to fragments
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -628,18 +630,26 @@ __global__ __launch_bounds__(512) void fp8_gemm_strip_kernel(
         dma4(rs, s_voff, min(step * KC + wave, KB - 1) * as_cs * 4, ls0 + buf * ls_buf);
     };
 
-    // ---- weight fragments straight from global memory: lane -> row lane%16, 32-byte K slice lane/16
+    // ---- weight rows in whole lines: lane l loads piece l & 7 of row 8 t + (l >> 3), t = 0, 1, of every K block
     const int frow = lane & 15, fk = lane >> 4;
-    const uint8_t* bp = bg + (size_t)min(n0 + wave * 16 + frow, N - 1) * K + fk * 32;
-    uint4 blo[KC], bhi[KC];
-    auto load_b = [&](int step) {
+    const int r8 = lane >> 3, pc = lane & 7;
+    const uint8_t* bld0 = bg + (size_t)min(n0 + wave * 16 + r8, N - 1) * K + pc * 16;
+    const uint8_t* bld1 = bg + (size_t)min(n0 + wave * 16 + 8 + r8, N - 1) * K + pc * 16;
+    // Two register sets, filled by loads the compiler does not count (like the copies into LDS): the waits are the
+    // explicit vmcnt below, so the loads of step s+1 stay in flight across the wait for step s.
+    intx4 bset0[KC][2], bset1[KC][2];
+    auto load_b = [&](int step, intx4 (&v)[KC][2]) {
 #pragma unroll
         for (int kc = 0; kc < KC; ++kc) {
             const int kb = min(step * KC + kc, KB - 1);      // the clamped duplicates are never used
-            blo[kc] = load_nt16(bp + (size_t)kb * 128);
-            bhi[kc] = load_nt16(bp + (size_t)kb * 128 + 16);
+            asm volatile("global_load_dwordx4 %0, %1, off nt" : "=&v"(v[kc][0]) : "v"(bld0 + (size_t)kb * 128) : "memory");
+            asm volatile("global_load_dwordx4 %0, %1, off nt" : "=&v"(v[kc][1]) : "v"(bld1 + (size_t)kb * 128) : "memory");
         }
     };
+    // the wave's LDS tile: piece p of row r at r * 128 + ((p ^ (r & 7)) * 16)
+    uint8_t* bt = lds_bt[wave];
+    const int bt_wr = r8 * 128 + ((pc ^ r8) << 4);
+    const int bt_lo = frow * 128 + (((2 * fk) ^ (frow & 7)) << 4), bt_hi = frow * 128 + (((2 * fk + 1) ^ (frow & 7)) << 4);
     const int a_rd0 = frow * 128 + (((2 * fk) ^ swz(frow)) << 4);
     const int a_rd1 = frow * 128 + (((2 * fk + 1) ^ swz(frow)) << 4);
 
@@ -651,20 +661,29 @@ __global__ __launch_bounds__(512) void fp8_gemm_strip_kernel(
         const intx4 rbs = make_rsrc(b_s + ((size_t)g * NB + min(n0 >> 7, NB - 1)) * KB, (uint32_t)KB * 4u);
         for (int cc = 0; cc < KB; cc += 64) dma4(rbs, lane * 4, cc * 4, lds_addr(&lds_bs[cc]));
     }
-    copy_step(0, 0);
-    for (int step = 0; step < steps; ++step) {
+    auto run_step = [&](int step, intx4 (&cur)[KC][2], intx4 (&nxt)[KC][2]) {
         const int buf = step & 1;
-        load_b(step);                                   // this step's weight rows: the long-latency part
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();                                // the step's activation rows are in LDS; buffer buf^1 is free
+        // the next step's weight rows, then wait for all but those: this step's weights and copies.  No load whose
+        // registers are never read is issued: the compiler would hand such registers to other values while the load is
+        // still on its way.
+        if (step + 1 < steps) {
+            load_b(step + 1, nxt);
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * KC) : "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        __builtin_amdgcn_s_barrier();                   // the step's activation rows are in LDS; buffer buf^1 is free
+        asm volatile("" ::: "memory");
         if (step + 1 < steps) copy_step(step + 1, buf ^ 1);
 #pragma unroll
         for (int kc = 0; kc < KC; ++kc) {
             const int kb = step * KC + kc;
             if (kb < KB) {
                 const float sb = lds_bs[kb];
-                const intx8 fb = intx8{(int)blo[kc].x, (int)blo[kc].y, (int)blo[kc].z, (int)blo[kc].w,
-                                       (int)bhi[kc].x, (int)bhi[kc].y, (int)bhi[kc].z, (int)bhi[kc].w};
+                *reinterpret_cast<intx4*>(bt + bt_wr) = cur[kc][0];
+                *reinterpret_cast<intx4*>(bt + 1024 + bt_wr) = cur[kc][1];
+                const intx4 wlo = *reinterpret_cast<const intx4*>(bt + bt_lo), whi = *reinterpret_cast<const intx4*>(bt + bt_hi);
+                const intx8 fb = intx8{wlo[0], wlo[1], wlo[2], wlo[3], whi[0], whi[1], whi[2], whi[3]};
 #pragma unroll
                 for (int i = 0; i < MT; ++i) {
                     const uint8_t* la = &lds_a[buf][kc][i * 2048];
@@ -677,7 +696,15 @@ __global__ __launch_bounds__(512) void fp8_gemm_strip_kernel(
                 }
             }
         }
+    };
+    copy_step(0, 0);
+    load_b(0, bset0);
+    int step = 0;
+    for (; step + 1 < steps; step += 2) {      // unrolled by two: the register sets swap without moves
+        run_step(step, bset0, bset1);
+        run_step(step + 1, bset1, bset0);
     }
+    if (step < steps) run_step(step, bset0, bset1);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
     const bool vec_ok = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
