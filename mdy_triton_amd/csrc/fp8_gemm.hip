@@ -892,19 +892,18 @@ static int launch_strip(const uint8_t* a, const float* a_s, int64_t as_rs, int64
 // 5.4 against 3.8; M=1 N=4096 K=4096 5.0 against 4.4; but M=1 N=2048 K=7168 4.0 against 5.0, N=18432 24.5 against 26.6).
 static bool gemv_pays(int64_t M, int64_t K) { return M == 1 && K > 4096 && K <= kGemvMaxK; }
 
-// few rows per group and enough 128-column strips to fill the CUs without splitting K (with a handful of rows the
-// 16-column kernel re-reads so little of a that it stays ahead)
-// The whole-line small-M kernel (5 or more rows; K % 128 == 0, 16-byte aligned operands: the caller checks): up to 24
-// rows always, up to 32 unless the weight is very wide, up to 64 for a middling N.  Measured per call in a replayed graph,
-// K=7168 unless noted: M=32 N=16384 31.3 us there, 34.9 us on 128x128 tiles; N=18432 42.0 against 34.8 us; M=32 N=129280
-// 240 against 206 us on strips; M=16 N=129280 161 against 182 us on strips; M=24 N=25600 K=4096 28.3 against 34.6 us;
-// M=64 N=7168 K=2048 6.6 against 8.7 us on 64x64 tiles, N=12800 K=2048 11.7 against 8.9 us, N=4096 17.1 against 24.8 us on
-// the fragment-loading kernel, N=2048 16.2 against 15.5 us.
+// The whole-line small-M kernel (K % 128 == 0, 16-byte aligned operands: the caller checks): up to 16 rows always, up to
+// 24 unless there are 200 strips of 128 columns (then the strip kernel), up to 32 unless the weight is very wide, up to 64
+// for a middling N.  Measured per call in a replayed graph, K=7168 unless noted: M=32 N=16384 31.3 us here, 34.9 us on
+// 128x128 tiles; N=18432 42.0 against 34.8 us; M=16 N=129280 165 against 184 us on strips; M=8 N=32768 42.5 against 59 us;
+// M=24 N=32768 K=2048 19.1 against 17.4 us on strips; M=64 N=7168 K=2048 6.6 against 8.7 us on 64x64 tiles, N=12800 K=2048
+// 11.7 against 8.9 us, N=4096 17.1 against 24.8 us on the fragment-loading kernel, N=2048 16.2 against 15.5 us.
 static bool lines_pays(int64_t M, int64_t N) {
     const int64_t strips = (N + 127) / 128;
-    return (M <= 24 || (M <= 32 && strips < 136) || (M <= 64 && N >= 3200 && strips < 100));
+    return (M <= 16 || (M <= 24 && strips < 200) || (M <= 32 && strips < 136) || (M <= 64 && N >= 3200 && strips < 100));
 }
 
+// the strip kernel: few rows (per group) and enough 128-column strips to fill the CUs without splitting K
 static bool strip_pays(int64_t max_rows, int64_t strips) { return max_rows > 4 && max_rows <= 64 && strips >= 200; }
 
 // Up to 64 rows (K % 128 == 0, aligned operands: the caller checks; big_ok: the scales also fit the tile kernels'
@@ -1394,13 +1393,13 @@ static int dispatch_grouped(const uint8_t* a, const float* a_s, int64_t as_rs, i
     if (tiled_ok) {
         int64_t max_rows = 0;
         for (int g = 0; g < G; ++g) max_rows = m_splits[g] > max_rows ? m_splits[g] : max_rows;
-        // few rows per group (routed experts at decode): the whole-line small-M kernel up to 24 rows, and up to 64 when
-        // there are too few strips for the strip kernel (per call in a replayed graph, old -> new: 32 groups x 16 rows,
-        // N=4096, K=7168 191 -> 173 us = 5.4 TB/s of weights; 64 x 2 rows 322 -> 276 us = 6.8 TB/s; 8 x 4 rows, N=2048 43 -> 21 us;
-        // 4 x 16 rows, N=2048 42 -> 13 us; 16 x 24 rows, N=1536, K=4096 28.7 -> 26.2 us; but 32 x 40 rows 215 us on strips,
-        // 288 us here, 32 x 64 rows 225 against 324 us)
+        // few rows per group (routed experts at decode): the whole-line small-M kernel up to 16 rows, and up to 64 when
+        // there are too few strips for the strip kernel (per call in a replayed graph, strip or tile kernel -> here:
+        // 32 groups x 16 rows, N=4096, K=7168 191 -> 176 us = 5.3 TB/s of weights; 64 x 2 rows 323 -> 279 us = 6.7 TB/s;
+        // 8 x 4 rows, N=2048 43 -> 21 us; 4 x 16 rows, N=2048 42 -> 13 us; 16 x 24 rows, N=1536, K=4096 28.7 -> 26.5 us; but
+        // 32 x 24 rows 201 us on strips, 230 us here; 32 x 40 rows 168 against 288 us; 32 x 64 rows 200 against 324 us)
         const bool strips = strip_pays(max_rows, (int64_t)G * ((N + 127) / 128));
-        if (max_rows <= 24 || (max_rows <= 64 && !strips))
+        if (max_rows <= 16 || (max_rows <= 64 && !strips))
             return launch_grouped_lines<OUT>(a, a_s, as_rs, as_cs, b, b_s, c, bias, m_splits, G, (int)max_rows, N, K, stream);
         if (strips)
             return launch_strip<OUT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, m_splits, G, (int)max_rows, N, K,

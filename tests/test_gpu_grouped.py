@@ -85,14 +85,15 @@ def test_grouped_gemm_exact_integer(m_splits, N, K):
 
 @pytest.mark.parametrize("m_splits,N,K", [([1, 64, 0, 17, 33, 48, 16, 5], 3300, 896),    # ragged rows and columns, K tail step
                                           ([40] * 40, 640, 128),                          # one K block
+                                          ([24] * 9, 3000, 2560),                         # 5 steps of 4 K blocks: odd number of steps
                                           ([64] * 4, 6400, 1152)])
 def test_grouped_gemm_exact_integer_strip_kernel(m_splits, N, K):
-    """25..64 rows in the largest group and >= 200 strips of 128 columns: the weight-streaming strip kernel runs."""
-    assert 24 < max(m_splits) <= 64 and len(m_splits) * ((N + 127) // 128) >= 200
+    """17..64 rows in the largest group and >= 200 strips of 128 columns: the weight-streaming strip kernel runs."""
+    assert 16 < max(m_splits) <= 64 and len(m_splits) * ((N + 127) // 128) >= 200
     exact_grouped_case(m_splits, N, K, 3 * sum(m_splits) + N + K, call_f32)
 
 
-@pytest.mark.parametrize("m_splits,N,K", [([1, 16, 0, 7, 3, 24, 9, 2], 3300, 896),        # one or two row tiles, ragged N, 7 K blocks
+@pytest.mark.parametrize("m_splits,N,K", [([1, 16, 0, 7, 3, 24, 9, 2], 3001, 896),        # one or two row tiles, ragged N, 7 K blocks
                                           ([16] * 40, 640, 128),                          # one K block: 7 of 8 waves idle
                                           ([2] * 64, 1030, 7168),                         # routed experts at decode, 7 K blocks per wave
                                           ([33, 64, 0, 40], 2050, 1152),                  # up to 64 rows, too few strips for the strip kernel
@@ -100,10 +101,10 @@ def test_grouped_gemm_exact_integer_strip_kernel(m_splits, N, K):
                                           ([5, 0, 0, 11], 290, 9344),                     # several passes over K
                                           ([12] * 3, 515, 3072), ([20, 4], 777, 5120)])   # pass depths that round up (3 -> 4, 5 -> 7 blocks)
 def test_grouped_gemm_exact_integer_whole_line_kernel(m_splits, N, K):
-    """At most 24 rows in the largest group, or at most 64 with fewer than 200 strips: every group is a small-M GEMM of
+    """At most 16 rows in the largest group, or at most 64 with fewer than 200 strips: every group is a small-M GEMM of
     the whole-line kernel (one grid row per group, empty groups return at once)."""
     strips = len(m_splits) * ((N + 127) // 128)
-    assert max(m_splits) <= 24 or (max(m_splits) <= 64 and strips < 200)
+    assert max(m_splits) <= 16 or (max(m_splits) <= 64 and strips < 200)
     exact_grouped_case(m_splits, N, K, 5 * sum(m_splits) + N + K, call_f32)
 
 
