@@ -149,131 +149,13 @@ __global__ __launch_bounds__(512) void fp8_grouped_gemm_kernel(
         fp8_gemm_tile<256, 256, 2, 4, 2, OUT>(a, a_s, as_rs, as_cs, as_bytes, bg, bsg, c, biasg, m0, r1, m_total, n0, N, K, N, duty, 0, KB, pool);
 }
 
-// ---------------------------------------------------------------------------
-// Small-M kernel: M <= 16*MT rows (decode / routed-expert shapes).  Pure weight
-// streaming: one workgroup of 8 waves per 16 output columns; wave w takes K blocks
-// w, w+8, ... and keeps the loads of the next block in flight while the MFMAs of
-// the current one run; B fragments come straight from global memory (each row
-// slice of a K block is one full 128-byte line, read once, non-temporal), A
-// fragments too (A is tiny and L2 resident).  Partial sums are reduced through LDS.
-// ---------------------------------------------------------------------------
-constexpr int kSmWaves = 8;
-
-template <int MT, int NC, typename OUT, int FMT = 0>
-__global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_kernel(const uint8_t* __restrict__ a,
-                                                                          const float* __restrict__ a_s, int64_t as_rs,
-                                                                          int64_t as_cs, const uint8_t* __restrict__ b,
-                                                                          const float* __restrict__ b_s,
-                                                                          OUT* __restrict__ c,
-                                                                          const uint16_t* __restrict__ bias, int M,
-                                                                          int N, int K) {
-    // NC groups of 16 weight columns per workgroup: the activation fragments of a K block are loaded once per wave
-    // and used for all of them (with NC = 2 half as many workgroups re-read the activation rows)
-    static_assert(NC * MT <= kSmWaves, "one wave reduces one (column group, row sub-tile) pair");
-    __shared__ float red[kSmWaves][NC * MT][64][4];
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int frow = lane & 15, fk = lane >> 4;
-    const int n0 = blockIdx.x * (16 * NC);
-    const int KB = K >> 7, NB = (N + 127) >> 7;
-    const int m_base = blockIdx.y * (MT * 16);     // grid.y splits the rows when there are few column groups
-    const uint8_t* bp[NC];
-    const float* bsp[NC];
-#pragma unroll
-    for (int j = 0; j < NC; ++j) {
-        const int nrow = min(n0 + 16 * j + frow, N - 1);
-        bp[j] = b + (int64_t)nrow * K + fk * 32;
-        bsp[j] = b_s + (int64_t)min((n0 + 16 * j) >> 7, NB - 1) * KB;
-    }
-    const uint8_t* ap[MT];
-    const float* asp[MT];
-#pragma unroll
-    for (int i = 0; i < MT; ++i) {
-        const int m = min(m_base + i * 16 + frow, M - 1);
-        ap[i] = a + (int64_t)m * K + fk * 32;
-        asp[i] = a_s + (int64_t)m * as_rs;
-    }
-
-    floatx4 acc[NC][MT];
-#pragma unroll
-    for (int j = 0; j < NC; ++j)
-#pragma unroll
-        for (int i = 0; i < MT; ++i) acc[j][i] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-    // everything one K block needs: NC B fragments, MT A fragments, MT activation scales, NC weight scales
-    struct Operands {
-        uint4 blo[NC], bhi[NC];
-        intx4 alo[MT], ahi[MT];
-        float sa[MT];
-        float sb[NC];
-    };
-    auto load_block = [&](int kb, Operands& o) {
-#pragma unroll
-        for (int j = 0; j < NC; ++j) {
-            o.blo[j] = load_nt16(bp[j] + (int64_t)kb * 128);
-            o.bhi[j] = load_nt16(bp[j] + (int64_t)kb * 128 + 16);
-            o.sb[j] = bsp[j][kb];
-        }
-#pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            o.alo[i] = *reinterpret_cast<const intx4*>(ap[i] + (int64_t)kb * 128);
-            o.ahi[i] = *reinterpret_cast<const intx4*>(ap[i] + (int64_t)kb * 128 + 16);
-            o.sa[i] = asp[i][(int64_t)kb * as_cs];
-        }
-    };
-    Operands cur, nxt;
-    int kb = wave;
-    if (kb < KB) load_block(kb, cur);
-    for (; kb < KB; kb += kSmWaves) {
-        const bool more = kb + kSmWaves < KB;
-        if (more) load_block(kb + kSmWaves, nxt);   // in flight while this block's MFMAs run
-#pragma unroll
-        for (int j = 0; j < NC; ++j) {
-            const intx8 fb = intx8{(int)cur.blo[j].x, (int)cur.blo[j].y, (int)cur.blo[j].z, (int)cur.blo[j].w,
-                                   (int)cur.bhi[j].x, (int)cur.bhi[j].y, (int)cur.bhi[j].z, (int)cur.bhi[j].w};
-#pragma unroll
-            for (int i = 0; i < MT; ++i) {
-                const intx8 fa = intx8{cur.alo[i][0], cur.alo[i][1], cur.alo[i][2], cur.alo[i][3],
-                                       cur.ahi[i][0], cur.ahi[i][1], cur.ahi[i][2], cur.ahi[i][3]};
-                const float sc = cur.sa[i] * cur.sb[j];
-                const floatx4 p = mfma_block<FMT>(fb, fa);
-                fold(acc[j][i], p, sc);
-            }
-        }
-        if (more) cur = nxt;
-    }
-#pragma unroll
-    for (int j = 0; j < NC; ++j)
-#pragma unroll
-        for (int i = 0; i < MT; ++i)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) red[wave][j * MT + i][lane][e] = acc[j][i][e];
-    __syncthreads();
-    if (wave < NC * MT) {
-        // wave (j, i) reduces column group j, row sub-tile i (fixed order, so results do not depend on timing)
-        const int j = wave / MT, i = wave % MT;
-        const bool vec_ok = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
-        float v[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            float t = 0.0f;
-#pragma unroll
-            for (int w = 0; w < kSmWaves; ++w) t += red[w][wave][lane][e];
-            v[e] = t;
-        }
-        const int m = m_base + i * 16 + frow, n = n0 + 16 * j + 4 * fk;
-        if (bias != nullptr) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (n + e < N) v[e] += bf16_one(bias[n + e]);
-        }
-        store4<OUT>(c, N, m, n, M, N, v, vec_ok);
-    }
-}
+constexpr int kSmWaves = 8;      // waves per workgroup of the small-M kernels
 
 // ---------------------------------------------------------------------------
-// Small-M kernel with whole-line loads (up to 16*MT rows).  The kernel above loads MFMA fragments straight from global
-// memory: per instruction 16 rows x 4 pieces of 16 bytes, 64 of every 128-byte line, the line's other half by the
+// Small-M kernel with whole-line loads (up to 16*MT rows; decode and routed-expert shapes): pure weight streaming, one
+// workgroup of 8 waves per 16*NC output columns, the waves share out the K blocks and their partial sums are reduced
+// through LDS.  An MFMA operand wants lane (r, q) to hold 32 bytes of row r, so fragment loads straight from global
+// memory touch, per instruction, 16 rows x 4 pieces of 16 bytes: 64 of every 128-byte line, the line's other half by the
 // next instruction.  Measured on loads alone (M=16, N=2048, K=7168, replayed graph): 8.5 us per call that way, 3.4 us
 // when every load instruction covers whole lines (8 rows x the 128 bytes of one K block: lane l has piece l & 7 of
 // row l >> 3).  So here a wave loads its K blocks that way, UF blocks before the first use, and turns a block into
@@ -924,7 +806,13 @@ static int dispatch_small(const uint8_t* a, const float* a_s, int64_t as_rs, int
         const int64_t one = M;
         return launch_strip<OUT, FMT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, &one, 1, M, N, K, stream);
     }
-    if (lines) {
+    // 32..64 rows against a wide weight: the whole-line kernel re-reads the activation rows in every one of its N/16 or
+    // N/32 workgroups, and from 32 rows on that traffic costs more than the empty rows of an MFMA tile (see lines_pays).
+    if (!lines && M >= 32 && M <= 64 && big_ok && (N + 127) / 128 >= 128)
+        return launch_mfma<128, 128, 2, 2, 4, OUT, FMT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
+    if (!lines && M >= 32 && M <= 64 && big_ok && (N + 63) / 64 >= 100)
+        return launch_mfma<64, 64, 2, 2, 8, OUT, FMT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
+    {      // everything else, and what lines_pays prefers: the whole-line kernel
         // 32 columns per workgroup when that still leaves ~200 workgroups (loads alone, M=16: N=7168, K=2048 2.9 -> 2.5 us
         // per call; N=2048, K=7168 3.4 -> 4.1 us); the K blocks of a wave in passes of up to 8 (up to 16 rows) or 4
         const bool wide = (N + 31) / 32 >= 200;
@@ -974,39 +862,7 @@ static int dispatch_small(const uint8_t* a, const float* a_s, int64_t as_rs, int
 #undef MDY_LINES
         return (int)hipGetLastError();
     }
-    // 32..64 rows against a wide weight: the kernel below re-reads the activation rows in every one of its
-    // N/16 workgroups, and from 32 rows on that traffic costs more than the empty rows of an MFMA tile.
-    // Measured (M=64): N=18432, K=7168 121 -> 64 us with 128x128 tiles; N=7168, K=16384 110 -> 80 us with 64x64.
-    if (M >= 32 && M <= 64 && big_ok && (N + 127) / 128 >= 128)
-        return launch_mfma<128, 128, 2, 2, 4, OUT, FMT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
-    if (M >= 32 && M <= 64 && big_ok && (N + 63) / 64 >= 100)
-        return launch_mfma<64, 64, 2, 2, 8, OUT, FMT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
-    if (M <= 64) {
-        // one workgroup streams 16 weight columns against MT row sub-tiles; every workgroup re-reads its rows of
-        // a, so with few column groups (N small) the rows are split over grid.y as well: more workgroups, less
-        // traffic through each CU's L1
-        const int sub = (M + 15) / 16;
-        int mt = sub;
-        if ((N + 15) / 16 < 200 && sub >= 2) mt = (sub + 1) / 2;
-        // two column groups per workgroup when that still leaves enough workgroups: the activation rows are
-        // fetched by half as many of them (measured: pays from 17 rows on with 288 workgroups, from 5 rows on with
-        // 512; M=31, N=18432, K=7168: 70 -> 59 us)
-        const long wgs32 = (N + 31) / 32;
-        const bool two = mt <= 2 && ((M > 16 && wgs32 >= 288) || (M > 4 && wgs32 >= 512));
-        dim3 grid((unsigned)(two ? (N + 31) / 32 : (N + 15) / 16), (unsigned)((sub + mt - 1) / mt));
-#define MDY_SM(MT, NC)                                                                                             \
-    hipLaunchKernelGGL((fp8_gemm_smallm_kernel<MT, NC, OUT, FMT>), grid, dim3(kSmWaves * 64), 0, stream, a, a_s, as_rs, as_cs, b, \
-                       b_s, c, bias, M, N, K)
-        if (two && mt == 1) MDY_SM(1, 2);
-        else if (two) MDY_SM(2, 2);
-        else if (mt == 1) MDY_SM(1, 1);
-        else if (mt == 2) MDY_SM(2, 1);
-        else if (mt == 3) MDY_SM(3, 1);
-        else MDY_SM(4, 1);
-#undef MDY_SM
-        return (int)hipGetLastError();
-    }
-    return -1;   // not reached: M <= 64 ends in the weight-streaming kernel above
+    return -1;   // not reached: every M <= 64 ends in the whole-line kernel above
 }
 
 // The MFMA tile kernels for more than 64 rows (K % 128 == 0, aligned operands, scales within 2^31 bytes: the caller

@@ -429,19 +429,20 @@ def test_e5m2_tile_kernels_exact_integer(M, N, K):
 
 
 # (M, N, K) -> the branch of the <= 64-row dispatch it lands in
-E5M2_SMALL = [(1, 512, 256), (5, 512, 384), (16, 520, 256), (17, 512, 256), (33, 512, 256), (64, 512, 256),      # weight streaming, one column group, rows split over grid.y from 17 on
-              (48, 3600, 256), (64, 3200, 128),                                                                  # weight streaming, 3 and 4 row sub-tiles per workgroup
-              (5, 16384, 256), (17, 9216, 256), (31, 9216, 128),                                                   # two column groups per workgroup
-              (5, 25600, 256), (16, 25600, 128), (33, 25616, 256), (64, 25600, 128),                               # strip kernel
+E5M2_SMALL = [(1, 512, 256), (5, 512, 384), (16, 520, 256), (17, 512, 256), (33, 512, 256), (64, 512, 256),      # whole-line kernel: 1, 2 and 4 row tiles, 16 columns per workgroup
+              (48, 3600, 256), (64, 3200, 128), (48, 6400, 256), (64, 6404, 128),                                   # the same with 4 row tiles against a middling N
+              (5, 16384, 256), (17, 9216, 256), (31, 9216, 128), (5, 25600, 256), (16, 25600, 128),                # 32 columns per workgroup
+              (20, 25600, 256), (33, 25616, 256), (64, 25600, 128),                                                # strip kernel
               (48, 16384, 256), (33, 16400, 128),                                                                  # 128x128 tiles
-              (48, 6400, 256), (64, 6404, 128)]                                                                    # 64x64 tiles
+              (48, 12800, 256), (64, 12804, 128)]                                                                  # 64x64 tiles
 
 
 @pytest.mark.parametrize("M,N,K", E5M2_SMALL)
 def test_e5m2_small_m_exact_integer(M, N, K):
-    """e5m2 operands, up to 64 rows: every branch of the small-M dispatch (weight streaming with one and two column
-    groups, the strip kernel, 128x128 and 64x64 tiles against a wide weight), exact on integer operands with power-of-two
-    scales; fp32 and bf16 output, bias in the epilogue, through the C entry point and through fp8_matmul."""
+    """e5m2 operands, up to 64 rows: every branch of the small-M dispatch (the whole-line kernel with 16 and 32 columns per
+    workgroup and 1, 2 or 4 row tiles, the strip kernel, 128x128 and 64x64 tiles against a wide weight), exact on integer
+    operands with power-of-two scales; fp32 and bf16 output, bias in the epilogue, through the C entry point and through
+    fp8_matmul."""
     from mdy_triton_amd import _lib
     g = torch.Generator().manual_seed(7 * M + N + K)
     ai = torch.randint(-4, 5, (M, K), generator=g)
