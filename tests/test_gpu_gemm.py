@@ -472,6 +472,21 @@ def test_gemm_decode_shapes(M, N, K):
     assert (got.cpu().double() - truth).abs().max() <= 2 ** -8 * truth.abs().max() + 1e-6
 
 
+@pytest.mark.parametrize("M,N,K", [(5, 1536, 1536), (24, 2112, 7168), (32, 4096, 4096), (48, 3328, 2048),      # whole-line kernel: 1, 2, 4 row tiles
+                                   (8, 25728, 512),                                                             # 32 columns per workgroup, wide N
+                                   (40, 25600, 1024), (20, 25728, 640),                                         # strip kernel
+                                   (9, 300, 9344)])                                                             # several passes over K
+def test_gemm_small_m_kernels_against_oracle(M, N, K):
+    """The small-M kernels on quantized Gaussian activations and weights (not only exact-integer operands): within the
+    GEMM tolerance of the oracle's dequantize + fp32 matmul, and within 2^-8 of the float64 result's scale."""
+    a, a_s, wq, ws = quantized_problem("normal", M, N, K, seed=M + N + K)
+    ref = O.fp8_gemm(a, a_s, wq, ws, dtype=torch.bfloat16)
+    got = m.fp8_gemm(a.to(DEV), a_s.to(DEV), wq.to(DEV), ws.to(DEV), out_dtype=torch.bfloat16)
+    assert close(got, ref)
+    truth = O.fp8_gemm_f64(a, a_s, wq, ws)
+    assert (got.cpu().double() - truth).abs().max() <= 2 ** -8 * truth.abs().max() + 1e-6
+
+
 def test_gemm_scalar_fallback_warns_for_large_aligned_shapes():
     """K > 65536 with more than 64 rows runs on the one-thread-per-output kernel: correct, but the wrapper says so
     (once per shape); K % 128 != 0, the kernel's intended use, stays silent."""
