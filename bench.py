@@ -596,6 +596,8 @@ def load_probe_lib():
     L.mdy_probe_copy_wd.argtypes = [p, p, p, i64, i64, p]
     L.mdy_probe_mfma_loop.argtypes = [i, p, p, i, i, p]
     L.mdy_probe_empty.argtypes = [p]
+    L.mdy_probe_load_pattern.argtypes = [i, p, p, p, i64, i64, p]
+    L.mdy_probe_load_pattern.restype = i
     for f in (L.mdy_fp8_gemm_probe, L.mdy_probe_copy_aq, L.mdy_probe_copy_wd, L.mdy_probe_mfma_loop, L.mdy_probe_empty):
         f.restype = i
     return L
@@ -706,6 +708,20 @@ def ceilings(torch, m, timer, dev):
             smi = smi or {}
             print("  %-58s %-30s %8.1f us  %6.2f PFLOP/s (%4.1f %% of 5.0)  %6s W  %5s MHz" % (
                 label, sname, us, flop / us / 1e9, flop / us / 1e9 / 5.0 * 100, smi.get("socket_power_w"), smi.get("gfx_clock_mhz")), flush=True)
+
+    print("== operand loads of a small-M GEMM alone (16 weight rows + 16 re-read activation rows per workgroup of 8 waves, every load "
+          "of a wave up front): per call inside a replayed HIP graph of 20 calls")
+    act = torch.randint(0, 255, (16, 8192), dtype=torch.uint8, device=dev)
+    sink = torch.zeros(1 << 16, dtype=torch.int32, device=dev)
+    for (N, K) in ((2048, 7168), (7168, 2048)):
+        wbytes = torch.randint(0, 255, (N, K), dtype=torch.uint8, device=dev)
+        row = []
+        for pat, label in ((0, "MFMA fragments from memory (16 lines x 64 B per instruction)"), (1, "whole lines (8 rows x 128 B)"),
+                           (2, "whole rows (1 KB per instruction)")):
+            us = graph_replay_us(torch, lambda pat=pat: ok(L.mdy_probe_load_pattern(pat, wbytes.data_ptr(), act.data_ptr(), sink.data_ptr(),
+                                                                                    N, K, stream_ptr(dev)), "load_pattern"))
+            row.append("%s %5.2f us" % (label, us))
+        print("  N=%d K=%d (%d workgroups): %s" % (N, K, N // 16, " | ".join(row)), flush=True)
 
     print("== launch floor: per call inside a replayed HIP graph of 20 calls")
     e_us = graph_replay_us(torch, lambda: ok(L.mdy_probe_empty(stream_ptr(dev)), "empty"))

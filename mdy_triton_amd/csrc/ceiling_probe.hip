@@ -9,6 +9,8 @@
 //   mfma_loop    a register-resident loop of v_mfma_f32_16x16x128_f8f6f4 only (8 + 4 operand fragments per wave, 32 MFMAs
 //                per iteration, no memory access): accumulating in place, or starting from zero and folded into an fp32
 //                accumulator with 4 v_fma_f32 per MFMA as the block-scaled GEMM has to
+//   load_pattern the operand loads of a small-M GEMM (16 weight rows and 16 activation rows per workgroup) as MFMA fragments
+//                straight from memory, as whole 128-byte lines, and as whole rows
 //   empty        a kernel that does nothing (the launch floor inside a replayed graph)
 #include <cstdint>
 
@@ -184,6 +186,59 @@ __global__ __launch_bounds__(512) void mfma32_loop_kernel(const uint32_t* __rest
     out[blockIdx.x * 512 + threadIdx.x] = r;
 }
 
+// Load patterns of a small-M GEMM's operands with the arithmetic taken out: a workgroup of 8 waves owns 16 weight rows
+// (b: [N, K] bytes) and re-reads 16 activation rows (a: [16, K] bytes); wave w takes the K blocks w, w + 8, .. and issues
+// all of its loads (up to 8 K blocks) before it folds them into one word that is never stored.
+//   PATTERN 0  MFMA fragments straight from memory: lane (r, q) = (lane % 16, lane / 16) loads the two 16-byte halves of
+//              bytes [32 q, 32 q + 32) of row r's K block - per instruction 16 lines, 64 bytes of each
+//   PATTERN 1  whole lines: lane l loads piece l % 8 of row l / 8 (and of row 8 + l / 8) of the K block - per instruction 8
+//              lines, all 128 bytes of each
+//   PATTERN 2  whole rows: wave w reads weight rows 2 w, 2 w + 1 and activation rows 2 w, 2 w + 1 end to end, 1 KB per
+//              instruction (K <= 8192)
+template <int PATTERN>
+__global__ __launch_bounds__(512) void load_pattern_kernel(const uint8_t* __restrict__ b, const uint8_t* __restrict__ a,
+                                                            uint32_t* __restrict__ out, int N, int K) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n0 = blockIdx.x * 16, KB = K >> 7;
+    uint4 v[8][4];
+    uint32_t x = 0;
+    if (PATTERN == 2) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (i * 1024 + lane * 16 < K) {
+                v[i][0] = *reinterpret_cast<const uint4*>(b + (size_t)(n0 + 2 * wave) * K + i * 1024 + lane * 16);
+                v[i][1] = *reinterpret_cast<const uint4*>(b + (size_t)(n0 + 2 * wave + 1) * K + i * 1024 + lane * 16);
+                v[i][2] = *reinterpret_cast<const uint4*>(a + (size_t)(2 * wave) * K + i * 1024 + lane * 16);
+                v[i][3] = *reinterpret_cast<const uint4*>(a + (size_t)(2 * wave + 1) * K + i * 1024 + lane * 16);
+            }
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (i * 1024 + lane * 16 < K)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) x ^= v[i][t].x ^ v[i][t].y ^ v[i][t].z ^ v[i][t].w;
+    } else {
+        const int row = PATTERN == 0 ? (lane & 15) : (lane >> 3);
+        const int o0 = PATTERN == 0 ? (lane >> 4) * 32 : (lane & 7) * 16;
+        const int second_row = PATTERN == 0 ? 0 : 8, second_off = PATTERN == 0 ? 16 : 0;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int kb = wave + 8 * u;
+            if (kb < KB) {
+                v[u][0] = *reinterpret_cast<const uint4*>(b + (size_t)(n0 + row) * K + kb * 128 + o0);
+                v[u][1] = *reinterpret_cast<const uint4*>(b + (size_t)(n0 + row + second_row) * K + kb * 128 + o0 + second_off);
+                v[u][2] = *reinterpret_cast<const uint4*>(a + (size_t)row * K + kb * 128 + o0);
+                v[u][3] = *reinterpret_cast<const uint4*>(a + (size_t)(row + second_row) * K + kb * 128 + o0 + second_off);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (wave + 8 * u < KB)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) x ^= v[u][t].x ^ v[u][t].y ^ v[u][t].z ^ v[u][t].w;
+    }
+    if (x == 0x12345678u) out[blockIdx.x] = x;      // keeps the loads; practically never taken
+}
+
 __global__ void empty_kernel() {}
 
 }  // namespace mdy
@@ -223,6 +278,20 @@ extern "C" int mdy_probe_mfma_loop(int fold, const void* seed, float* out, int w
     else
         hipLaunchKernelGGL(mdy::mfma_loop_kernel<false>, dim3((unsigned)workgroups), dim3(512), 0, static_cast<hipStream_t>(stream),
                            static_cast<const uint32_t*>(seed), out, iters, 1.0f);
+    return (int)hipGetLastError();
+}
+
+// b: N x K bytes, a: 16 x K bytes, out: N / 16 words; N % 16 == 0, K % 128 == 0, K <= 8192; pattern 0, 1 or 2
+extern "C" int mdy_probe_load_pattern(int pattern, const void* b, const void* a, void* out, int64_t N, int64_t K, void* stream) {
+    if (!b || !a || !out || N < 16 || N % 16 != 0 || K < 128 || K % 128 != 0 || K > 8192 || pattern < 0 || pattern > 2) return -2;
+    dim3 grid((unsigned)(N / 16)), block(512);
+    const uint8_t* bp = static_cast<const uint8_t*>(b);
+    const uint8_t* ap = static_cast<const uint8_t*>(a);
+    uint32_t* op = static_cast<uint32_t*>(out);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (pattern == 0) hipLaunchKernelGGL(mdy::load_pattern_kernel<0>, grid, block, 0, st, bp, ap, op, (int)N, (int)K);
+    else if (pattern == 1) hipLaunchKernelGGL(mdy::load_pattern_kernel<1>, grid, block, 0, st, bp, ap, op, (int)N, (int)K);
+    else hipLaunchKernelGGL(mdy::load_pattern_kernel<2>, grid, block, 0, st, bp, ap, op, (int)N, (int)K);
     return (int)hipGetLastError();
 }
 
