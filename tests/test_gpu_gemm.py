@@ -328,6 +328,13 @@ def test_gemm_row_vector_kernel_exact_integer(M, N, K, fmt):
     _small_m_exact_through_c_abi(M, N, K, fmt, longer_k=(fmt == "e4m3fn"))
 
 
+def test_gemm_whole_line_kernel_long_k_exact_integer():
+    """Up to 64 rows against K > 65536 (beyond the tile kernels' 32-bit addressing): the whole-line kernel takes it in
+    many passes; exact on integer operands."""
+    test_gemm_exact_integer_cases_all_kernels(8, 48, 65536 + 512)
+    test_gemm_exact_integer_cases_all_kernels(40, 80, 65536 + 128)
+
+
 @pytest.mark.parametrize("fmt", ["e4m3fn", "e5m2"])
 @pytest.mark.parametrize("M,N,K", [(16, 2048, 7168), (16, 7168, 2048), (5, 272, 128), (8, 1000, 1024), (9, 6401, 3072),
                                    (12, 1536, 1536), (16, 530, 4096), (13, 6500, 5120), (7, 333, 6144), (16, 4096, 8192),
