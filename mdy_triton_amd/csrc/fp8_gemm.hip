@@ -165,7 +165,7 @@ constexpr int kSmWaves = 8;      // waves per workgroup of the small-M kernels
 // [w per, (w+1) per), per = ceil(KB / 8): no branch depends on the block, so the waits the compiler places count
 // exactly; a block beyond the wave's range is a re-read of the last valid one whose product is replaced by zero.
 // ---------------------------------------------------------------------------
-template <int MT, int NC, int UF, typename OUT, int FMT>
+template <int MT, int NC, int UF, typename OUT, int FMT, bool HALF = false>
 __device__ __forceinline__ void smallm_lines_body(const uint8_t* __restrict__ a, const float* __restrict__ a_s, int64_t as_rs, int64_t as_cs,
                                                   const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
                                                   const uint16_t* __restrict__ bias, int M, int N, int K) {
@@ -179,15 +179,19 @@ __device__ __forceinline__ void smallm_lines_body(const uint8_t* __restrict__ a,
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int frow = lane & 15, fk = lane >> 4;
     const int r8 = lane >> 3, pc = lane & 7;
-    const int n0 = blockIdx.x * (16 * NC);
+    // HALF: 8 weight columns per workgroup (the other half of the MFMA's 16 rows stays unused): twice the workgroups for a
+    // narrow weight
+    static_assert(!HALF || NC == 1, "half a column group per workgroup: one group");
+    constexpr int BT = HALF ? 1 : 2 * NC;              // 8-row weight loads per K block
+    const int n0 = blockIdx.x * (HALF ? 8 : 16 * NC);
     const int KB = K >> 7, NB = (N + 127) >> 7;
     const int per = (KB + kSmWaves - 1) / kSmWaves;
     const int k_begin = min(wave * per, KB), k_end = min(k_begin + per, KB);      // this wave's K blocks
     // global: lane l loads piece l & 7 of row 8 t + (l >> 3) for t = 0, 1 of every 16-row tile
-    const uint8_t* bld[2 * NC];
+    const uint8_t* bld[BT];
     const uint8_t* ald[2 * MT];
 #pragma unroll
-    for (int t = 0; t < 2 * NC; ++t) bld[t] = b + (int64_t)min(n0 + 8 * t + r8, N - 1) * K + pc * 16;
+    for (int t = 0; t < BT; ++t) bld[t] = b + (int64_t)min(n0 + 8 * t + r8, N - 1) * K + pc * 16;
 #pragma unroll
     for (int t = 0; t < 2 * MT; ++t) ald[t] = a + (int64_t)min(8 * t + r8, M - 1) * K + pc * 16;
     const float* bsp[NC];
@@ -207,13 +211,13 @@ __device__ __forceinline__ void smallm_lines_body(const uint8_t* __restrict__ a,
         for (int i = 0; i < MT; ++i) acc[j][i] = floatx4{0.f, 0.f, 0.f, 0.f};
 
     for (int kp = k_begin; kp < k_end; kp += UF) {      // uniform in the wave
-        intx4 vb[UF][2 * NC], va[UF][2 * MT];      // plain vectors: a struct type here ends up in scratch memory
+        intx4 vb[UF][BT], va[UF][2 * MT];      // plain vectors: a struct type here ends up in scratch memory
         float sb[UF][NC], sraw[SV][MT];
 #pragma unroll
         for (int u = 0; u < UF; ++u) {
             const int kb = min(kp + u, k_end - 1);
 #pragma unroll
-            for (int t = 0; t < 2 * NC; ++t) vb[u][t] = __builtin_nontemporal_load(reinterpret_cast<const intx4*>(bld[t] + (int64_t)kb * 128));
+            for (int t = 0; t < BT; ++t) vb[u][t] = __builtin_nontemporal_load(reinterpret_cast<const intx4*>(bld[t] + (int64_t)kb * 128));
 #pragma unroll
             for (int t = 0; t < 2 * MT; ++t) va[u][t] = *reinterpret_cast<const intx4*>(ald[t] + (int64_t)kb * 128);
 #pragma unroll
@@ -231,7 +235,7 @@ __device__ __forceinline__ void smallm_lines_body(const uint8_t* __restrict__ a,
         auto through_lds = [&](int u) {      // block u of the pass: registers -> this wave's LDS -> fragments
             uint8_t* buf = lds[wave][u % NBUF];
 #pragma unroll
-            for (int t = 0; t < 2 * NC; ++t) *reinterpret_cast<intx4*>(buf + t * 1024 + wr_off) = vb[u][t];
+            for (int t = 0; t < BT; ++t) *reinterpret_cast<intx4*>(buf + t * 1024 + wr_off) = vb[u][t];
 #pragma unroll
             for (int t = 0; t < 2 * MT; ++t) *reinterpret_cast<intx4*>(buf + (2 * NC + t) * 1024 + wr_off) = va[u][t];
 #pragma unroll
@@ -290,7 +294,7 @@ __device__ __forceinline__ void smallm_lines_body(const uint8_t* __restrict__ a,
             for (int e = 0; e < 4; ++e)
                 if (n + e < N) v[e] += bf16_one(bias[n + e]);
         }
-        store4<OUT>(c, N, m, n, M, N, v, vec_ok);
+        if (!HALF || fk < 2) store4<OUT>(c, N, m, n, M, N, v, vec_ok);      // HALF: columns 8 .. 15 of the tile belong to the next workgroup
     }
 }
 
@@ -300,6 +304,15 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_lines_kernel(co
                                                                                const float* __restrict__ b_s, OUT* __restrict__ c,
                                                                                const uint16_t* __restrict__ bias, int M, int N, int K) {
     smallm_lines_body<MT, NC, UF, OUT, FMT>(a, a_s, as_rs, as_cs, b, b_s, c, bias, M, N, K);
+}
+
+// up to 16 rows against a narrow weight: 8 columns per workgroup
+template <int UF, typename OUT, int FMT>
+__global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_lines_half_kernel(const uint8_t* __restrict__ a, const float* __restrict__ a_s,
+                                                                                    int64_t as_rs, int64_t as_cs, const uint8_t* __restrict__ b,
+                                                                                    const float* __restrict__ b_s, OUT* __restrict__ c,
+                                                                                    const uint16_t* __restrict__ bias, int M, int N, int K) {
+    smallm_lines_body<1, 1, UF, OUT, FMT, true>(a, a_s, as_rs, as_cs, b, b_s, c, bias, M, N, K);
 }
 
 // The same for a grouped GEMM whose groups have at most 16*MT rows each (routed experts at decode): blockIdx.y is the group,
@@ -842,7 +855,26 @@ static int dispatch_small(const uint8_t* a, const float* a_s, int64_t as_rs, int
         case 8: MDY_LINES(MT, NC, 8); break;          \
         default: MDY_LINES_UF4(MT, NC)                \
     }
-        if (M <= 16 && wide) {
+        // a narrow weight (fewer than 100 groups of 16 columns): 8 columns per workgroup, twice the workgroups (per call in
+        // a replayed graph: M=16 N=1584 K=4096 4.6 -> 3.8 us, M=16 N=1024 K=8192 7.2 -> 6.3, M=4 N=1536 K=7168 5.3 -> 4.8,
+        // M=16 N=576 K=7168 6.0 -> 5.8; N=2048 and wider: no gain)
+        if (M <= 16 && (N + 15) / 16 < 100) {
+            grid = dim3((unsigned)((N + 7) / 8));
+#define MDY_HALF(UF)                                                                                                                \
+    hipLaunchKernelGGL((fp8_gemm_smallm_lines_half_kernel<UF, OUT, FMT>), grid, dim3(kSmWaves * 64), 0, stream, a, a_s, as_rs, as_cs, b, \
+                       b_s, c, bias, M, N, K)
+            switch (uf) {
+                case 1: MDY_HALF(1); break;
+                case 2: MDY_HALF(2); break;
+                case 3: MDY_HALF(3); break;
+                case 4: MDY_HALF(4); break;
+                case 5: MDY_HALF(5); break;
+                case 6: MDY_HALF(6); break;
+                case 7: MDY_HALF(7); break;
+                default: MDY_HALF(8); break;
+            }
+#undef MDY_HALF
+        } else if (M <= 16 && wide) {
             MDY_LINES_UF8(1, 2)
         } else if (M <= 16) {
             MDY_LINES_UF8(1, 1)
