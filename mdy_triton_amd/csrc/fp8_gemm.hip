@@ -165,12 +165,15 @@ constexpr int kSmWaves = 8;      // waves per workgroup of the small-M kernels
 // [w per, (w+1) per), per = ceil(KB / 8): no branch depends on the block, so the waits the compiler places count
 // exactly; a block beyond the wave's range is a re-read of the last valid one whose product is replaced by zero.
 // ---------------------------------------------------------------------------
-template <int MT, int NC, int UF, typename OUT, int FMT, bool HALF = false>
+template <int MT, int NC, int UF, typename OUT, int FMT, bool HALF = false, int WK = kSmWaves>
 __device__ __forceinline__ void smallm_lines_body(const uint8_t* __restrict__ a, const float* __restrict__ a_s, int64_t as_rs, int64_t as_cs,
                                                   const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
                                                   const uint16_t* __restrict__ bias, int M, int N, int K) {
     constexpr int SUB = NC * MT, TILES = NC + MT;      // (column group, row sub-tile) pairs; 16-row operand tiles per K block
-    static_assert(SUB <= kSmWaves, "one wave reduces one (column group, row sub-tile) pair");
+    // WK waves share out the K blocks of one set of columns; with a short K (fewer blocks than waves) the 8 waves form
+    // 8 / WK such sets side by side instead of idling
+    constexpr int SETS = kSmWaves / WK;
+    static_assert(SUB <= WK && SETS * WK == kSmWaves, "one wave of a set reduces one (column group, row sub-tile) pair");
     constexpr int SV = (UF + 3) / 4;                    // activation-scale loads per row sub-tile and pass
     constexpr int NBUF = MT < 4 ? 2 : 1;               // LDS regions and fragment sets per wave (64 rows: no room for two)
     __shared__ __attribute__((aligned(16))) uint8_t lds[kSmWaves][NBUF][TILES * 2048];
@@ -183,10 +186,11 @@ __device__ __forceinline__ void smallm_lines_body(const uint8_t* __restrict__ a,
     // narrow weight
     static_assert(!HALF || NC == 1, "half a column group per workgroup: one group");
     constexpr int BT = HALF ? 1 : 2 * NC;              // 8-row weight loads per K block
-    const int n0 = blockIdx.x * (HALF ? 8 : 16 * NC);
+    const int set = wave / WK, wk = wave % WK;
+    const int n0 = (blockIdx.x * SETS + set) * (HALF ? 8 : 16 * NC);
     const int KB = K >> 7, NB = (N + 127) >> 7;
-    const int per = (KB + kSmWaves - 1) / kSmWaves;
-    const int k_begin = min(wave * per, KB), k_end = min(k_begin + per, KB);      // this wave's K blocks
+    const int per = (KB + WK - 1) / WK;
+    const int k_begin = min(wk * per, KB), k_end = min(k_begin + per, KB);      // this wave's K blocks
     // global: lane l loads piece l & 7 of row 8 t + (l >> 3) for t = 0, 1 of every 16-row tile
     const uint8_t* bld[BT];
     const uint8_t* ald[2 * MT];
@@ -276,16 +280,16 @@ __device__ __forceinline__ void smallm_lines_body(const uint8_t* __restrict__ a,
 #pragma unroll
             for (int e = 0; e < 4; ++e) red[wave][j * MT + i][lane][e] = acc[j][i][e];
     __syncthreads();
-    if (wave < SUB) {
-        // wave (j, i) reduces column group j, row sub-tile i (fixed order, so results do not depend on timing)
-        const int j = wave / MT, i = wave % MT;
+    if (wk < SUB) {
+        // wave (j, i) of a set reduces column group j, row sub-tile i (fixed order, so results do not depend on timing)
+        const int j = wk / MT, i = wk % MT;
         const bool vec_ok = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
         float v[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             float t = 0.0f;
 #pragma unroll
-            for (int w = 0; w < kSmWaves; ++w) t += red[w][wave][lane][e];
+            for (int w = 0; w < WK; ++w) t += red[set * WK + w][wk][lane][e];
             v[e] = t;
         }
         const int m = i * 16 + frow, n = n0 + 16 * j + 4 * fk;
@@ -304,6 +308,16 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_lines_kernel(co
                                                                                const float* __restrict__ b_s, OUT* __restrict__ c,
                                                                                const uint16_t* __restrict__ bias, int M, int N, int K) {
     smallm_lines_body<MT, NC, UF, OUT, FMT>(a, a_s, as_rs, as_cs, b, b_s, c, bias, M, N, K);
+}
+
+// up to 16 rows against a short K (1..4 K blocks): WK waves per set of 16 * NC columns, 8 / WK sets per workgroup
+template <int NC, int UF, int WK, typename OUT, int FMT>
+__global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_lines_shortk_kernel(const uint8_t* __restrict__ a,
+                                                                                      const float* __restrict__ a_s, int64_t as_rs,
+                                                                                      int64_t as_cs, const uint8_t* __restrict__ b,
+                                                                                      const float* __restrict__ b_s, OUT* __restrict__ c,
+                                                                                      const uint16_t* __restrict__ bias, int M, int N, int K) {
+    smallm_lines_body<1, NC, UF, OUT, FMT, false, WK>(a, a_s, as_rs, as_cs, b, b_s, c, bias, M, N, K);
 }
 
 // up to 16 rows against a narrow weight: 8 columns per workgroup
@@ -855,6 +869,25 @@ static int dispatch_small(const uint8_t* a, const float* a_s, int64_t as_rs, int
         case 8: MDY_LINES(MT, NC, 8); break;          \
         default: MDY_LINES_UF4(MT, NC)                \
     }
+        // a short K (1..4 K blocks) against a large weight: fewer waves along K, 2, 4 or 8 sets of columns per workgroup
+        // instead of idle waves (per call in a replayed graph: M=16 N=32768 K=512 7.0 -> 5.0 us, M=4 N=129280 K=512 27.3 -> 18.7;
+        // small weights lose 0.2 us: N=7168 K=512 2.9 -> 3.1; 12 K blocks as 4 waves x 3: no gain)
+        const int KBs = K / 128;
+        if (M <= 16 && KBs <= 4 && (int64_t)N * K >= (8 << 20)) {
+            const int wk = KBs == 1 ? 1 : KBs == 2 ? 2 : 4;
+            const int nc = (wide && wk >= 2) ? 2 : 1, sets = 8 / wk;
+            grid = dim3((unsigned)((N + 16 * nc * sets - 1) / (16 * nc * sets)));
+#define MDY_SK(NC, WK)                                                                                                              \
+    hipLaunchKernelGGL((fp8_gemm_smallm_lines_shortk_kernel<NC, 1, WK, OUT, FMT>), grid, dim3(kSmWaves * 64), 0, stream, a, a_s, as_rs, \
+                       as_cs, b, b_s, c, bias, M, N, K)
+            if (wk == 1) MDY_SK(1, 1);
+            else if (wk == 2 && nc == 2) MDY_SK(2, 2);
+            else if (wk == 2) MDY_SK(1, 2);
+            else if (nc == 2) MDY_SK(2, 4);
+            else MDY_SK(1, 4);
+#undef MDY_SK
+            return (int)hipGetLastError();
+        }
         // a narrow weight (fewer than 100 groups of 16 columns): 8 columns per workgroup, twice the workgroups (per call in
         // a replayed graph: M=16 N=1584 K=4096 4.6 -> 3.8 us, M=16 N=1024 K=8192 7.2 -> 6.3, M=4 N=1536 K=7168 5.3 -> 4.8,
         // M=16 N=576 K=7168 6.0 -> 5.8; N=2048 and wider: no gain)
