@@ -161,7 +161,7 @@ constexpr int kSmWaves = 8;      // waves per workgroup of the small-M kernels
 // row l >> 3).  So here a wave loads its K blocks that way, UF blocks before the first use, and turns a block into
 // fragments through LDS that only this wave touches - two 16-byte writes and two 16-byte reads per 16 rows, pieces
 // XOR-swizzled by the row so that both fall on all banks - which needs no barrier: every wave runs on as its own
-// loads arrive, block u+1 on its way through LDS while the MFMAs of block u run.  Wave w owns the K blocks
+// loads arrive (and, with two LDS tiles per wave, block u+1 on its way through LDS while the MFMAs of block u run).  Wave w owns the K blocks
 // [w per, (w+1) per), per = ceil(KB / 8): no branch depends on the block, so the waits the compiler places count
 // exactly; a block beyond the wave's range is a re-read of the last valid one whose product is replaced by zero.
 // ---------------------------------------------------------------------------
@@ -175,7 +175,11 @@ __device__ __forceinline__ void smallm_lines_body(const uint8_t* __restrict__ a,
     constexpr int SETS = kSmWaves / WK;
     static_assert(SUB <= WK && SETS * WK == kSmWaves, "one wave of a set reduces one (column group, row sub-tile) pair");
     constexpr int SV = (UF + 3) / 4;                    // activation-scale loads per row sub-tile and pass
-    constexpr int NBUF = MT < 4 ? 2 : 1;               // LDS regions and fragment sets per wave (64 rows: no room for two)
+    // LDS regions and fragment sets per wave: two (block u + 1 on its way through LDS while the MFMAs of block u run) where
+    // one workgroup per CU is all there is (16 rows x 16 columns against a long K: M=16 N=2048 K=7168 5.4 us against 7.2 with
+    // one); one elsewhere, so that two or three workgroups fit a CU's LDS (M=16 N=24576 K=1536 10.0 -> 8.3 us, N=129280
+    // K=7168 165 -> 154 us; 17..32 rows: 10.0 -> 9.6 us at N=2048 K=7168)
+    constexpr int NBUF = (MT == 1 && NC == 1) ? 2 : 1;
     __shared__ __attribute__((aligned(16))) uint8_t lds[kSmWaves][NBUF][TILES * 2048];
     __shared__ float red[kSmWaves][SUB][64][4];
     const int tid = threadIdx.x, lane = tid & 63;
