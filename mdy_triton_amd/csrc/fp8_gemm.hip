@@ -314,6 +314,14 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_lines_kernel(co
     smallm_lines_body<MT, NC, UF, OUT, FMT>(a, a_s, as_rs, as_cs, b, b_s, c, bias, M, N, K);
 }
 
+// up to 16 rows, 32 columns per workgroup, registers held to 128 per lane so that two workgroups share a CU
+template <int UF, typename OUT, int FMT>
+__global__ __launch_bounds__(kSmWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void fp8_gemm_smallm_lines_occ2_kernel(
+    const uint8_t* __restrict__ a, const float* __restrict__ a_s, int64_t as_rs, int64_t as_cs, const uint8_t* __restrict__ b,
+    const float* __restrict__ b_s, OUT* __restrict__ c, const uint16_t* __restrict__ bias, int M, int N, int K) {
+    smallm_lines_body<1, 2, UF, OUT, FMT>(a, a_s, as_rs, as_cs, b, b_s, c, bias, M, N, K);
+}
+
 // up to 16 rows against a short K (1..4 K blocks): WK waves per set of 16 * NC columns, 8 / WK sets per workgroup
 template <int NC, int UF, int WK, typename OUT, int FMT>
 __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_lines_shortk_kernel(const uint8_t* __restrict__ a,
@@ -911,6 +919,15 @@ static int dispatch_small(const uint8_t* a, const float* a_s, int64_t as_rs, int
                 default: MDY_HALF(8); break;
             }
 #undef MDY_HALF
+        } else if (M <= 16 && wide && (uf == 4 || uf == 5)) {
+            // passes of 4 or 5 K blocks need 129..138 registers: held to 128, two workgroups share a CU (M=16 N=24576 K=4096
+            // 21.7 -> 19.5 us, M=8 N=32768 K=5120 28.5 -> 26.1; deeper passes would spill: N=16384 K=7168 21.8 -> 30.4 us)
+            if (uf == 4)
+                hipLaunchKernelGGL((fp8_gemm_smallm_lines_occ2_kernel<4, OUT, FMT>), grid, dim3(kSmWaves * 64), 0, stream, a, a_s, as_rs,
+                                   as_cs, b, b_s, c, bias, M, N, K);
+            else
+                hipLaunchKernelGGL((fp8_gemm_smallm_lines_occ2_kernel<5, OUT, FMT>), grid, dim3(kSmWaves * 64), 0, stream, a, a_s, as_rs,
+                                   as_cs, b, b_s, c, bias, M, N, K);
         } else if (M <= 16 && wide) {
             MDY_LINES_UF8(1, 2)
         } else if (M <= 16) {

@@ -343,7 +343,8 @@ def test_gemm_whole_line_kernel_long_k_exact_integer():
                                    (32, 1000, 4096), (25, 300, 16384), (32, 290, 9344),
                                    (64, 7168, 2048), (33, 3201, 1024), (48, 6402, 4096), (64, 3300, 2176), (50, 4099, 128),
                                    (16, 32768, 512), (9, 16500, 512), (16, 24576, 1536), (3, 22000, 384),                    # short K against a large
-                                   (16, 33000, 256), (2, 32768, 256), (13, 65540, 128), (1, 70000, 128)])                     # weight: 2, 4 or 8 column sets
+                                   (16, 33000, 256), (2, 32768, 256), (13, 65540, 128), (1, 70000, 128),                      # weight: 2, 4 or 8 column sets
+                                   (16, 6500, 4096), (4, 6404, 4224)])                                                        # passes of 4 / 5 blocks, registers held to 128
 def test_gemm_whole_line_kernel_exact_integer(M, N, K, fmt):
     """5..32 rows, and up to 64 against a middling N, run on the whole-line kernel (one, two or four 16-row activation
     tiles, 16 or 32 weight columns per workgroup by N, 1..8 K blocks per wave and pass by K, several passes for long K,
