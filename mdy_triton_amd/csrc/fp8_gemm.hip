@@ -853,9 +853,11 @@ static int dispatch_small(const uint8_t* a, const float* a_s, int64_t as_rs, int
         return launch_mfma<64, 64, 2, 2, 8, OUT, FMT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
     {      // everything else, and what lines_pays prefers: the whole-line kernel
         // 32 columns per workgroup when that still leaves ~200 workgroups (loads alone, M=16: N=7168, K=2048 2.9 -> 2.5 us
-        // per call; N=2048, K=7168 3.4 -> 4.1 us); the K blocks of a wave in passes of up to 8 (up to 16 rows) or 4
+        // per call; N=2048, K=7168 3.4 -> 4.1 us); the K blocks of a wave in passes of up to 8 (up to 16 rows, and up to 32 with 16
+        // columns per workgroup: M=20 N=2048 K=5120 9.5 -> 6.3 us, M=24 N=4096 K=7168 10.0 -> 8.3 us against passes of 4), 4
+        // (33..64 rows, 16 columns: M=64 N=5120 K=4096 17.3 -> 15.2 us against passes of 2) or 2
         const bool wide = (N + 31) / 32 >= 200;
-        const int per = (K / 128 + kSmWaves - 1) / kSmWaves, cap = M <= 16 ? 8 : M <= 32 ? 4 : 2;
+        const int per = (K / 128 + kSmWaves - 1) / kSmWaves, cap = M <= 16 ? 8 : M <= 32 ? (wide ? 4 : 8) : (wide ? 2 : 4);
         int uf = per;
         if (per > cap) {
             uf = cap;
@@ -935,13 +937,12 @@ static int dispatch_small(const uint8_t* a, const float* a_s, int64_t as_rs, int
         } else if (M <= 32 && wide) {
             MDY_LINES_UF4(2, 2)
         } else if (M <= 32) {
-            MDY_LINES_UF4(2, 1)
+            MDY_LINES_UF8(2, 1)
         } else if (wide) {
             if (uf == 1) MDY_LINES(4, 2, 1);
             else MDY_LINES(4, 2, 2);
         } else {
-            if (uf == 1) MDY_LINES(4, 1, 1);
-            else MDY_LINES(4, 1, 2);
+            MDY_LINES_UF4(4, 1)
         }
 #undef MDY_LINES_UF8
 #undef MDY_LINES_UF4
