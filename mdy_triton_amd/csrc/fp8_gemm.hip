@@ -503,14 +503,16 @@ __global__ __launch_bounds__(512) void fp8_gemv_kernel(const uint8_t* __restrict
 // their scales are copied into LDS ONCE per workgroup and shared by the 8 waves - in the small-M kernels every
 // 16 or 32 columns re-read them.  grid = (ceil(N/128), groups).
 // ---------------------------------------------------------------------------
-constexpr int kStripKC = 4;   // K blocks per step
+constexpr int kStripKC = 4;   // K blocks per step; the 64-row variant takes 2 (59 KB of LDS instead of 92, two workgroups per CU)
 
-template <int MT, typename OUT, int FMT = 0>
+template <int MT, typename OUT, int FMT = 0, int KC_ = kStripKC>
 __global__ __launch_bounds__(512) void fp8_gemm_strip_kernel(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, int as_rs, int as_cs, uint32_t as_bytes,
     const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
     const uint16_t* __restrict__ bias, int N, int K, const GroupTable tbl) {
-    constexpr int ROWS = MT * 16, KC = kStripKC;
+    constexpr int ROWS = MT * 16, KC = KC_;
+    constexpr int CPW = KC * MT / 4;      // activation copy instructions (8 rows x one K block) per wave and step
+    static_assert(CPW * 4 == KC * MT, "the step's copies divide evenly among the 8 waves");
     __shared__ __attribute__((aligned(1024))) uint8_t lds_a[2][KC][ROWS * 128];
     __shared__ __attribute__((aligned(256))) float lds_sa[2][KC][64];
     __shared__ __attribute__((aligned(256))) float lds_bs[512];
@@ -535,8 +537,8 @@ __global__ __launch_bounds__(512) void fp8_gemm_strip_kernel(
     intx4 rs = make_rsrc(a_s, as_bytes);
     if (wave >= KC) rs[2] = 0;
     const int prow = lane >> 3;
-    // a wave's instructions all land on row groups of the same parity (j / KC = wave / 4 + 2t): one swizzle per wave
-    const int voff = prow * K + (((lane & 7) ^ swz(((wave >> 2) & 1) * 8 + prow)) << 4);
+    // a wave's instructions all land on row groups of the same parity (j / KC = wave / KC + (8 / KC) t): one swizzle per wave
+    const int voff = prow * K + (((lane & 7) ^ swz(((wave / KC) & 1) * 8 + prow)) << 4);
     const int s_voff = min(r0 + min(lane, rows - 1), m_total - 1) * as_rs * 4;
     const uint32_t la0 = lds_addr(&lds_a[0][0][0]);
     const uint32_t ls0 = wave < KC ? lds_addr(&lds_sa[0][wave][0]) : lds_addr(&lds_dummy[0]) + wave * 1024;
@@ -544,7 +546,7 @@ __global__ __launch_bounds__(512) void fp8_gemm_strip_kernel(
     auto copy_step = [&](int step, int buf) {
         // instruction j of the step: K block j % KC, row group j / KC (8 rows); wave w takes j = w, w + 8, ...
 #pragma unroll
-        for (int t = 0; t < MT; ++t) {
+        for (int t = 0; t < CPW; ++t) {
             const int j = wave + 8 * t, kc = j % KC, rg = j / KC;
             dma16(ra, voff, rg * 8 * K + (step * KC + kc) * 128, la0 + (buf * KC + kc) * (ROWS * 128) + rg * 1024);
         }
@@ -802,7 +804,10 @@ static int launch_strip(const uint8_t* a, const float* a_s, int64_t as_rs, int64
     if (max_rows <= 16) MDY_STRIP(1);
     else if (max_rows <= 32) MDY_STRIP(2);
     else if (max_rows <= 48) MDY_STRIP(3);
-    else MDY_STRIP(4);
+    else      // 49..64 rows: 2 K blocks per step, so that two workgroups fit a CU's LDS (32 groups x 64 rows, N=4096, K=7168
+              // 201 -> 174..193 us; 64 x 56 rows, N=4096, K=2048 127 -> 109 us; M=64, N=36864 79 -> 71 us)
+        hipLaunchKernelGGL((fp8_gemm_strip_kernel<4, OUT, FMT, 2>), grid, block, 0, stream, a, a_s, (int)as_rs, (int)as_cs, as_bytes, b, b_s,
+                           c, bias, N, K, tbl);
 #undef MDY_STRIP
     return (int)hipGetLastError();
 }
