@@ -72,9 +72,13 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
     if (i >= MN) return;
     if (VEC) {   // N % 4 == 0: the 4 elements lie in one row
         float4 s = *reinterpret_cast<const float4*>(ws + i);
-        for (int k = 1; k < ksplit; ++k) {
-            const float4 v = *reinterpret_cast<const float4*>(ws + (int64_t)k * MN + i);
-            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+        for (int k0 = 1; k0 < ksplit; k0 += 4) {      // four slabs' loads in flight; added in slab order
+            float4 v[4];
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) v[kk] = *reinterpret_cast<const float4*>(ws + (int64_t)min(k0 + kk, ksplit - 1) * MN + i);
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk)
+                if (k0 + kk < ksplit) { s.x += v[kk].x; s.y += v[kk].y; s.z += v[kk].z; s.w += v[kk].w; }
         }
         if (bias != nullptr) {
             const int n = (int)(i % N);
@@ -168,7 +172,8 @@ constexpr int kSmWaves = 8;      // waves per workgroup of the small-M kernels
 template <int MT, int NC, int UF, typename OUT, int FMT, bool HALF = false, int WK = kSmWaves>
 __device__ __forceinline__ void smallm_lines_body(const uint8_t* __restrict__ a, const float* __restrict__ a_s, int64_t as_rs, int64_t as_cs,
                                                   const uint8_t* __restrict__ b, const float* __restrict__ b_s, OUT* __restrict__ c,
-                                                  const uint16_t* __restrict__ bias, int M, int N, int K) {
+                                                  const uint16_t* __restrict__ bias, int M, int N, int K, int kb_lo = 0,
+                                                  int kb_hi = -1) {
     constexpr int SUB = NC * MT, TILES = NC + MT;      // (column group, row sub-tile) pairs; 16-row operand tiles per K block
     // WK waves share out the K blocks of one set of columns; with a short K (fewer blocks than waves) the 8 waves form
     // 8 / WK such sets side by side instead of idling
@@ -193,8 +198,9 @@ __device__ __forceinline__ void smallm_lines_body(const uint8_t* __restrict__ a,
     const int set = wave / WK, wk = wave % WK;
     const int n0 = (blockIdx.x * SETS + set) * (HALF ? 8 : 16 * NC);
     const int KB = K >> 7, NB = (N + 127) >> 7;
-    const int per = (KB + WK - 1) / WK;
-    const int k_begin = min(wk * per, KB), k_end = min(k_begin + per, KB);      // this wave's K blocks
+    const int k_hi = kb_hi < 0 ? KB : kb_hi;                                     // the workgroup's K blocks: [kb_lo, k_hi)
+    const int per = (k_hi - kb_lo + WK - 1) / WK;
+    const int k_begin = min(kb_lo + wk * per, k_hi), k_end = min(k_begin + per, k_hi);      // this wave's K blocks
     // global: lane l loads piece l & 7 of row 8 t + (l >> 3) for t = 0, 1 of every 16-row tile
     const uint8_t* bld[BT];
     const uint8_t* ald[2 * MT];
@@ -312,6 +318,19 @@ __global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_lines_kernel(co
                                                                                const float* __restrict__ b_s, OUT* __restrict__ c,
                                                                                const uint16_t* __restrict__ bias, int M, int N, int K) {
     smallm_lines_body<MT, NC, UF, OUT, FMT>(a, a_s, as_rs, as_cs, b, b_s, c, bias, M, N, K);
+}
+
+// 33..64 rows against a narrow weight and a long K: K is cut into slabs as well (grid row = slab), workgroup (32 columns, slab)
+// writes the fp32 partial sums of its K blocks into slab blockIdx.y of a workspace [slabs][M][N], and splitk_reduce_kernel adds
+// the slabs in slab order.
+template <int UF>
+__global__ __launch_bounds__(kSmWaves * 64) void fp8_gemm_smallm_lines_slab_kernel(const uint8_t* __restrict__ a, const float* __restrict__ a_s,
+                                                                                    int64_t as_rs, int64_t as_cs, const uint8_t* __restrict__ b,
+                                                                                    const float* __restrict__ b_s, float* __restrict__ ws, int M,
+                                                                                    int N, int K, int kb_per) {
+    const int kb_lo = blockIdx.y * kb_per;
+    smallm_lines_body<4, 2, UF, float, 0>(a, a_s, as_rs, as_cs, b, b_s, ws + (size_t)blockIdx.y * M * N, nullptr, M, N, K, kb_lo,
+                                          min(K >> 7, kb_lo + kb_per));
 }
 
 // up to 16 rows, 32 columns per workgroup, registers held to 128 per lane so that two workgroups share a CU
@@ -1024,7 +1043,7 @@ static int dispatch(const uint8_t* a, const float* a_s, int64_t as_rs, int64_t a
 
 // ---- split-K plan: which tile, how many K slices; ksplit == 1 means "do not split"
 struct SplitPlan {
-    int config;     // 1: 128x128 tiles (ring of 4)   2: 128x64 (ring of 6)   3: 64x64 (ring of 8)
+    int config;     // 1: 128x128 tiles (ring of 4)   2: 128x64 (ring of 6)   3: 64x64 (ring of 8)   4: whole-line kernel, 32 columns
     int ksplit;     // slabs of the workspace
     int kb_per;     // K blocks per slab
 };
@@ -1040,6 +1059,24 @@ static SplitPlan plan_split(int64_t M, int64_t N, int64_t K) {
     if (M <= 64 && strip_pays(M, (N + 127) / 128)) return p;
     // up to 32 K blocks the whole-line kernel is as fast without the second pass (M=64 N=6400 K=4096: 10.6 against 12.9 us)
     if (lines_pays(M, N) && KB <= 32) return p;
+    // 33..64 rows against a weight so narrow that its groups of 32 columns leave three quarters of the CUs idle: the
+    // whole-line kernel over slabs of K (per call in a replayed graph: M=64 N=2048 K=7168 11.3 -> 9.5 us, M=40 11.4 -> 8.9 us,
+    // M=64 N=1536 K=7168 11.0 -> 9.2 us against 64x64 tiles; N=4096: 12.9 against 12.8 us, so wider weights keep the tiles)
+    if (M <= 64) {
+        const long strips = (N + 31) / 32;
+        long ks = cus / strips;
+        if (ks > KB / 8) ks = KB / 8;
+        if (ks > 8) ks = 8;
+        if (strips * 4 <= cus && ks >= 2) {
+            p.config = 4;
+            p.kb_per = (int)((KB + ks - 1) / ks);
+            p.ksplit = (KB + p.kb_per - 1) / p.kb_per;
+            return p;
+        }
+        // up to 32 K blocks the whole-line kernel in one launch is ahead of tiles over slabs of K (M=64 N=3072 K=4096: 8.7
+        // against 10.5 us)
+        if (KB <= 32) return p;
+    }
     // the largest tile that, cut into slabs of at least 8 K blocks, still yields a workgroup for most CUs
     const long rows128 = (M + 127) / 128, rows64 = (M + 63) / 64;
     const long cols128 = (N + 127) / 128, cols64 = (N + 63) / 64;
@@ -1113,7 +1150,15 @@ static int launch_splitk(const uint8_t* a, const float* a_s, int64_t as_rs, int6
                            dim3(256), 0, stream, a, a_s, (int)as_rs, (int)as_cs, (uint32_t)as_extent, b, b_s, ws, M, N, K, \
                            tiles_m, tiles_n, p.ksplit, p.kb_per);                                                     \
     }
-    if (p.config == 1) MDY_SPLIT(128, 128, 4)
+    if (p.config == 4) {
+        dim3 grid((unsigned)((N + 31) / 32), (unsigned)p.ksplit);
+        if (p.kb_per <= kSmWaves)
+            hipLaunchKernelGGL((fp8_gemm_smallm_lines_slab_kernel<1>), grid, dim3(kSmWaves * 64), 0, stream, a, a_s, as_rs, as_cs, b, b_s, ws,
+                               M, N, K, p.kb_per);
+        else
+            hipLaunchKernelGGL((fp8_gemm_smallm_lines_slab_kernel<2>), grid, dim3(kSmWaves * 64), 0, stream, a, a_s, as_rs, as_cs, b, b_s, ws,
+                               M, N, K, p.kb_per);
+    } else if (p.config == 1) MDY_SPLIT(128, 128, 4)
     else if (p.config == 2) MDY_SPLIT(128, 64, 6)
     else MDY_SPLIT(64, 64, 8)
 #undef MDY_SPLIT

@@ -135,14 +135,19 @@ def test_gemm_exact_integer_random_mid_shapes(M, N, K):
     test_gemm_exact_integer_cases_all_kernels(M, N, K)
 
 
-SPLIT_SHAPES = [(128, 1536, 4096), (100, 777, 4224), (64, 2048, 4352), (40, 300, 8192), (256, 4096, 4096),
-                (130, 1100, 5120), (33, 130, 4096)]
+SPLIT_SHAPES = [(128, 1536, 4096), (100, 777, 4224), (256, 4096, 4096), (130, 1100, 5120),
+                (64, 2304, 4352), (48, 4096, 7168),                                 # 33..64 rows on 64x64 tiles
+                # 33..64 rows against at most 2048 columns: the whole-line kernel over slabs of K (one or two K blocks per
+                # wave and pass, several passes, ragged N with the scalar reduction, a slab count that does not divide K)
+                (64, 2048, 4352), (40, 300, 8192), (33, 130, 4096), (50, 1536, 7168), (37, 2042, 8192), (64, 1024, 16384),
+                (48, 256, 32768)]
 
 
 @pytest.mark.parametrize("M,N,K", SPLIT_SHAPES)
 def test_gemm_exact_integer_split_k(M, N, K):
     """Few rows against a long K: fp8_gemm hands the library a workspace and the shape runs split along K
-    (64x64, 128x64 and 128x128 tiles; N % 4 != 0 takes the scalar reduction).  Exact operands stay exact."""
+    (64x64, 128x64 and 128x128 tiles, or the whole-line kernel for up to 64 rows against a narrow weight; N % 4 != 0 takes
+    the scalar reduction).  Exact operands stay exact."""
     assert _lib.load().mdy_fp8_gemm_workspace_bytes(M, N, K) >= 2 * M * N * 4
     test_gemm_exact_integer_cases_all_kernels(M, N, K)
 
@@ -166,7 +171,7 @@ def _raw_gemm(a, a_s, b, b_s, bias, dtype, ws, ws_bytes=None):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("M,N,K", [(128, 1536, 7168), (100, 777, 4224), (64, 2048, 7168)])
+@pytest.mark.parametrize("M,N,K", [(128, 1536, 7168), (100, 777, 4224), (64, 2048, 7168), (64, 2304, 7168), (45, 1000, 5120)])
 def test_gemm_split_k_against_oracle_and_plain_path(M, N, K, dtype):
     """Through the C ABI: with a workspace the result is within the GEMM tolerance of the oracle and of the
     single-pass kernel (another summation order), deterministic, and the bias is added once; without one, or
