@@ -267,7 +267,7 @@ int mdy_fp8_gemm_nt_ws(const void* a, const float* a_s, int64_t as_row_stride, i
 #define MDY_PATH_SMALL_M 1
 #define MDY_PATH_STRIP 2
 #define MDY_PATH_TILES 3
-#define MDY_PATH_TILES_SPLIT_K 4
+#define MDY_PATH_TILES_SPLIT_K 4 /* K cut into slabs of the workspace: MFMA tiles, or the small-M kernel for up to 64 rows */
 int mdy_fp8_gemm_path(const void* a, const void* b, int64_t as_row_stride, int64_t as_col_stride, int64_t M,
                       int64_t N, int64_t K, int with_workspace);
 

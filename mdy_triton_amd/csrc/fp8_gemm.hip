@@ -31,9 +31,10 @@
 // workspace also splits K (fp8_gemm_splitk_kernel + splitk_reduce_kernel).  The 128x192 tile (mid-size
 // shapes whose 128x256 tiles would leave a quarter of the CUs idle) runs a second body with producer and
 // consumer waves (fp8_gemm_tile_ws in fp8_gemm_tile.h).
-// Small-M kernel (M <= 64): weight streaming, one workgroup of 8 waves per 16 columns,
-// waves split K (next block prefetched) and reduce through LDS.  Strip kernel: 5..64 rows against
-// many 128-column strips.  Scalar kernel: any other shape/alignment.
+// Small-M kernel (M <= 64): weight streaming in whole 128-byte lines, one workgroup of 8 waves per 8, 16 or 32
+// columns, the waves split K and reduce through LDS (with a workspace also over slabs of K for 33..64 rows against
+// a narrow weight).  Strip kernel: 17..64 rows against many 128-column strips.  Scalar kernel: any other
+// shape/alignment.
 #include <cstdlib>
 #include <mutex>
 
