@@ -42,10 +42,12 @@ def _bits(t):
     return t.cpu().view(torch.int16 if t.dtype == torch.bfloat16 else torch.int32).numpy()
 
 
-# (first call, second smaller call): split along K with 128x128 / 64x64 tiles, then a shape that needs no scratch
+# (first call, second smaller call): split along K with 128x128 / 128x64 tiles and, for (40, 300, 8192), the whole-line kernel over
+# slabs of K; then a shape that needs no scratch
 CASES = [((256, 4096, 4096), (128, 1536, 4096)),
          ((130, 1100, 5120), (40, 300, 8192)),
-         ((128, 2112, 7168), (16, 2048, 7168))]
+         ((128, 2112, 7168), (16, 2048, 7168)),
+         ((64, 2048, 7168), (33, 130, 4096))]
 
 
 @pytest.mark.parametrize("first,second", CASES)
