@@ -136,6 +136,7 @@ def test_gemm_exact_integer_random_mid_shapes(M, N, K):
 
 
 SPLIT_SHAPES = [(128, 1536, 4096), (100, 777, 4224), (256, 4096, 4096), (130, 1100, 5120),
+                (130, 520, 6528), (300, 1536, 4480), (1000, 640, 8192),             # slabs of 9 / 12 and 11 / 11 K blocks, 3 and 8 tile rows
                 (64, 2304, 4352), (48, 4096, 7168),                                 # 33..64 rows on 64x64 tiles
                 # 33..64 rows against at most 2048 columns: the whole-line kernel over slabs of K (one or two K blocks per
                 # wave and pass, several passes, ragged N with the scalar reduction, a slab count that does not divide K)
@@ -146,7 +147,7 @@ SPLIT_SHAPES = [(128, 1536, 4096), (100, 777, 4224), (256, 4096, 4096), (130, 11
 @pytest.mark.parametrize("M,N,K", SPLIT_SHAPES)
 def test_gemm_exact_integer_split_k(M, N, K):
     """Few rows against a long K: fp8_gemm hands the library a workspace and the shape runs split along K
-    (64x64, 128x64 and 128x128 tiles, or the whole-line kernel for up to 64 rows against a narrow weight; N % 4 != 0 takes
+    (64x64 tiles, 128x64 and 128x128 tiles on the producer / consumer kernel, or the whole-line kernel for up to 64 rows against a narrow weight; N % 4 != 0 takes
     the scalar reduction).  Exact operands stay exact."""
     assert _lib.load().mdy_fp8_gemm_workspace_bytes(M, N, K) >= 2 * M * N * 4
     test_gemm_exact_integer_cases_all_kernels(M, N, K)
@@ -171,7 +172,8 @@ def _raw_gemm(a, a_s, b, b_s, bias, dtype, ws, ws_bytes=None):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("M,N,K", [(128, 1536, 7168), (100, 777, 4224), (64, 2048, 7168), (64, 2304, 7168), (45, 1000, 5120)])
+@pytest.mark.parametrize("M,N,K", [(128, 1536, 7168), (100, 777, 4224), (64, 2048, 7168), (64, 2304, 7168), (45, 1000, 5120),
+                                   (300, 1536, 4480)])
 def test_gemm_split_k_against_oracle_and_plain_path(M, N, K, dtype):
     """Through the C ABI: with a workspace the result is within the GEMM tolerance of the oracle and of the
     single-pass kernel (another summation order), deterministic, and the bias is added once; without one, or
