@@ -893,8 +893,14 @@ static int dispatch_small(const uint8_t* a, const float* a_s, int64_t as_rs, int
     }
     // 32..64 rows against a wide weight: the whole-line kernel re-reads the activation rows in every one of its N/16 or
     // N/32 workgroups, and from 32 rows on that traffic costs more than the empty rows of an MFMA tile (see lines_pays).
-    if (!lines && M >= 32 && M <= 64 && big_ok && (N + 127) / 128 >= 128)
-        return launch_mfma<128, 128, 2, 2, 4, OUT, FMT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
+    // (128..199 tiles of 128x128, one per CU, on the producer / consumer body: against the one-body tile, back to back, M=64
+    // N=18432 K=7168 36.1 -> 28.2 us, M=48 N=16384 K=2048 13.5 -> 10.7 us, M=64 N=24576 K=1536 12.6 -> 10.5 us; 2-3 % after a flush)
+    if (!lines && M >= 32 && M <= 64 && big_ok && (N + 127) / 128 >= 128) {
+        const int tiles_n = (N + 127) / 128;
+        hipLaunchKernelGGL((fp8_gemm_ws_kernel<128, 128, 2, 2, 4, 4, OUT, FMT>), dim3((unsigned)tiles_n), dim3(512), 0, stream, a, a_s,
+                           (int)as_rs, (int)as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, 1, tiles_n, pretouch_enabled() ? 1 : 0);
+        return (int)hipGetLastError();
+    }
     if (!lines && M >= 32 && M <= 64 && big_ok && (N + 63) / 64 >= 100)
         return launch_mfma<64, 64, 2, 2, 8, OUT, FMT>(a, a_s, as_rs, as_cs, (uint32_t)as_extent, b, b_s, c, bias, M, N, K, N, stream);
     {      // everything else, and what lines_pays prefers: the whole-line kernel
