@@ -86,7 +86,9 @@ def test_grouped_gemm_exact_integer(m_splits, N, K):
 @pytest.mark.parametrize("m_splits,N,K", [([1, 64, 0, 17, 33, 48, 16, 5], 3300, 896),    # ragged rows and columns, K tail step
                                           ([40] * 40, 640, 128),                          # one K block
                                           ([24] * 9, 3000, 2560),                         # 5 steps of 4 K blocks: odd number of steps
-                                          ([64] * 4, 6400, 1152)])
+                                          ([64] * 4, 6400, 1152),                         # 49..64 rows: steps of 2 K blocks, 9 K blocks
+                                          ([56] * 25, 1024, 128), ([50, 64] * 13, 1000, 256),     # the same with one K block / one step
+                                          ([49] * 30, 900, 640)])
 def test_grouped_gemm_exact_integer_strip_kernel(m_splits, N, K):
     """17..64 rows in the largest group and >= 200 strips of 128 columns: the weight-streaming strip kernel runs."""
     assert 16 < max(m_splits) <= 64 and len(m_splits) * ((N + 127) // 128) >= 200
